@@ -1,0 +1,283 @@
+"""Pins the CPU oracle (oracle/denox_oracle.c) against library routines, closed
+forms and brute force -- independent statements of the same mathematics, so a
+dropped term, a swapped index or a transposed weight fails here.
+
+torch.nn.functional on CPU in fp32 is the library routine; it is local torch,
+not reference code."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+
+def hwc_to_nchw(x):
+    return torch.from_numpy(np.ascontiguousarray(x)).permute(2, 0, 1).unsqueeze(0)
+
+
+def nchw_to_hwc(t):
+    return t.squeeze(0).permute(1, 2, 0).contiguous().numpy()
+
+
+# ----------------------------------------------------------------------------- f16
+def test_f16_to_f32_all_patterns(oracle):
+    bits = np.arange(65536, dtype=np.uint16)
+    got = oracle.f16_to_f32(bits)
+    want = bits.view(np.float16).astype(np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+
+
+def test_f32_to_f16_rne(oracle):
+    rng = np.random.default_rng(1)
+    # every f16 value, its neighbours' midpoints (ties) and random values across the range
+    h = np.arange(0, 0x7C00, dtype=np.uint16).view(np.float16).astype(np.float32)
+    mids = (h[:-1].astype(np.float64) + h[1:].astype(np.float64)) / 2
+    vals = np.concatenate([
+        h, -h, mids.astype(np.float32), -mids.astype(np.float32),
+        np.nextafter(mids.astype(np.float32), np.float32(np.inf)),
+        np.nextafter(mids.astype(np.float32), np.float32(-np.inf)),
+        rng.standard_normal(200000).astype(np.float32) * np.float32(10.0) ** rng.integers(-9, 6, 200000).astype(np.float32),
+        np.array([65504, 65519.99, 65520, 70000, 1e30, np.inf, -np.inf, 2.0 ** -24, 2.0 ** -25, 2.0 ** -25 * 1.0001,
+                  2.0 ** -26, 0.0, -0.0], np.float32),
+    ])
+    got = oracle.f32_to_f16_bits(vals)
+    with np.errstate(over="ignore"):
+        want = vals.astype(np.float16).view(np.uint16)
+    assert np.array_equal(got, want)
+    assert np.isnan(oracle.f32_to_f16_bits(np.array([np.nan], np.float32)).view(np.float16))[0]
+
+
+# ----------------------------------------------------------------------------- conv
+CONV_CASES = [
+    # H, W, C, K, R, S, stride, pad
+    (9, 11, 3, 16, 3, 3, 1, 1),
+    (8, 8, 9, 32, 3, 3, 1, 1),
+    (13, 7, 16, 3, 3, 3, 1, 1),
+    (6, 10, 48, 16, 3, 3, 1, 1),
+    (5, 5, 73, 64, 3, 3, 1, 1),
+    (12, 12, 8, 8, 1, 1, 1, 0),
+    (12, 13, 4, 6, 5, 5, 1, 2),
+    (12, 13, 4, 6, 3, 3, 2, 1),
+    (7, 9, 5, 4, 3, 1, 1, 0),
+]
+
+
+@pytest.mark.parametrize("H,W,C,K,R,S,stride,pad", CONV_CASES)
+@pytest.mark.parametrize("use_bias,act", [(False, "none"), (True, "relu"), (True, "leaky")])
+def test_conv_vs_torch_fp32(oracle, H, W, C, K, R, S, stride, pad, use_bias, act):
+    rng = np.random.default_rng(H * 131 + W * 17 + C + K)
+    x = rng.standard_normal((H, W, C)).astype(np.float16)
+    w = (rng.standard_normal((K, C, R, S)) * np.sqrt(2.0 / (R * S * C))).astype(np.float16)
+    b = (rng.standard_normal(K) * 0.1).astype(np.float16) if use_bias else None
+    a = {"none": oracle.ACT_NONE, "relu": oracle.ACT_RELU, "leaky": oracle.ACT_LEAKY_RELU}[act]
+    got = oracle.conv2d(x, w, b, (stride, stride), (pad, pad), a, 0.1)
+    t = F.conv2d(hwc_to_nchw(x.astype(np.float32)), torch.from_numpy(w.astype(np.float32)),
+                 None if b is None else torch.from_numpy(b.astype(np.float32)), stride=stride, padding=pad)
+    if act == "relu":
+        t = F.relu(t)
+    elif act == "leaky":
+        t = F.leaky_relu(t, 0.1)
+    want = nchw_to_hwc(t)
+    assert got.shape == want.shape
+    # both are fp32 sums of the same terms in different orders
+    np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-5)
+
+
+def test_conv_centre_tap_is_identity(oracle):
+    rng = np.random.default_rng(3)
+    C = 7
+    x = rng.standard_normal((10, 12, C)).astype(np.float16)
+    w = np.zeros((C, C, 3, 3), np.float16)
+    for c in range(C):
+        w[c, c, 1, 1] = 1
+    got = oracle.conv2d(x, w, None)
+    assert np.array_equal(got, x.astype(np.float32))
+
+
+def test_conv_single_off_centre_tap_shifts(oracle):
+    # W[k=0, c=0, r=0, s=2] = 1  =>  out[y, x] = in[y - 1, x + 1] with zeros outside:
+    # catches a transposed (r, s) or a flipped kernel.
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((6, 8, 1)).astype(np.float16)
+    w = np.zeros((1, 1, 3, 3), np.float16)
+    w[0, 0, 0, 2] = 1
+    got = oracle.conv2d(x, w, None)[:, :, 0]
+    want = np.zeros((6, 8), np.float32)
+    want[1:, :-1] = x[:-1, 1:, 0].astype(np.float32)
+    assert np.array_equal(got, want)
+
+
+def test_conv_all_ones_counts_in_bounds_taps(oracle):
+    # all-ones input and weights: out = C * (#taps inside the image): 9C interior, 6C edge, 4C corner
+    H, W, C, K = 6, 7, 5, 4
+    got = oracle.conv2d(np.ones((H, W, C), np.float16), np.ones((K, C, 3, 3), np.float16), None)
+    assert np.all(got[1:-1, 1:-1] == 9 * C)
+    assert np.all(got[0, 1:-1] == 6 * C) and np.all(got[-1, 1:-1] == 6 * C)
+    assert np.all(got[1:-1, 0] == 6 * C) and np.all(got[1:-1, -1] == 6 * C)
+    for yy, xx in [(0, 0), (0, -1), (-1, 0), (-1, -1)]:
+        assert np.all(got[yy, xx] == 4 * C)
+
+
+def test_conv_bruteforce_fp64(oracle):
+    rng = np.random.default_rng(5)
+    H, W, C, K = 5, 6, 3, 4
+    x = rng.standard_normal((H, W, C)).astype(np.float16)
+    w = rng.standard_normal((K, C, 3, 3)).astype(np.float16)
+    b = rng.standard_normal(K).astype(np.float16)
+    want = np.zeros((H, W, K))
+    for y in range(H):
+        for xx in range(W):
+            for k in range(K):
+                acc = float(b[k])
+                for r in range(3):
+                    for s in range(3):
+                        iy, ix = y + r - 1, xx + s - 1
+                        if 0 <= iy < H and 0 <= ix < W:
+                            for c in range(C):
+                                acc += float(x[iy, ix, c]) * float(w[k, c, r, s])
+                want[y, xx, k] = max(acc, 0.0)
+    got = oracle.conv2d(x, w, b, act=oracle.ACT_RELU)
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5)
+
+
+def test_conv_round_f16_is_rne_of_fp32(oracle):
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((7, 7, 8)).astype(np.float16)
+    w = rng.standard_normal((8, 8, 3, 3)).astype(np.float16)
+    a = oracle.conv2d(x, w, None)
+    b = oracle.conv2d(x, w, None, round_f16_out=True)
+    assert np.array_equal(b, a.astype(np.float16).astype(np.float32))
+
+
+# ----------------------------------------------------------------------------- movement ops
+@pytest.mark.parametrize("H,W,C", [(8, 8, 3), (9, 7, 16), (2, 2, 1), (11, 14, 24), (1, 5, 8)])
+def test_maxpool_vs_torch(oracle, H, W, C):
+    rng = np.random.default_rng(H * W + C)
+    x = rng.standard_normal((H, W, C)).astype(np.float16)
+    got = oracle.maxpool(x)
+    assert got.shape == (H // 2, W // 2, C)
+    if got.size:
+        want = nchw_to_hwc(F.max_pool2d(hwc_to_nchw(x.astype(np.float32)), 2)).astype(np.float16)
+        assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+        # membership: every output bit pattern is one of its window's four
+        win = x[:H // 2 * 2, :W // 2 * 2].reshape(H // 2, 2, W // 2, 2, C)
+        assert np.all((win.view(np.uint16) == got.view(np.uint16)[:, None, :, None, :]).any(axis=(1, 3)))
+
+
+@pytest.mark.parametrize("H,W,C,f", [(4, 5, 3, 2), (7, 3, 16, 2), (3, 3, 9, 3), (1, 1, 8, 2)])
+def test_upsample_vs_torch(oracle, H, W, C, f):
+    rng = np.random.default_rng(H + W + C)
+    x = rng.standard_normal((H, W, C)).astype(np.float16)
+    got = oracle.upsample_nearest(x, f)
+    want = nchw_to_hwc(F.interpolate(hwc_to_nchw(x.astype(np.float32)), scale_factor=f, mode="nearest")).astype(np.float16)
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+
+
+def test_concat_and_channel_copy_vs_torch(oracle):
+    rng = np.random.default_rng(7)
+    a = rng.standard_normal((5, 6, 32)).astype(np.float16)
+    b = rng.standard_normal((5, 6, 9)).astype(np.float16)
+    got = oracle.concat(a, b)
+    want = torch.cat([hwc_to_nchw(a), hwc_to_nchw(b)], 1)
+    assert np.array_equal(got.view(np.uint16), nchw_to_hwc(want).view(np.uint16))
+    dst = np.zeros((5, 6, 20), np.float16)
+    oracle.copy_channels(a, 3, dst, 7, 5)
+    assert np.array_equal(dst[:, :, 7:12], a[:, :, 3:8]) and not dst[:, :, :7].any() and not dst[:, :, 12:].any()
+    with pytest.raises(ValueError):
+        oracle.copy_channels(a, 30, dst, 0, 5)
+
+
+@pytest.mark.parametrize("l,r,t,b", [(0, 0, 0, 8), (0, 3, 0, 11), (2, 1, 3, 0), (0, 0, 0, 0), (5, 5, 5, 5)])
+def test_pad_replicate_vs_torch(oracle, l, r, t, b):
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((4, 5, 9)).astype(np.float16)
+    got = oracle.pad_replicate(x, l, r, t, b)
+    want = nchw_to_hwc(F.pad(hwc_to_nchw(x.astype(np.float32)), (l, r, t, b), mode="replicate")).astype(np.float16)
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+
+
+def test_slice_vs_indexing(oracle):
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((9, 10, 3)).astype(np.float16)
+    got = oracle.slice_hw(x, left=2, top=1, out_h=5, out_w=7)
+    want = nchw_to_hwc(hwc_to_nchw(x)[:, :, 1:6, 2:9])
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    with pytest.raises(ValueError):
+        oracle.slice_hw(x, left=5, top=0, out_h=9, out_w=6)
+
+
+def test_activation_vs_torch_fp16(oracle):
+    bits = np.arange(65536, dtype=np.uint16)
+    x = bits.view(np.float16)
+    finite = np.isfinite(x)
+    x = x[finite]
+    got = oracle.activation(x, oracle.ACT_RELU)
+    want = F.relu(torch.from_numpy(x.astype(np.float32))).numpy().astype(np.float16)
+    assert np.array_equal(got, want)
+    assert not np.signbit(got).any()  # max(v, 0) never yields -0
+    alpha = 0.1
+    got = oracle.activation(x, oracle.ACT_LEAKY_RELU, alpha)
+    ah = np.float16(alpha)
+    want = np.maximum(x, (ah * x).astype(np.float16))  # binary16 product, as a 16-bit ALU computes it
+    assert np.array_equal(got, want)
+
+
+# ----------------------------------------------------------------------------- layouts
+@pytest.mark.parametrize("H,W,C", [(3, 5, 8), (4, 4, 16), (2, 7, 24)])
+def test_layouts_vs_permute(oracle, H, W, C):
+    rng = np.random.default_rng(10)
+    hwc = rng.standard_normal((H, W, C)).astype(np.float16)
+    chw = oracle.relayout(hwc, oracle.LAYOUT_HWC, oracle.LAYOUT_CHW, H, W, C)
+    assert np.array_equal(chw.reshape(C, H, W), hwc.transpose(2, 0, 1))
+    c8 = oracle.relayout(hwc, oracle.LAYOUT_HWC, oracle.LAYOUT_CHWC8, H, W, C)
+    assert np.array_equal(c8.reshape(C // 8, H, W, 8), hwc.reshape(H, W, C // 8, 8).transpose(2, 0, 1, 3))
+    back = oracle.relayout(c8, oracle.LAYOUT_CHWC8, oracle.LAYOUT_HWC, H, W, C)
+    assert np.array_equal(back.reshape(H, W, C), hwc)
+    with pytest.raises(ValueError):
+        oracle.relayout(np.zeros(2 * 2 * 9, np.float16), oracle.LAYOUT_HWC, oracle.LAYOUT_CHWC8, 2, 2, 9)
+
+
+# ----------------------------------------------------------------------------- SymIR
+def test_symir_known_programs(oracle):
+    o = oracle
+    H, W = 1080, 1920
+    # cdiv(W, 16) = (W + 15) / 16 ; H/2 ; max(a + b, c) ; non-negative mod ; constant-lhs sub / div
+    ops = [
+        (o.SYM_ADD | o.SYM_RHSC, 1, 15),      # 2: W + 15
+        (o.SYM_DIV | o.SYM_RHSC, 2, 16),      # 3: (W+15)/16
+        (o.SYM_DIV | o.SYM_RHSC, 0, 2),       # 4: H/2
+        (o.SYM_ADD, 3, 4),                    # 5: 120 + 540
+        (o.SYM_MAX | o.SYM_RHSC, 5, 1000),    # 6: max(660, 1000)
+        (o.SYM_SUB | o.SYM_LHSC, 16, 0),      # 7: 16 - H
+        (o.SYM_MOD | o.SYM_RHSC, 7, 16),      # 8: (16 - 1080) mod 16, non-negative
+        (o.SYM_MUL | o.SYM_LHSC, 3, 0),       # 9: 3 * H
+        (o.SYM_DIV | o.SYM_LHSC, 100000, 1),  # 10: 100000 / W
+        (o.SYM_MIN, 0, 1),                    # 11
+        (o.SYM_DIV | o.SYM_RHSC, 7, 16),      # 12: truncating division of a negative
+        (o.SYM_MOD | o.SYM_LHSC, -7, 0),      # 13: -7 mod H
+    ]
+    dp = o.symir_eval([H, W], ops)
+    assert dp[:2] == [H, W]
+    assert dp[2:] == [1935, 120, 540, 660, 1000, -1064, 8, 3240, 52, 1080, -66, 1073]
+    with pytest.raises(ValueError):
+        o.symir_eval([H, W], [(o.SYM_DIV | o.SYM_RHSC, 0, 0)])
+    with pytest.raises(ValueError):
+        o.symir_eval([H, W], [(o.SYM_ADD, 0, 5)])  # forward reference
+
+
+def test_run_graph_modes_agree_on_data_movement(oracle):
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((6, 10, 8)).astype(np.float16)
+    ops = [
+        {"op": "pad", "src": "x", "dst": "p", "left": 0, "right": 2, "top": 0, "bottom": 2},
+        {"op": "pool", "src": "p", "dst": "q"},
+        {"op": "upsample", "src": "q", "dst": "u"},
+        {"op": "concat", "src": ["u", "p"], "dst": "c"},
+        {"op": "activation", "src": "c", "dst": "r", "func": "relu"},
+        {"op": "slice", "src": "r", "dst": "y", "left": 0, "top": 0, "out_h": 6, "out_w": 10},
+    ]
+    a = oracle.run_graph(ops, {"x": x}, "fp32")["y"]
+    b = oracle.run_graph(ops, {"x": x}, "f16")["y"]
+    assert a.shape == (6, 10, 16)
+    assert np.array_equal(a, b.astype(np.float32))
