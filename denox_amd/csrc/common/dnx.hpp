@@ -1,0 +1,103 @@
+// In-memory form and byte serialisation of a compiled model ("dnx").
+//
+// Mirrors the reference schema dnx.fbs:1-195 table by table -- Model{tensors,
+// initializers, inputs, outputs, buffers, dispatches, shader_binaries, sym_ir,
+// value_names}, ComputeDispatch{binary_id, workgroup_count_{x,y,z}, entry_point,
+// bindings, push_constant, info} -- with the two changes a HIP backend needs:
+//   * ShaderBinary carries a gfx950 code object (bytes) instead of SPIR-V words
+//     (dnx.fbs:169-171);
+//   * ComputeDispatch gains the workgroup size, which SPIR-V bakes into the
+//     module as local_size but a HIP launch takes as an argument.
+// FlatBuffers (flatc and its headers) are not available, so the bytes on the
+// wire are a plain little-endian tagged stream with a bounds-checked reader;
+// the field set, not the byte layout, is what matches the reference.
+#pragma once
+#include "error.hpp"
+#include "sym.hpp"
+#include <cstdint>
+#include <string>
+#include <vector>
+
+namespace denox::dnx {
+
+enum class ScalarType : uint8_t { I16 = 0, U16 = 1, I32 = 2, U32 = 3, I64 = 4, U64 = 5, F16 = 6, F32 = 7, F64 = 8 };
+enum class Access : uint8_t { ReadOnly = 0, WriteOnly = 1, ReadWrite = 2 };
+enum class TensorFormat : uint16_t { UNKNOWN = 0, SSBO_HWC = 1, SSBO_CHW = 2, SSBO_CHWC8 = 3, TEX_RGBA = 4, TEX_RGB = 5, TEX_RG = 6, TEX_R = 7 };
+enum class TensorStorage : uint16_t { StorageBuffer = 0, StorageImage = 1, SampledStorageImage = 2 };
+
+inline size_t scalarSize(ScalarType t) {
+  switch (t) {
+  case ScalarType::I16: case ScalarType::U16: case ScalarType::F16: return 2;
+  case ScalarType::I32: case ScalarType::U32: case ScalarType::F32: return 4;
+  default: return 8;
+  }
+}
+
+// union ScalarSource { literal, symbolic } (dnx.fbs:16-29).  Literals are kept
+// as int64 (all literals this backend emits are integers).
+struct ScalarSource {
+  bool symbolic = false;
+  ScalarType dtype = ScalarType::I64; // dtype of a literal
+  int64_t value = 0;                  // literal value or SymRef.sid
+  static ScalarSource fromSym(Sym s, ScalarType t = ScalarType::I64) { return ScalarSource{s.symbolic, t, s.v}; }
+  int64_t eval(const std::vector<int64_t> &dp) const {
+    if (!symbolic) return value;
+    if (value < 0 || static_cast<size_t>(value) >= dp.size()) fail(Status::InvalidModel, "SymRef out of range");
+    return dp[static_cast<size_t>(value)];
+  }
+};
+
+struct PushConstantField { ScalarType dtype; uint16_t offset; ScalarSource source; };
+struct PushConstant { uint16_t size = 0; std::vector<PushConstantField> fields; };
+struct DescriptorBinding { uint16_t binding; Access access; uint32_t tensor; };
+struct DescriptorSetBinding { uint16_t set; std::vector<DescriptorBinding> bindings; };
+struct DispatchInfo {
+  std::string name, debug_info, src_path;
+  bool has_reads = false, has_writes = false, has_flops = false;
+  ScalarSource memory_reads, memory_writes, flops;
+};
+struct ComputeDispatch {
+  uint32_t binary_id = 0;
+  ScalarSource workgroup_count_x, workgroup_count_y, workgroup_count_z;
+  uint32_t workgroup_size[3] = {1, 1, 1}; // HIP addition: threads per workgroup
+  std::string entry_point;
+  std::vector<DescriptorSetBinding> bindings;
+  PushConstant push_constant;
+  DispatchInfo info;
+};
+struct Buffer { ScalarSource size; uint16_t alignment = 16; };
+struct TensorInfo {
+  bool has_extent = false;
+  ScalarSource width, height, channels;
+  TensorFormat format = TensorFormat::UNKNOWN;
+  TensorStorage storage = TensorStorage::StorageBuffer;
+  ScalarType type = ScalarType::F16;
+  std::string name;
+};
+struct Tensor { uint32_t buffer = 0; ScalarSource offset, size; TensorInfo info; };
+struct TensorInitializer { uint32_t tensor; std::vector<uint8_t> data; };
+struct ValueName { std::string name; ScalarSource value; };
+struct ShaderBinary { std::vector<uint8_t> code_object; };
+struct ModelInfo { std::string producer, producer_version, model_version; };
+
+struct Model {
+  uint16_t version = 0;
+  ModelInfo info;
+  std::vector<Tensor> tensors;
+  std::vector<TensorInitializer> initializers;
+  std::vector<uint32_t> inputs, outputs;
+  std::vector<Buffer> buffers;
+  std::vector<ComputeDispatch> dispatches;
+  std::vector<ShaderBinary> shader_binaries;
+  SymIR sym_ir;
+  std::vector<ValueName> value_names;
+};
+
+std::vector<uint8_t> serialize(const Model &m);
+// Throws Error(InvalidModel) on a truncated, corrupt or inconsistent stream
+// (the role of the FlatBuffers verifier in runtime/src/denox/runtime/model.cpp:639-644).
+Model deserialize(const void *data, size_t size);
+// Index / reference consistency checks shared by the reader and the compiler.
+void validate(const Model &m);
+
+} // namespace denox::dnx

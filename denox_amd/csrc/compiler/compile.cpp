@@ -1,0 +1,365 @@
+#include "compile.hpp"
+#include <algorithm>
+#include <cstring>
+#include <map>
+#include <set>
+
+namespace denox::compiler {
+
+std::vector<int64_t> assumed_symeval(const Model &model, const SymGraph &sym, const CompileOptions &opt) {
+  std::vector<int64_t> vars;
+  for (const std::string &n : sym.varNames()) {
+    int64_t v = opt.defaultAssumedExtent;
+    auto it = opt.assumptions.find(n);
+    if (it != opt.assumptions.end()) v = it->second;
+    else
+      for (const auto &nv : model.valueNames()) // a variable may be known under several names
+        if (nv.value.symbolic && sym.varNames().size() > static_cast<size_t>(nv.value.v) && sym.varNames()[nv.value.v] == n) {
+          auto jt = opt.assumptions.find(nv.name);
+          if (jt != opt.assumptions.end()) v = jt->second;
+        }
+    vars.push_back(v);
+  }
+  return sym.eval(vars);
+}
+
+std::vector<uint8_t> push_constant_bytes(const ComputeDispatch &d, const std::vector<int64_t> &dp, std::vector<uint16_t> *offsets) {
+  // fields laid out in registration order at their natural alignment (serialize.cpp:379-398 of the reference)
+  std::vector<uint8_t> bytes;
+  if (offsets) offsets->clear();
+  for (const auto &pc : d.pushConstants) {
+    const size_t sz = dnx::scalarSize(pc.dtype);
+    while (bytes.size() % sz) bytes.push_back(0);
+    if (offsets) offsets->push_back(static_cast<uint16_t>(bytes.size()));
+    const int64_t v = symValue(dp, pc.value);
+    uint8_t tmp[8];
+    std::memcpy(tmp, &v, 8); // little endian: the low bytes are the narrower value
+    bytes.insert(bytes.end(), tmp, tmp + sz);
+  }
+  return bytes;
+}
+
+static double estimate_dispatch_ms(const ComputeDispatch &d, const std::vector<int64_t> &dp, const CompileOptions &opt) {
+  const double bytes = (d.info.hasReads ? static_cast<double>(symValue(dp, d.info.memoryReads)) : 0.0) +
+                       (d.info.hasWrites ? static_cast<double>(symValue(dp, d.info.memoryWrites)) : 0.0);
+  const double flops = d.info.hasFlops ? static_cast<double>(symValue(dp, d.info.flops)) : 0.0;
+  // conservative fractions of the published peaks plus a fixed launch cost
+  const double tMem = bytes / (0.5 * opt.deviceInfo.hbmBytesPerSecond);
+  const double tMath = flops / (0.3 * opt.deviceInfo.fp16MfmaFlops);
+  return (std::max(tMem, tMath) + 3e-6) * 1e3;
+}
+
+double edge_cost_ms(const SuperGraphEdge &e, const std::vector<int64_t> &dp, const Db *db, const CompileOptions &opt, bool *measured) {
+  double total = 0.0;
+  bool all = db != nullptr;
+  if (db) {
+    for (const auto &d : e.dispatches) {
+      const uint32_t wg[3] = {static_cast<uint32_t>(symValue(dp, d.workgroupCountX)), static_cast<uint32_t>(symValue(dp, d.workgroupCountY)),
+                              static_cast<uint32_t>(symValue(dp, d.workgroupCountZ))};
+      auto lat = db->query_dispatch_latency(d.kernel.sha256(), push_constant_bytes(d, dp), wg);
+      if (!lat) { all = false; break; }
+      total += *lat;
+    }
+  }
+  if (measured) *measured = all;
+  if (all) return total;
+  total = 0.0;
+  for (const auto &d : e.dispatches) total += estimate_dispatch_ms(d, dp, opt);
+  // estimates cannot tell configurations apart; the shader's prior breaks ties
+  return total / std::max(1e-3f, e.speedup);
+}
+
+namespace {
+struct Selector {
+  const Model &model;
+  const SuperGraph &g;
+  const std::vector<double> &cost;
+  std::vector<std::vector<size_t>> producers;
+  std::map<std::vector<int>, std::pair<double, long>> memo; // needed set -> (cost, edge chosen for its largest member)
+
+  double solve(const std::vector<int> &needed) {
+    if (needed.empty()) return 0.0;
+    auto it = memo.find(needed);
+    if (it != memo.end()) return it->second.first;
+    const int t = needed.back(); // largest handle: nothing else still needed depends on it being produced later
+    std::vector<int> rest(needed.begin(), needed.end() - 1);
+    double best = 1e300;
+    long bestEdge = -1;
+    for (size_t e : producers[t]) {
+      std::vector<int> sub = rest;
+      for (int in : g.edges[e].inputs)
+        if (!model.tensors()[in].isInput) sub.push_back(in);
+      std::sort(sub.begin(), sub.end());
+      sub.erase(std::unique(sub.begin(), sub.end()), sub.end());
+      const double c = cost[e] + solve(sub);
+      if (c < best) { best = c; bestEdge = static_cast<long>(e); }
+    }
+    memo[needed] = {best, bestEdge};
+    return best;
+  }
+};
+} // namespace
+
+std::vector<size_t> select_schedule(const Model &model, const SuperGraph &g, const std::vector<double> &edgeCost) {
+  Selector s{model, g, edgeCost, {}, {}};
+  s.producers.resize(model.tensors().size());
+  for (size_t e = 0; e < g.edges.size(); ++e) {
+    const auto &edge = g.edges[e];
+    for (int in : edge.inputs)
+      if (in >= edge.output) fail(Status::Internal, "super-graph edge is not topologically ordered");
+    s.producers[edge.output].push_back(e);
+  }
+  std::vector<int> needed;
+  for (TensorHandle o : model.outputs())
+    if (!model.tensors()[o].isInput) needed.push_back(o);
+  std::sort(needed.begin(), needed.end());
+  needed.erase(std::unique(needed.begin(), needed.end()), needed.end());
+  const double total = s.solve(needed);
+  if (total >= 1e299) fail(Status::Unsupported, "no kernel implements part of this graph (a layer has no matching shader)");
+  // walk the memo to recover the chosen edges
+  std::vector<size_t> chosen;
+  std::vector<int> cur = needed;
+  while (!cur.empty()) {
+    const auto &entry = s.memo.at(cur);
+    const size_t e = static_cast<size_t>(entry.second);
+    chosen.push_back(e);
+    std::vector<int> sub(cur.begin(), cur.end() - 1);
+    for (int in : g.edges[e].inputs)
+      if (!model.tensors()[in].isInput) sub.push_back(in);
+    std::sort(sub.begin(), sub.end());
+    sub.erase(std::unique(sub.begin(), sub.end()), sub.end());
+    cur = std::move(sub);
+  }
+  // producers come before consumers when sorted by output handle
+  std::sort(chosen.begin(), chosen.end(), [&](size_t a, size_t b) { return g.edges[a].output < g.edges[b].output; });
+  return chosen;
+}
+
+static dnx::ScalarSource src(Sym s, dnx::ScalarType t = dnx::ScalarType::I64) { return dnx::ScalarSource::fromSym(s, t); }
+
+std::vector<uint8_t> compile(const Model &modelIn, const hip::HipCompiler &hipc, const Db *db, const CompileOptions &opt, CompileReport *report) {
+  if (modelIn.outputs().empty()) fail(Status::InvalidArgument, "model has no outputs");
+  Model model = modelIn; // the symbol graph grows while dispatches are built
+  SymGraph &sym = model.symGraph();
+  const auto shaders = get_all_shaders(&hipc);
+  SuperGraph g = implement(model, sym, shaders, opt);
+  const std::vector<int64_t> dp = assumed_symeval(model, sym, opt);
+  std::vector<double> cost(g.edges.size());
+  std::vector<bool> measured(g.edges.size());
+  for (size_t e = 0; e < g.edges.size(); ++e) {
+    bool m = false;
+    cost[e] = edge_cost_ms(g.edges[e], dp, db, opt, &m);
+    measured[e] = m;
+  }
+  const std::vector<size_t> chosen = select_schedule(model, g, cost);
+
+  dnx::Model out;
+  out.version = 0;
+  out.info.producer = "denox-hip";
+  out.info.producer_version = "0.1";
+
+  // ---- placement: one buffer per live tensor (placement.cpp:232-300 of the reference) ----
+  std::map<uint32_t, uint32_t> tensorIndex; // super-graph tensor -> dnx tensor
+  auto place = [&](uint32_t st) -> uint32_t {
+    auto it = tensorIndex.find(st);
+    if (it != tensorIndex.end()) return it->second;
+    const SuperTensor &t = g.tensors[st];
+    dnx::Buffer b;
+    b.size = src(t.byteSize);
+    b.alignment = t.alignment;
+    out.buffers.push_back(b);
+    dnx::Tensor dt;
+    dt.buffer = static_cast<uint32_t>(out.buffers.size() - 1);
+    dt.offset = src(Sym::Const(0));
+    dt.size = src(t.byteSize);
+    dt.info.format = t.format;
+    dt.info.type = t.type;
+    dt.info.name = t.name;
+    if (t.modelTensor >= 0) {
+      const TensorNode &n = model.tensors()[t.modelTensor];
+      dt.info.has_extent = true;
+      dt.info.width = src(n.width);
+      dt.info.height = src(n.height);
+      dt.info.channels = src(Sym::Const(n.channels));
+    }
+    out.tensors.push_back(std::move(dt));
+    const uint32_t id = static_cast<uint32_t>(out.tensors.size() - 1);
+    tensorIndex.emplace(st, id);
+    return id;
+  };
+
+  // ---- kernels: distinct variants by hash (compile_shaders.cpp:35-48 of the reference) ----
+  std::map<std::string, uint32_t> binaryIndex;
+  auto binaryOf = [&](const hip::HipCompilerInstance &k) -> uint32_t {
+    const std::string key = k.sha256();
+    auto it = binaryIndex.find(key);
+    if (it != binaryIndex.end()) return it->second;
+    dnx::ShaderBinary sb;
+    sb.code_object = k.compile();
+    out.shader_binaries.push_back(std::move(sb));
+    const uint32_t id = static_cast<uint32_t>(out.shader_binaries.size() - 1);
+    binaryIndex.emplace(key, id);
+    return id;
+  };
+
+  auto emitDispatch = [&](const ComputeDispatch &d) {
+    dnx::ComputeDispatch o;
+    o.binary_id = binaryOf(d.kernel);
+    o.entry_point = d.entryPoint;
+    o.workgroup_count_x = src(d.workgroupCountX);
+    o.workgroup_count_y = src(d.workgroupCountY);
+    o.workgroup_count_z = src(d.workgroupCountZ);
+    for (int i = 0; i < 3; ++i) o.workgroup_size[i] = d.workgroupSize[i];
+    dnx::DescriptorSetBinding set;
+    set.set = 0;
+    for (const auto &b : d.bindings) set.bindings.push_back(dnx::DescriptorBinding{b.binding, b.access, place(b.tensor.index)});
+    o.bindings.push_back(std::move(set));
+    uint16_t off = 0;
+    for (const auto &pc : d.pushConstants) {
+      const uint16_t sz = static_cast<uint16_t>(dnx::scalarSize(pc.dtype));
+      off = static_cast<uint16_t>((off + sz - 1) / sz * sz);
+      o.push_constant.fields.push_back(dnx::PushConstantField{pc.dtype, off, src(pc.value, pc.dtype)});
+      off = static_cast<uint16_t>(off + sz);
+    }
+    o.push_constant.size = off;
+    o.info.name = d.info.name;
+    o.info.debug_info = d.info.config.empty() ? d.kernel.defineString() : d.info.config + " | " + d.kernel.defineString();
+    o.info.src_path = d.info.srcPath;
+    o.info.has_reads = d.info.hasReads; o.info.memory_reads = src(d.info.memoryReads);
+    o.info.has_writes = d.info.hasWrites; o.info.memory_writes = src(d.info.memoryWrites);
+    o.info.has_flops = d.info.hasFlops; o.info.flops = src(d.info.flops);
+    out.dispatches.push_back(std::move(o));
+  };
+
+  // ---- interface tensors and layout conversion ----
+  auto formatOf = [](const std::vector<InterfaceTensorDescriptor> &descs, const std::string &name, size_t index) {
+    for (const auto &d : descs) if (d.name == name) return d.format;
+    if (index < descs.size() && descs[index].name.empty()) return descs[index].format;
+    return dnx::TensorFormat::SSBO_HWC;
+  };
+  auto layoutId = [](dnx::TensorFormat f) -> int {
+    switch (f) {
+    case dnx::TensorFormat::SSBO_HWC: return 0;
+    case dnx::TensorFormat::SSBO_CHW: return 1;
+    case dnx::TensorFormat::SSBO_CHWC8: return 2;
+    default: fail(Status::Unsupported, "interface tensors must be SSBO_HWC, SSBO_CHW or SSBO_CHWC8");
+    }
+  };
+  auto relayout = [&](TensorHandle t, dnx::TensorFormat from, dnx::TensorFormat to, bool external_is_source) -> uint32_t {
+    // creates the externally visible tensor in its declared format plus the conversion dispatch
+    const TensorNode &n = model.tensors()[t];
+    if ((from == dnx::TensorFormat::SSBO_CHWC8 || to == dnx::TensorFormat::SSBO_CHWC8) && n.channels % 8) fail(Status::InvalidArgument, "CHWC8 needs a channel count divisible by 8");
+    SuperTensor ext = g.tensors[t];
+    ext.format = external_is_source ? from : to;
+    ext.name = n.name;
+    g.tensors.push_back(ext);
+    const uint32_t extId = static_cast<uint32_t>(g.tensors.size() - 1);
+    ComputeDispatch d;
+    d.kernel = hipc.read("relayout.hip");
+    d.kernel.define("CH", n.channels); d.kernel.define("SRC_LAYOUT", layoutId(from)); d.kernel.define("DST_LAYOUT", layoutId(to));
+    d.entryPoint = "relayout";
+    d.workgroupCountX = sym.cdiv(sym.mul(n.width, n.height), 256);
+    d.workgroupCountY = d.workgroupCountZ = Sym::Const(1);
+    d.workgroupSize[0] = 256;
+    TensorBinding in{0, 0, dnx::Access::ReadOnly, TensorId{external_is_source ? extId : static_cast<uint32_t>(t)}, BindingType::Input};
+    TensorBinding ob{0, 1, dnx::Access::WriteOnly, TensorId{external_is_source ? static_cast<uint32_t>(t) : extId}, BindingType::Output};
+    d.bindings = {in, ob};
+    d.pushConstants = {PushConstantDesc{n.width, dnx::ScalarType::U32}, PushConstantDesc{n.height, dnx::ScalarType::U32}};
+    d.info.name = "relayout"; d.info.operation = "relayout"; d.info.srcPath = "relayout.hip";
+    d.info.hasReads = d.info.hasWrites = d.info.hasFlops = true;
+    d.info.memoryReads = d.info.memoryWrites = g.tensors[t].byteSize;
+    d.info.flops = Sym::Const(0);
+    emitDispatch(d);
+    return place(extId);
+  };
+
+  for (size_t i = 0; i < model.inputs().size(); ++i) {
+    const TensorHandle t = model.inputs()[i];
+    const dnx::TensorFormat f = formatOf(opt.inputDescriptors, model.tensors()[t].name, i);
+    if (f == dnx::TensorFormat::SSBO_HWC) out.inputs.push_back(place(static_cast<uint32_t>(t)));
+    else out.inputs.push_back(relayout(t, f, dnx::TensorFormat::SSBO_HWC, true));
+  }
+
+  double total = 0.0;
+  for (size_t e : chosen) {
+    const SuperGraphEdge &edge = g.edges[e];
+    for (const auto &p : edge.parameters) {
+      const uint32_t id = place(p.tensor.index);
+      dnx::TensorInitializer init;
+      init.tensor = id;
+      init.data = p.lazyValue();
+      if (init.data.size() != static_cast<size_t>(g.tensors[p.tensor.index].byteSize.v)) fail(Status::Internal, "parameter blob size mismatch");
+      out.initializers.push_back(std::move(init));
+    }
+    for (const auto &d : edge.dispatches) emitDispatch(d);
+    // implicit concat: src0 at offset 0, src1 behind it, dst aliases both (placement.cpp:253-255 of the reference)
+    for (const auto &mc : edge.memoryConstrains) {
+      const uint32_t a = place(mc.src0.index), b = place(mc.src1.index), dd = place(mc.dst.index);
+      out.tensors[a].buffer = out.tensors[dd].buffer;
+      out.tensors[b].buffer = out.tensors[dd].buffer;
+      out.tensors[a].offset = src(Sym::Const(0));
+      out.tensors[b].offset = out.tensors[a].size;
+    }
+    total += cost[e];
+    if (report) {
+      report->schedule.push_back(ScheduleEntry{edge.shader, edge.config, edge.dispatches.empty() ? "" : edge.dispatches[0].info.name, cost[e], measured[e]});
+      if (db && !measured[e]) report->warnings.push_back("no measured latency for " + edge.shader + " " + edge.config + "; used the roofline estimate");
+    }
+  }
+
+  for (size_t i = 0; i < model.outputs().size(); ++i) {
+    const TensorHandle t = model.outputs()[i];
+    const dnx::TensorFormat f = formatOf(opt.outputDescriptors, model.tensors()[t].name, i);
+    if (f == dnx::TensorFormat::SSBO_HWC) out.outputs.push_back(place(static_cast<uint32_t>(t)));
+    else out.outputs.push_back(relayout(t, dnx::TensorFormat::SSBO_HWC, f, false));
+  }
+
+  out.sym_ir = sym.compile();
+  for (const auto &nv : model.valueNames()) out.value_names.push_back(dnx::ValueName{nv.name, src(nv.value)});
+  dnx::validate(out);
+  if (report) {
+    report->superGraphEdges = g.edges.size();
+    report->selectedEdges = chosen.size();
+    report->dispatches = out.dispatches.size();
+    report->estimatedMs = total;
+    report->kernelsCompiled = hipc.stats().compiled;
+    report->kernelCacheHits = hipc.stats().cacheHits;
+  }
+  return dnx::serialize(out);
+}
+
+size_t populate(Db &db, const Model &modelIn, const hip::HipCompiler &hipc, const CompileOptions &opt) {
+  Model model = modelIn;
+  SymGraph &sym = model.symGraph();
+  const auto shaders = get_all_shaders(&hipc);
+  const SuperGraph g = implement(model, sym, shaders, opt);
+  const std::vector<int64_t> dp = assumed_symeval(model, sym, opt);
+  size_t added = 0;
+  for (const auto &edge : g.edges)
+    for (const auto &d : edge.dispatches) {
+      DbDispatch row;
+      row.sha256 = d.kernel.sha256();
+      row.pushConstants = push_constant_bytes(d, dp);
+      row.wg[0] = static_cast<uint32_t>(symValue(dp, d.workgroupCountX));
+      row.wg[1] = static_cast<uint32_t>(symValue(dp, d.workgroupCountY));
+      row.wg[2] = static_cast<uint32_t>(symValue(dp, d.workgroupCountZ));
+      row.srcPath = d.kernel.sourcePath();
+      row.defines = d.kernel.defineString();
+      row.entryPoint = d.entryPoint;
+      for (int i = 0; i < 3; ++i) row.block[i] = d.workgroupSize[i];
+      for (const auto &b : d.bindings) {
+        const SuperTensor &t = g.tensors[b.tensor.index];
+        row.bindings.push_back(DbBinding{static_cast<uint64_t>(symValue(dp, t.byteSize)), t.alignment, t.isParam, static_cast<uint8_t>(b.access)});
+      }
+      row.operation = d.info.operation; row.shader = edge.shader; row.config = d.info.config;
+      row.memoryReads = d.info.hasReads ? static_cast<uint64_t>(symValue(dp, d.info.memoryReads)) : 0;
+      row.memoryWrites = d.info.hasWrites ? static_cast<uint64_t>(symValue(dp, d.info.memoryWrites)) : 0;
+      row.flops = d.info.hasFlops ? static_cast<uint64_t>(symValue(dp, d.info.flops)) : 0;
+      const size_t before = db.rows().size();
+      db.insert_dispatch(row);
+      if (db.rows().size() > before) ++added;
+    }
+  return added;
+}
+
+} // namespace denox::compiler

@@ -1,0 +1,147 @@
+#include "model.hpp"
+
+namespace denox::compiler {
+
+const TensorNode &Model::get(TensorHandle h) const {
+  if (h < 0 || static_cast<size_t>(h) >= m_tensors.size()) fail(Status::InvalidArgument, "invalid tensor handle");
+  return m_tensors[static_cast<size_t>(h)];
+}
+
+TensorHandle Model::newTensor(Sym w, Sym h, unsigned c, int producer) {
+  TensorNode t;
+  t.width = w; t.height = h; t.channels = c; t.producer = producer;
+  m_tensors.push_back(std::move(t));
+  return static_cast<TensorHandle>(m_tensors.size() - 1);
+}
+
+TensorHandle Model::input(const std::string &name, Sym width, Sym height, unsigned channels) {
+  if (channels == 0) fail(Status::InvalidArgument, "input with zero channels");
+  TensorHandle t = newTensor(width, height, channels, -1);
+  m_tensors[t].name = name;
+  m_tensors[t].isInput = true;
+  m_inputs.push_back(t);
+  return t;
+}
+
+TensorHandle Model::conv2d(TensorHandle src, unsigned K, unsigned C, unsigned R, unsigned S, const uint16_t *w,
+                           const uint16_t *bias, unsigned strideX, unsigned strideY, unsigned padX, unsigned padY,
+                           unsigned dilX, unsigned dilY) {
+  const TensorNode in = get(src);
+  if (in.channels != C) fail(Status::InvalidArgument, "conv2d: filter expects " + std::to_string(C) + " input channels, tensor has " + std::to_string(in.channels));
+  if (!w || K == 0 || R == 0 || S == 0 || strideX == 0 || strideY == 0 || dilX == 0 || dilY == 0) fail(Status::InvalidArgument, "conv2d: bad filter description");
+  Op op;
+  op.kind = OpKind::Conv;
+  op.inputs = {src};
+  op.K = K; op.C = C; op.R = R; op.S = S;
+  op.weights.assign(w, w + static_cast<size_t>(K) * C * R * S);
+  op.hasBias = bias != nullptr;
+  if (bias) op.bias.assign(bias, bias + K);
+  op.strideX = strideX; op.strideY = strideY; op.padX = padX; op.padY = padY; op.dilX = dilX; op.dilY = dilY;
+  const Sym ow = m_sym.pool(in.width, S, padX, strideX, dilX);
+  const Sym oh = m_sym.pool(in.height, R, padY, strideY, dilY);
+  op.output = newTensor(ow, oh, K, static_cast<int>(m_ops.size()));
+  m_tensors[src].consumers.push_back(static_cast<int>(m_ops.size()));
+  m_ops.push_back(std::move(op));
+  return m_ops.back().output;
+}
+
+TensorHandle Model::activation(TensorHandle src, ActivationFunction func, float alpha) {
+  const TensorNode in = get(src);
+  Op op;
+  op.kind = OpKind::Activation;
+  op.inputs = {src};
+  op.func = func; op.alpha = alpha;
+  op.output = newTensor(in.width, in.height, in.channels, static_cast<int>(m_ops.size()));
+  m_tensors[src].consumers.push_back(static_cast<int>(m_ops.size()));
+  m_ops.push_back(std::move(op));
+  return m_ops.back().output;
+}
+
+TensorHandle Model::upsample(TensorHandle src, unsigned f, FilterMode) {
+  const TensorNode in = get(src);
+  if (f == 0) fail(Status::InvalidArgument, "upsample: zero scaling factor");
+  Op op;
+  op.kind = OpKind::Upsample;
+  op.inputs = {src};
+  op.scale = f;
+  op.output = newTensor(m_sym.mul(in.width, f), m_sym.mul(in.height, f), in.channels, static_cast<int>(m_ops.size()));
+  m_tensors[src].consumers.push_back(static_cast<int>(m_ops.size()));
+  m_ops.push_back(std::move(op));
+  return m_ops.back().output;
+}
+
+TensorHandle Model::pool(TensorHandle src, unsigned kx, unsigned ky, unsigned px, unsigned py, unsigned sx, unsigned sy, PoolFunction) {
+  const TensorNode in = get(src);
+  if (kx == 0 || ky == 0 || sx == 0 || sy == 0) fail(Status::InvalidArgument, "pool: bad window");
+  Op op;
+  op.kind = OpKind::Pool;
+  op.inputs = {src};
+  op.kernelX = kx; op.kernelY = ky; op.poolPadX = px; op.poolPadY = py; op.poolStrideX = sx; op.poolStrideY = sy;
+  op.output = newTensor(m_sym.pool(in.width, kx, px, sx, 1), m_sym.pool(in.height, ky, py, sy, 1), in.channels, static_cast<int>(m_ops.size()));
+  m_tensors[src].consumers.push_back(static_cast<int>(m_ops.size()));
+  m_ops.push_back(std::move(op));
+  return m_ops.back().output;
+}
+
+TensorHandle Model::concat(TensorHandle src0, TensorHandle src1) {
+  const TensorNode a = get(src0), b = get(src1);
+  // extents must agree; when both are constants this is checked here, symbolic
+  // extents are the caller's responsibility (as in the reference importer)
+  if (a.width.isConst() && b.width.isConst() && a.width.v != b.width.v) fail(Status::InvalidArgument, "concat: widths differ");
+  if (a.height.isConst() && b.height.isConst() && a.height.v != b.height.v) fail(Status::InvalidArgument, "concat: heights differ");
+  Op op;
+  op.kind = OpKind::Concat;
+  op.inputs = {src0, src1};
+  op.output = newTensor(a.width, a.height, a.channels + b.channels, static_cast<int>(m_ops.size()));
+  m_tensors[src0].consumers.push_back(static_cast<int>(m_ops.size()));
+  m_tensors[src1].consumers.push_back(static_cast<int>(m_ops.size()));
+  m_ops.push_back(std::move(op));
+  return m_ops.back().output;
+}
+
+TensorHandle Model::pad(TensorHandle src, Sym left, Sym right, Sym top, Sym bottom, PaddingMode) {
+  const TensorNode in = get(src);
+  Op op;
+  op.kind = OpKind::Pad;
+  op.inputs = {src};
+  op.left = left; op.right = right; op.top = top; op.bottom = bottom;
+  op.output = newTensor(m_sym.add(m_sym.add(in.width, left), right), m_sym.add(m_sym.add(in.height, top), bottom), in.channels, static_cast<int>(m_ops.size()));
+  m_tensors[src].consumers.push_back(static_cast<int>(m_ops.size()));
+  m_ops.push_back(std::move(op));
+  return m_ops.back().output;
+}
+
+TensorHandle Model::slice(TensorHandle src, Sym left, Sym right, Sym top, Sym bottom) {
+  const TensorNode in = get(src);
+  Op op;
+  op.kind = OpKind::Slice;
+  op.inputs = {src};
+  op.left = left; op.right = right; op.top = top; op.bottom = bottom;
+  // [left, right) x [top, bottom) in source coordinates (frontend/model/Model.cpp:233-253 of the reference)
+  op.output = newTensor(m_sym.sub(right, left), m_sym.sub(bottom, top), in.channels, static_cast<int>(m_ops.size()));
+  m_tensors[src].consumers.push_back(static_cast<int>(m_ops.size()));
+  m_ops.push_back(std::move(op));
+  return m_ops.back().output;
+}
+
+void Model::output(TensorHandle src, const std::string &name) {
+  (void)get(src);
+  m_tensors[src].isOutput = true;
+  if (m_tensors[src].name.empty()) m_tensors[src].name = name;
+  m_outputs.push_back(src);
+}
+
+void Model::assignValueName(const std::string &name, Sym value) {
+  for (auto &nv : m_valueNames)
+    if (nv.name == name) { nv.value = value; return; }
+  m_valueNames.push_back(NamedValue{name, value});
+}
+
+Sym Model::requireValueOfName(const std::string &name) {
+  for (const auto &nv : m_valueNames) if (nv.name == name) return nv.value;
+  Sym v = m_sym.var(name);
+  m_valueNames.push_back(NamedValue{name, v});
+  return v;
+}
+
+} // namespace denox::compiler

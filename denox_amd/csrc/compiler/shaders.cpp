@@ -1,0 +1,442 @@
+// Kernel families.  Each one matches a pattern of layer operations, lists the
+// configurations it can be compiled in and registers the dispatches.
+//
+// Counterparts in the reference (compiler/src/denox/compiler/implement/shaders/):
+//   ConvMfmaShader        conv/DirectConvShader.cpp:26-575, conv/DirectConvShaderCM.cpp:40-695,
+//                         conv/ConcatConvCMShader.cpp:39-965
+//   BasicPoolShader       pool/BasicPoolShader.cpp:11-610
+//   BasicUpsampleShader   upsample/BasicUpsampleShader.cpp:13-604
+//   CopyTransformShader   copy/CopyTransformShader.cpp:155-541
+//   BasicActivationShader activation/BasicActivationShader.cpp
+//   MemoryPadShader       pad/MemoryPadShader.cpp
+//   MemorySliceShader     slice/MemorySliceShader.cpp
+// registry: shaders.cpp:16-50.
+#include "implement.hpp"
+#include "../common/f16.hpp"
+#include <algorithm>
+#include <cstring>
+#include <sstream>
+
+namespace denox::compiler {
+
+namespace {
+
+constexpr unsigned WG_BANDWIDTH = 256; // threads per workgroup of the bandwidth kernels
+
+bool singleUse(const Model &m, TensorHandle t) {
+  const TensorNode &n = m.tensors()[t];
+  return n.consumers.size() == 1 && !n.isOutput;
+}
+
+Sym bytesOf(SymGraph &sym, const TensorNode &t) { return sym.mul(sym.mul(t.width, t.height), static_cast<int64_t>(t.channels) * 2); }
+
+std::string fmtFloat(float v) {
+  std::ostringstream o;
+  o.precision(9);
+  o << std::scientific << v << "f";
+  return o.str();
+}
+
+// ------------------------------------------------------------------ conv
+struct ConvConfig { unsigned waves, rpw, ck; const char *name; };
+const ConvConfig kConvConfigs[] = {
+    {4, 2, 16, "w4r2k16"}, {4, 2, 32, "w4r2k32"}, {4, 4, 16, "w4r4k16"}, {4, 4, 32, "w4r4k32"},
+    {8, 2, 16, "w8r2k16"}, {8, 2, 32, "w8r2k32"}, {4, 2, 64, "w4r2k64"}, {8, 1, 16, "w8r1k16"},
+};
+constexpr unsigned kNumConvConfigs = sizeof(kConvConfigs) / sizeof(kConvConfigs[0]);
+
+enum ConvPatternBits : unsigned { PAT_CONCAT = 1, PAT_UPSAMPLE = 2, PAT_ACT = 4, PAT_POOL = 8 };
+
+struct ConvGeometry {
+  unsigned CA, CB, C, CPAD, K, KOUTP, KT;
+  size_t ldsBytes;
+};
+
+// Output channels per workgroup: the largest divisor of KOUTP (in blocks of 32)
+// whose weight slice fits LDS next to the halo and whose accumulators fit the
+// register file.
+bool chooseKT(const ConvConfig &cfg, unsigned CA, unsigned CB, unsigned K, unsigned ldsLimit, ConvGeometry &g) {
+  g.CA = CA; g.CB = CB; g.C = CA + CB; g.CPAD = (g.C + 15) / 16 * 16; g.K = K; g.KOUTP = (K + 31) / 32 * 32;
+  const unsigned th = cfg.waves * cfg.rpw;
+  const unsigned haloPix = (th + 2) * 34;
+  const unsigned ckp = cfg.ck + 8;
+  const unsigned blocks = g.KOUTP / 32;
+  for (unsigned kb = blocks; kb >= 1; --kb) {
+    if (blocks % kb) continue;
+    if (kb * cfg.rpw > 8) continue; // <= 128 accumulator registers per lane
+    const size_t lds = (static_cast<size_t>(haloPix) + 9u * kb * 32u) * ckp * 2u;
+    if (lds > ldsLimit) continue;
+    g.KT = kb * 32;
+    g.ldsBytes = lds;
+    return true;
+  }
+  return false;
+}
+
+// Weight layout the kernel reads: [kt][chunk][tap r*3+s][KT rows][len(chunk)], rows
+// permuted so that MFMA row rho of a 32-block holds output channel
+// 16*((rho>>2)&1) + 4*(rho>>3) + (rho&3) of that block; zero for c >= C or k >= K.
+std::vector<uint8_t> packConvWeights(const Op &conv, const ConvGeometry &g, unsigned ck) {
+  std::vector<uint16_t> out(static_cast<size_t>(g.KOUTP) * 9 * g.CPAD, 0);
+  const unsigned nkt = g.KOUTP / g.KT;
+  size_t pos = 0;
+  for (unsigned kt = 0; kt < nkt; ++kt)
+    for (unsigned c0 = 0; c0 < g.CPAD; c0 += ck) {
+      const unsigned len = std::min(ck, g.CPAD - c0);
+      for (unsigned tap = 0; tap < 9; ++tap) {
+        const unsigned r = tap / 3, s = tap % 3;
+        for (unsigned row = 0; row < g.KT; ++row) {
+          const unsigned rho = row & 31;
+          const unsigned k = kt * g.KT + (row & ~31u) + 16 * ((rho >> 2) & 1) + 4 * (rho >> 3) + (rho & 3);
+          for (unsigned e = 0; e < len; ++e, ++pos) {
+            const unsigned c = c0 + e;
+            if (k < g.K && c < g.C) out[pos] = conv.weights[((static_cast<size_t>(k) * g.C + c) * 3 + r) * 3 + s];
+          }
+        }
+      }
+    }
+  std::vector<uint8_t> bytes(out.size() * 2);
+  std::memcpy(bytes.data(), out.data(), bytes.size());
+  return bytes;
+}
+
+class ConvMfmaShader final : public IShader {
+public:
+  explicit ConvMfmaShader(const hip::HipCompiler *c) : m_compiler(c) {}
+  std::string name() const override { return "conv3x3_mfma"; }
+
+  std::vector<Match> matchAll(const Model &model, const CompileOptions &opt) const override {
+    std::vector<Match> out;
+    const auto &ops = model.ops();
+    for (size_t i = 0; i < ops.size(); ++i) {
+      const Op &conv = ops[i];
+      if (conv.kind != OpKind::Conv) continue;
+      if (conv.R != 3 || conv.S != 3 || conv.strideX != 1 || conv.strideY != 1 || conv.padX != 1 || conv.padY != 1 || conv.dilX != 1 || conv.dilY != 1) continue;
+      struct Pro { unsigned bits; std::vector<int> ops; std::vector<int> inputs; };
+      std::vector<Pro> pros;
+      const TensorHandle in = conv.inputs[0];
+      pros.push_back(Pro{0, {}, {in}});
+      const int prod = model.tensors()[in].producer;
+      if (prod >= 0 && singleUse(model, in)) {
+        const Op &p = ops[prod];
+        if (p.kind == OpKind::Concat && opt.features.enableConcatConvFusion) {
+          pros.push_back(Pro{PAT_CONCAT, {prod}, {p.inputs[0], p.inputs[1]}});
+          const TensorHandle a = p.inputs[0];
+          const int ap = model.tensors()[a].producer;
+          if (ap >= 0 && singleUse(model, a) && ops[ap].kind == OpKind::Upsample && ops[ap].scale == 2 && opt.features.enableUpsampleFusion)
+            pros.push_back(Pro{PAT_CONCAT | PAT_UPSAMPLE, {ap, prod}, {ops[ap].inputs[0], p.inputs[1]}});
+        } else if (p.kind == OpKind::Upsample && p.scale == 2 && opt.features.enableUpsampleFusion) {
+          pros.push_back(Pro{PAT_UPSAMPLE, {prod}, {p.inputs[0]}});
+        }
+      }
+      struct Epi { unsigned bits; std::vector<int> ops; int output; };
+      std::vector<Epi> epis;
+      epis.push_back(Epi{0, {}, conv.output});
+      auto poolOk = [](const Op &q) { return q.kind == OpKind::Pool && q.kernelX == 2 && q.kernelY == 2 && q.poolStrideX == 2 && q.poolStrideY == 2 && q.poolPadX == 0 && q.poolPadY == 0; };
+      if (singleUse(model, conv.output)) {
+        const int c1 = model.tensors()[conv.output].consumers[0];
+        const Op &n1 = ops[c1];
+        if (n1.kind == OpKind::Activation && opt.features.enableConvReluFusion) {
+          epis.push_back(Epi{PAT_ACT, {c1}, n1.output});
+          if (singleUse(model, n1.output)) {
+            const int c2 = model.tensors()[n1.output].consumers[0];
+            if (poolOk(ops[c2]) && opt.features.enablePoolFusion) epis.push_back(Epi{PAT_ACT | PAT_POOL, {c1, c2}, ops[c2].output});
+          }
+        } else if (poolOk(n1) && opt.features.enablePoolFusion) {
+          epis.push_back(Epi{PAT_POOL, {c1}, n1.output});
+        }
+      }
+      for (const auto &p : pros)
+        for (const auto &e : epis) {
+          Match m;
+          m.pattern = p.bits | e.bits;
+          m.ops = p.ops;
+          m.ops.push_back(static_cast<int>(i));
+          m.ops.insert(m.ops.end(), e.ops.begin(), e.ops.end());
+          m.inputs = p.inputs;
+          m.output = e.output;
+          out.push_back(std::move(m));
+        }
+    }
+    return out;
+  }
+
+  const Op &convOf(const Model &model, const Match &m) const {
+    for (int o : m.ops) if (model.ops()[o].kind == OpKind::Conv) return model.ops()[o];
+    fail(Status::Internal, "conv match without conv");
+  }
+
+  std::vector<unsigned> acceptMatch(const Model &model, const Match &m, const CompileOptions &opt) const override {
+    const Op &conv = convOf(model, m);
+    const unsigned CA = model.tensors()[m.inputs[0]].channels;
+    const unsigned CB = m.inputs.size() > 1 ? model.tensors()[m.inputs[1]].channels : 0;
+    const unsigned cpad = (CA + CB + 15) / 16 * 16;
+    std::vector<unsigned> out;
+    for (unsigned c = 0; c < kNumConvConfigs; ++c) {
+      const ConvConfig &cfg = kConvConfigs[c];
+      if (!opt.forceConvConfig.empty() && opt.forceConvConfig != cfg.name) continue;
+      if (cfg.ck > cpad && cfg.ck != 16) continue; // a larger stage than the whole reduction adds nothing
+      if ((m.pattern & PAT_POOL) && (cfg.rpw % 2)) continue;
+      if (cfg.waves * 64 > opt.deviceInfo.maxComputeWorkGroupInvocations) continue;
+      ConvGeometry g;
+      if (!chooseKT(cfg, CA, CB, conv.K, ldsLimit(opt), g)) continue;
+      out.push_back(c);
+    }
+    if (out.empty() && !opt.forceConvConfig.empty()) fail(Status::Unsupported, "conv configuration '" + opt.forceConvConfig + "' is not valid for this layer");
+    return out;
+  }
+
+  static unsigned ldsLimit(const CompileOptions &opt) { return opt.deviceInfo.maxComputeSharedMemory; }
+
+  size_t parameterMemorySize(const Model &model, const Match &m) const override {
+    const Op &conv = convOf(model, m);
+    const unsigned C = conv.C, cpad = (C + 15) / 16 * 16, kp = (conv.K + 31) / 32 * 32;
+    return static_cast<size_t>(kp) * 9 * cpad * 2 + static_cast<size_t>(kp) * 2;
+  }
+
+  void implement(OpImpl &impl, const Model &model, const Match &m, unsigned config, SymGraph &sym, const CompileOptions &opt) const override {
+    const ConvConfig &cfg = kConvConfigs[config];
+    const Op &conv = convOf(model, m);
+    const TensorNode &convIn = model.tensors()[conv.inputs[0]];
+    const TensorNode &tA = model.tensors()[m.inputs[0]];
+    const unsigned CA = tA.channels;
+    const unsigned CB = m.inputs.size() > 1 ? model.tensors()[m.inputs[1]].channels : 0;
+    ConvGeometry g;
+    if (!chooseKT(cfg, CA, CB, conv.K, ldsLimit(opt), g)) fail(Status::Internal, "conv config rejected at implement time");
+    int act = 0;
+    float alpha = 0.0f;
+    for (int o : m.ops)
+      if (model.ops()[o].kind == OpKind::Activation) {
+        act = model.ops()[o].func == ActivationFunction::ReLU ? 1 : 2;
+        alpha = model.ops()[o].alpha;
+      }
+    const bool pool = (m.pattern & PAT_POOL) != 0, up = (m.pattern & PAT_UPSAMPLE) != 0;
+
+    hip::HipCompilerInstance k = m_compiler->read("conv3x3_mfma.hip");
+    k.define("CA", CA); k.define("CB", CB); k.define("UPA", up ? 1 : 0);
+    k.define("KOUT", conv.K); k.define("KT", g.KT);
+    k.define("ACT", act);
+    if (act == 2) k.define("ALPHA", fmtFloat(alpha));
+    k.define("POOL", pool ? 1 : 0); k.define("HAS_BIAS", conv.hasBias ? 1 : 0);
+    k.define("WAVES", cfg.waves); k.define("RPW", cfg.rpw); k.define("CK", cfg.ck);
+
+    const Sym W = convIn.width, H = convIn.height;
+    const unsigned th = cfg.waves * cfg.rpw;
+    auto d = impl.registerDispatch(k, "conv3x3_mfma", sym.cdiv(W, 32), sym.cdiv(H, th), Sym::Const(g.KOUTP / g.KT), cfg.waves * 64);
+    d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
+    if (CB) d.addBinding(dnx::Access::ReadOnly, m.inputs[1]);
+    d.addBinding(dnx::Access::WriteOnly, m.output);
+    const Op convCopy = conv; // the lazy packers outlive the model reference
+    const unsigned ck = cfg.ck;
+    TensorId wt = impl.createParameter(static_cast<size_t>(g.KOUTP) * 9 * g.CPAD * 2, dnx::ScalarType::F16,
+                                       [convCopy, g, ck]() { return packConvWeights(convCopy, g, ck); });
+    d.addParamBinding(wt);
+    if (conv.hasBias) {
+      const unsigned koutp = g.KOUTP;
+      TensorId bt = impl.createParameter(static_cast<size_t>(koutp) * 2, dnx::ScalarType::F16, [convCopy, koutp]() {
+        std::vector<uint8_t> b(static_cast<size_t>(koutp) * 2, 0);
+        std::memcpy(b.data(), convCopy.bias.data(), convCopy.bias.size() * 2);
+        return b;
+      });
+      d.addParamBinding(bt);
+    }
+    d.addPushConstant(W, dnx::ScalarType::U32);
+    d.addPushConstant(H, dnx::ScalarType::U32);
+
+    std::string nm = "conv3x3";
+    if (up) nm = "upsample+" + nm;
+    if (m.pattern & PAT_CONCAT) nm = "concat+" + nm;
+    if (act == 1) nm += "+relu"; else if (act == 2) nm += "+leaky_relu";
+    if (pool) nm += "+maxpool";
+    d.setName(nm);
+    d.setOperation(nm);
+    d.setConfig(std::string(cfg.name) + "/kt" + std::to_string(g.KT));
+    impl.edge().config = cfg.name;
+    // bytes that cross HBM: sources at their stored resolution, weights, bias; the (pooled) output
+    Sym reads = bytesOf(sym, tA);
+    if (CB) reads = sym.add(reads, bytesOf(sym, model.tensors()[m.inputs[1]]));
+    reads = sym.add(reads, static_cast<int64_t>(conv.K) * conv.C * 9 * 2 + (conv.hasBias ? conv.K * 2 : 0));
+    d.setMemoryReads(reads);
+    d.setMemoryWrites(bytesOf(sym, model.tensors()[m.output]));
+    d.setFlops(sym.mul(sym.mul(W, H), static_cast<int64_t>(2) * 9 * conv.C * conv.K));
+  }
+
+private:
+  const hip::HipCompiler *m_compiler;
+};
+
+// ------------------------------------------------------------------ bandwidth kernels
+Sym linearGrid(SymGraph &sym, Sym w, Sym h, unsigned vectorsPerPixel) {
+  return sym.cdiv(sym.mul(sym.mul(w, h), static_cast<int64_t>(vectorsPerPixel)), WG_BANDWIDTH);
+}
+
+class SingleOpShader : public IShader {
+public:
+  SingleOpShader(const hip::HipCompiler *c, OpKind kind) : m_compiler(c), m_kind(kind) {}
+  std::vector<Match> matchAll(const Model &model, const CompileOptions &) const override {
+    std::vector<Match> out;
+    for (size_t i = 0; i < model.ops().size(); ++i) {
+      const Op &op = model.ops()[i];
+      if (op.kind != m_kind || !supports(op)) continue;
+      Match m;
+      m.ops = {static_cast<int>(i)};
+      m.inputs = op.inputs;
+      m.output = op.output;
+      out.push_back(std::move(m));
+    }
+    return out;
+  }
+  std::vector<unsigned> acceptMatch(const Model &, const Match &, const CompileOptions &) const override { return {0}; }
+  virtual bool supports(const Op &) const { return true; }
+
+protected:
+  const hip::HipCompiler *m_compiler;
+  OpKind m_kind;
+};
+
+class BasicPoolShader final : public SingleOpShader {
+public:
+  explicit BasicPoolShader(const hip::HipCompiler *c) : SingleOpShader(c, OpKind::Pool) {}
+  std::string name() const override { return "basic_pool"; }
+  // kernel == stride, no padding (the reference's restriction, BasicPoolShader.cpp:165-180)
+  bool supports(const Op &op) const override { return op.kernelX == op.poolStrideX && op.kernelY == op.poolStrideY && op.poolPadX == 0 && op.poolPadY == 0; }
+  void implement(OpImpl &impl, const Model &model, const Match &m, unsigned, SymGraph &sym, const CompileOptions &) const override {
+    const Op &op = model.ops()[m.ops[0]];
+    const TensorNode &in = model.tensors()[m.inputs[0]], &out = model.tensors()[m.output];
+    const unsigned vec = in.channels % 8 == 0 ? 8 : 1;
+    auto k = m_compiler->read("pool.hip");
+    k.define("CH", in.channels); k.define("KX", op.kernelX); k.define("KY", op.kernelY); k.define("VEC", vec);
+    auto d = impl.registerDispatch(k, "pool_max", linearGrid(sym, out.width, out.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
+    d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
+    d.addBinding(dnx::Access::WriteOnly, m.output);
+    d.addPushConstant(in.width); d.addPushConstant(in.height);
+    d.setName("maxpool"); d.setOperation("maxpool"); d.setConfig("vec" + std::to_string(vec));
+    d.setMemoryReads(bytesOf(sym, in)); d.setMemoryWrites(bytesOf(sym, out)); d.setFlops(Sym::Const(0));
+  }
+};
+
+class BasicUpsampleShader final : public SingleOpShader {
+public:
+  explicit BasicUpsampleShader(const hip::HipCompiler *c) : SingleOpShader(c, OpKind::Upsample) {}
+  std::string name() const override { return "basic_upsample"; }
+  void implement(OpImpl &impl, const Model &model, const Match &m, unsigned, SymGraph &sym, const CompileOptions &) const override {
+    const Op &op = model.ops()[m.ops[0]];
+    const TensorNode &in = model.tensors()[m.inputs[0]], &out = model.tensors()[m.output];
+    const unsigned vec = in.channels % 8 == 0 ? 8 : 1;
+    auto k = m_compiler->read("upsample.hip");
+    k.define("CH", in.channels); k.define("SCALE", op.scale); k.define("VEC", vec);
+    auto d = impl.registerDispatch(k, "upsample_nearest", linearGrid(sym, in.width, in.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
+    d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
+    d.addBinding(dnx::Access::WriteOnly, m.output);
+    d.addPushConstant(in.width); d.addPushConstant(in.height);
+    d.setName("upsample"); d.setOperation("upsample"); d.setConfig("vec" + std::to_string(vec));
+    d.setMemoryReads(bytesOf(sym, in)); d.setMemoryWrites(bytesOf(sym, out)); d.setFlops(Sym::Const(0));
+  }
+};
+
+class CopyTransformShader final : public SingleOpShader {
+public:
+  explicit CopyTransformShader(const hip::HipCompiler *c) : SingleOpShader(c, OpKind::Concat) {}
+  std::string name() const override { return "copy_transform"; }
+  // Explicit concat: one strided channel copy per source (CopyTransformShader.cpp:437-537).
+  // The reference's zero-dispatch implicit concat needs channel-block-major
+  // tensors (CHWC8, CopyTransformShader.cpp:198-237); activations here are
+  // pixel-major HWC, where the sources interleave per pixel and cannot alias.
+  void implement(OpImpl &impl, const Model &model, const Match &m, unsigned, SymGraph &sym, const CompileOptions &) const override {
+    const TensorNode &out = model.tensors()[m.output];
+    unsigned off = 0;
+    for (int s = 0; s < 2; ++s) {
+      const TensorNode &in = model.tensors()[m.inputs[s]];
+      const unsigned vec = (in.channels % 8 == 0 && off % 8 == 0 && out.channels % 8 == 0) ? 8 : 1;
+      auto k = m_compiler->read("copy_transform.hip");
+      k.define("IN_CH", in.channels); k.define("IN_CH_OFFSET", 0); k.define("OUT_CH", out.channels); k.define("OUT_CH_OFFSET", off);
+      k.define("COUNT", in.channels); k.define("VEC", vec);
+      auto d = impl.registerDispatch(k, "copy_transform", linearGrid(sym, in.width, in.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
+      d.addBinding(dnx::Access::ReadOnly, m.inputs[s]);
+      d.addBinding(dnx::Access::WriteOnly, m.output);
+      d.addPushConstant(in.width); d.addPushConstant(in.height);
+      d.setName(s == 0 ? "concat-copy-src0" : "concat-copy-src1"); d.setOperation("concat"); d.setConfig("vec" + std::to_string(vec));
+      d.setMemoryReads(bytesOf(sym, in)); d.setMemoryWrites(bytesOf(sym, in)); d.setFlops(Sym::Const(0));
+      off += in.channels;
+    }
+  }
+};
+
+class BasicActivationShader final : public SingleOpShader {
+public:
+  explicit BasicActivationShader(const hip::HipCompiler *c) : SingleOpShader(c, OpKind::Activation) {}
+  std::string name() const override { return "basic_activation"; }
+  void implement(OpImpl &impl, const Model &model, const Match &m, unsigned, SymGraph &sym, const CompileOptions &) const override {
+    const Op &op = model.ops()[m.ops[0]];
+    const TensorNode &in = model.tensors()[m.inputs[0]];
+    const unsigned vec = in.channels % 8 == 0 ? 8 : 1;
+    auto k = m_compiler->read("activation.hip");
+    k.define("CH", in.channels); k.define("VEC", vec); k.define("ACT", op.func == ActivationFunction::ReLU ? 1 : 2);
+    if (op.func == ActivationFunction::LeakyReLU) k.define("ALPHA", fmtFloat(op.alpha));
+    auto d = impl.registerDispatch(k, "activation", linearGrid(sym, in.width, in.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
+    d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
+    d.addBinding(dnx::Access::WriteOnly, m.output);
+    d.addPushConstant(in.width); d.addPushConstant(in.height);
+    const char *nm = op.func == ActivationFunction::ReLU ? "relu" : "leaky_relu";
+    d.setName(nm); d.setOperation(nm); d.setConfig("vec" + std::to_string(vec));
+    d.setMemoryReads(bytesOf(sym, in)); d.setMemoryWrites(bytesOf(sym, in));
+    d.setFlops(sym.mul(sym.mul(in.width, in.height), static_cast<int64_t>(in.channels))); // one FLOP per element, as the reference counts it
+  }
+};
+
+class MemoryPadShader final : public SingleOpShader {
+public:
+  explicit MemoryPadShader(const hip::HipCompiler *c) : SingleOpShader(c, OpKind::Pad) {}
+  std::string name() const override { return "memory_pad"; }
+  void implement(OpImpl &impl, const Model &model, const Match &m, unsigned, SymGraph &sym, const CompileOptions &) const override {
+    const Op &op = model.ops()[m.ops[0]];
+    const TensorNode &in = model.tensors()[m.inputs[0]], &out = model.tensors()[m.output];
+    const unsigned vec = in.channels % 8 == 0 ? 8 : 1;
+    auto k = m_compiler->read("pad.hip");
+    k.define("CH", in.channels); k.define("VEC", vec);
+    auto d = impl.registerDispatch(k, "memory_pad", linearGrid(sym, out.width, out.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
+    d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
+    d.addBinding(dnx::Access::WriteOnly, m.output);
+    d.addPushConstant(out.width); d.addPushConstant(out.height);
+    d.addPushConstant(op.left); d.addPushConstant(op.right); d.addPushConstant(op.top); d.addPushConstant(op.bottom);
+    d.setName("pad"); d.setOperation("pad"); d.setConfig("vec" + std::to_string(vec));
+    d.setMemoryReads(bytesOf(sym, in)); d.setMemoryWrites(bytesOf(sym, out)); d.setFlops(Sym::Const(0));
+  }
+};
+
+class MemorySliceShader final : public SingleOpShader {
+public:
+  explicit MemorySliceShader(const hip::HipCompiler *c) : SingleOpShader(c, OpKind::Slice) {}
+  std::string name() const override { return "memory_slice"; }
+  void implement(OpImpl &impl, const Model &model, const Match &m, unsigned, SymGraph &sym, const CompileOptions &) const override {
+    const Op &op = model.ops()[m.ops[0]];
+    const TensorNode &in = model.tensors()[m.inputs[0]], &out = model.tensors()[m.output];
+    const unsigned vec = in.channels % 8 == 0 ? 8 : 1;
+    auto k = m_compiler->read("slice.hip");
+    k.define("CH", in.channels); k.define("VEC", vec);
+    auto d = impl.registerDispatch(k, "memory_slice", linearGrid(sym, out.width, out.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
+    d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
+    d.addBinding(dnx::Access::WriteOnly, m.output);
+    d.addPushConstant(op.top); d.addPushConstant(op.left);
+    d.addPushConstant(in.width); d.addPushConstant(in.height);
+    d.addPushConstant(out.width); d.addPushConstant(out.height);
+    d.setName("slice"); d.setOperation("slice"); d.setConfig("vec" + std::to_string(vec));
+    d.setMemoryReads(bytesOf(sym, out)); d.setMemoryWrites(bytesOf(sym, out)); d.setFlops(Sym::Const(0));
+  }
+};
+
+} // namespace
+
+std::vector<std::unique_ptr<IShader>> get_all_shaders(const hip::HipCompiler *c) {
+  std::vector<std::unique_ptr<IShader>> s;
+  s.push_back(std::make_unique<ConvMfmaShader>(c));
+  s.push_back(std::make_unique<BasicPoolShader>(c));
+  s.push_back(std::make_unique<BasicUpsampleShader>(c));
+  s.push_back(std::make_unique<CopyTransformShader>(c));
+  s.push_back(std::make_unique<BasicActivationShader>(c));
+  s.push_back(std::make_unique<MemoryPadShader>(c));
+  s.push_back(std::make_unique<MemorySliceShader>(c));
+  return s;
+}
+
+} // namespace denox::compiler

@@ -1,0 +1,145 @@
+#include "hip_compiler.hpp"
+#include "../common/error.hpp"
+#include "../common/sha256.hpp"
+#include <cstdio>
+#include <cstdlib>
+#include <dirent.h>
+#include <dlfcn.h>
+#include <fstream>
+#include <hip/hiprtc.h>
+#include <sstream>
+#include <sys/stat.h>
+#include <unistd.h>
+#include <algorithm>
+
+namespace denox::hip {
+
+// Packed-fp32 instruction selection is switched off for every kernel.
+static const char *const kFlags[] = {"-O3", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-ffp-contract=off"};
+
+static std::string readFile(const std::string &path) {
+  std::ifstream f(path, std::ios::binary);
+  if (!f) fail(Status::IoError, "cannot read " + path);
+  std::ostringstream ss;
+  ss << f.rdbuf();
+  return ss.str();
+}
+
+std::string libraryDirectory() {
+  Dl_info info;
+  if (dladdr(reinterpret_cast<void *>(&libraryDirectory), &info) && info.dli_fname) {
+    std::string p = info.dli_fname;
+    const size_t slash = p.rfind('/');
+    return slash == std::string::npos ? "." : p.substr(0, slash);
+  }
+  return ".";
+}
+
+std::string defaultKernelDir() {
+  if (const char *e = std::getenv("DENOX_HIP_KERNEL_DIR")) return e;
+  return libraryDirectory() + "/../csrc/kernels";
+}
+
+std::string defaultCacheDir() {
+  if (const char *e = std::getenv("DENOX_HIP_CACHE_DIR")) return e;
+  return libraryDirectory() + "/../kernel_cache";
+}
+
+HipCompiler::HipCompiler(std::string kernelDir, std::string cacheDir, std::string arch)
+    : m_kernelDir(std::move(kernelDir)), m_cacheDir(std::move(cacheDir)), m_arch(std::move(arch)) {
+  std::vector<std::string> headers;
+  if (DIR *d = opendir(m_kernelDir.c_str())) {
+    while (dirent *e = readdir(d)) {
+      std::string n = e->d_name;
+      if (n.size() > 2 && n.substr(n.size() - 2) == ".h") headers.push_back(n);
+    }
+    closedir(d);
+  } else {
+    fail(Status::IoError, "kernel directory not found: " + m_kernelDir);
+  }
+  std::sort(headers.begin(), headers.end());
+  for (const auto &h : headers) m_headerDigest += "//" + h + "\n" + readFile(m_kernelDir + "/" + h);
+  if (!m_cacheDir.empty()) mkdir(m_cacheDir.c_str(), 0755);
+}
+
+HipCompilerInstance HipCompiler::read(const std::string &relPath) const {
+  HipCompilerInstance inst;
+  inst.m_compiler = this;
+  inst.m_path = relPath;
+  inst.m_source = readFile(m_kernelDir + "/" + relPath);
+  return inst;
+}
+
+std::string HipCompilerInstance::defineString() const {
+  std::string s;
+  for (const auto &[k, v] : m_defines) {
+    if (!s.empty()) s += ' ';
+    s += k + "=" + v;
+  }
+  return s;
+}
+
+std::string HipCompilerInstance::sha256() const {
+  Sha256 h;
+  h.update(m_source);
+  h.update(std::string("\n//headers\n"));
+  h.update(m_compiler->m_headerDigest);
+  h.update(std::string("\n//defines\n"));
+  h.update(defineString());
+  h.update(std::string("\n//flags\n"));
+  for (const char *f : kFlags) h.update(std::string(f) + " ");
+  h.update(m_compiler->m_arch);
+  return Sha256::hex(h.digest());
+}
+
+std::vector<uint8_t> HipCompilerInstance::compile() const {
+  const std::string key = sha256();
+  const std::string cachePath = m_compiler->m_cacheDir.empty() ? "" : m_compiler->m_cacheDir + "/" + key + ".hsaco";
+  if (!cachePath.empty()) {
+    std::ifstream f(cachePath, std::ios::binary);
+    if (f) {
+      std::vector<uint8_t> code((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+      if (!code.empty()) {
+        ++m_compiler->m_stats.cacheHits;
+        return code;
+      }
+    }
+  }
+  hiprtcProgram prog;
+  if (hiprtcCreateProgram(&prog, m_source.c_str(), m_path.c_str(), 0, nullptr, nullptr) != HIPRTC_SUCCESS)
+    fail(Status::HipError, "hiprtcCreateProgram failed for " + m_path);
+  std::vector<std::string> opts;
+  opts.push_back("--offload-arch=" + m_compiler->m_arch);
+  for (const char *f : kFlags) opts.push_back(f);
+  opts.push_back("-I" + m_compiler->m_kernelDir);
+  for (const auto &[k, v] : m_defines) opts.push_back("-D" + k + "=" + v);
+  std::vector<const char *> copts;
+  for (const auto &o : opts) copts.push_back(o.c_str());
+  const hiprtcResult rc = hiprtcCompileProgram(prog, static_cast<int>(copts.size()), copts.data());
+  if (rc != HIPRTC_SUCCESS) {
+    size_t n = 0;
+    hiprtcGetProgramLogSize(prog, &n);
+    std::string log(n, '\0');
+    if (n) hiprtcGetProgramLog(prog, log.data());
+    hiprtcDestroyProgram(&prog);
+    fail(Status::CompileError, "hiprtc failed for " + m_path + " [" + defineString() + "]: " + hiprtcGetErrorString(rc) + "\n" + log);
+  }
+  size_t size = 0;
+  hiprtcGetCodeSize(prog, &size);
+  std::vector<uint8_t> code(size);
+  hiprtcGetCode(prog, reinterpret_cast<char *>(code.data()));
+  hiprtcDestroyProgram(&prog);
+  ++m_compiler->m_stats.compiled;
+  if (!cachePath.empty()) { // temp file + rename: concurrent compilers never see a partial file
+    const std::string tmp = cachePath + ".tmp." + std::to_string(getpid());
+    std::ofstream f(tmp, std::ios::binary);
+    if (f) {
+      f.write(reinterpret_cast<const char *>(code.data()), static_cast<std::streamsize>(code.size()));
+      f.close();
+      if (f && std::rename(tmp.c_str(), cachePath.c_str()) != 0) std::remove(tmp.c_str());
+    }
+  }
+  return code;
+}
+
+} // namespace denox::hip

@@ -1,0 +1,33 @@
+// activation.hip -- stand-alone elementwise activation in binary16.
+// Replaces compiler/src/denox/compiler/implement/shaders/activation/basic_activation.comp:26-184:
+//   ReLU: max(v, 0);  LeakyReLU: max(v, alpha * v) with alpha and the product in binary16.
+// Definitions: CH, ACT (1 ReLU, 2 LeakyReLU), ALPHA, VEC.
+#include "common.h"
+#ifndef ALPHA
+#define ALPHA 0.0f
+#endif
+struct PushConstants { unsigned int W, H; };
+__device__ DNX_INLINE _Float16 act1(_Float16 v) {
+#if ACT == 1
+  return v > (_Float16)0.0f ? v : (_Float16)0.0f;
+#else
+  const _Float16 av = (_Float16)(ALPHA) * v;
+  return v > av ? v : av;
+#endif
+}
+extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void activation(
+    const ushort_t *__restrict__ IN, ushort_t *__restrict__ OUT, PushConstants pc) {
+  constexpr unsigned CV = CH / VEC;
+  const unsigned long long idx = (unsigned long long)DNX_BID_X * WG + DNX_TID;
+  const unsigned long long total = (unsigned long long)pc.W * pc.H * CV;
+  if (idx >= total) return;
+  const vec_t v = ldv(IN + idx * VEC);
+#if VEC == 8
+  half8 a = __builtin_bit_cast(half8, v);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) a[e] = act1(a[e]);
+  stv(OUT + idx * VEC, __builtin_bit_cast(uint4v, a));
+#else
+  stv(OUT + idx * VEC, __builtin_bit_cast(ushort_t, act1(__builtin_bit_cast(_Float16, v))));
+#endif
+}

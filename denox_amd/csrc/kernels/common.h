@@ -1,0 +1,34 @@
+#include "prelude.h"
+// Shared helpers for the bandwidth kernels.  Every kernel processes VEC
+// channels per thread: VEC = 8 (one 16-byte access) when all channel counts and
+// offsets involved are multiples of 8, else VEC = 1 (2-byte accesses).
+typedef unsigned short ushort_t;
+typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+
+#ifndef WG
+#define WG 256
+#endif
+
+#if VEC == 8
+typedef uint4v vec_t;
+#elif VEC == 1
+typedef ushort_t vec_t;
+#else
+#error "VEC must be 1 or 8"
+#endif
+
+__device__ DNX_INLINE vec_t ldv(const ushort_t *p) {
+  return *reinterpret_cast<const vec_t *>(p);
+}
+__device__ DNX_INLINE void stv(ushort_t *p, vec_t v) {
+  *reinterpret_cast<vec_t *>(p) = v;
+}
+
+// binary16 "replace only when strictly greater", the order-dependent max the
+// pool uses; +0 and -0 compare equal so the earlier value is kept.
+__device__ DNX_INLINE ushort_t max_keep_first(ushort_t acc, ushort_t v) {
+  const _Float16 a = __builtin_bit_cast(_Float16, acc);
+  const _Float16 b = __builtin_bit_cast(_Float16, v);
+  return b > a ? v : acc;
+}

@@ -1,0 +1,110 @@
+#include "db_bench.hpp"
+#include <cstring>
+#include <sstream>
+
+namespace denox::runtime {
+
+static bool converged(const DbDispatch &d, const DbBenchOptions &opt) {
+  return d.samples >= opt.minSamples && d.relativeError() <= opt.maxRelativeError;
+}
+
+DbBenchResult db_bench(Db &db, const ContextHandle &ctx, const hip::HipCompiler &hipc, const DbBenchOptions &opt) {
+  DbBenchResult res;
+  ctx->makeCurrent();
+  hipStream_t s = ctx->stream();
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  hipCheck(hipEventCreate(&e0), "hipEventCreate");
+  hipCheck(hipEventCreate(&e1), "hipEventCreate");
+  void *scratch = nullptr;
+  uint64_t scratchBytes = 0;
+  size_t sinceWriteback = 0;
+  auto cleanup = [&]() {
+    if (scratch) (void)hipFree(scratch);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+  };
+  try {
+    for (size_t r = 0; r < db.rows().size(); ++r) {
+      DbDispatch &row = db.rows()[r];
+      if (!opt.filter.empty() && row.shader.find(opt.filter) == std::string::npos && row.operation.find(opt.filter) == std::string::npos) { ++res.skipped; continue; }
+      if (converged(row, opt)) { ++res.skipped; continue; }
+      // rebuild the kernel variant from its source path and definitions
+      hip::HipCompilerInstance k = hipc.read(row.srcPath);
+      std::stringstream ss(row.defines);
+      std::string kv;
+      while (ss >> kv) {
+        const size_t eq = kv.find('=');
+        if (eq == std::string::npos) fail(Status::IoError, "db: malformed definition '" + kv + "'");
+        k.define(kv.substr(0, eq), kv.substr(eq + 1));
+      }
+      if (k.sha256() != row.sha256) { ++res.failed; continue; } // kernel source changed since the row was made
+      const std::vector<uint8_t> code = k.compile();
+      hipModule_t mod = nullptr;
+      hipCheck(hipModuleLoadData(&mod, code.data()), "hipModuleLoadData");
+      try {
+        hipFunction_t fn = nullptr;
+        hipCheck(hipModuleGetFunction(&fn, mod, row.entryPoint.c_str()), "hipModuleGetFunction");
+        // pack the bindings into one scratch allocation
+        uint64_t need = 0;
+        std::vector<uint64_t> offs;
+        for (const auto &b : row.bindings) {
+          const uint64_t al = std::max<uint64_t>(b.alignment, 256);
+          need = (need + al - 1) / al * al;
+          offs.push_back(need);
+          need += b.byteSize + 256;
+        }
+        if (need > scratchBytes) {
+          if (scratch) hipCheck(hipFree(scratch), "hipFree");
+          scratch = nullptr;
+          hipCheck(hipMalloc(&scratch, need), "hipMalloc(scratch)");
+          scratchBytes = need;
+          // zeros are as good as any contents and keep fp16 arithmetic away from NaN slow paths
+          hipCheck(hipMemsetAsync(scratch, 0, need, s), "hipMemsetAsync");
+        }
+        std::vector<uint8_t> args(row.bindings.size() * sizeof(void *));
+        for (size_t i = 0; i < offs.size(); ++i) {
+          void *p = static_cast<uint8_t *>(scratch) + offs[i];
+          std::memcpy(args.data() + i * sizeof(void *), &p, sizeof(void *));
+        }
+        const size_t pcAlign = 4; // every push constant emitted is 32 bit
+        while (args.size() % pcAlign) args.push_back(0);
+        args.insert(args.end(), row.pushConstants.begin(), row.pushConstants.end());
+        size_t argSize = args.size();
+        void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, args.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &argSize, HIP_LAUNCH_PARAM_END};
+        auto launch = [&]() {
+          hipCheck(hipModuleLaunchKernel(fn, row.wg[0], row.wg[1], row.wg[2], row.block[0], row.block[1], row.block[2], 0, s, nullptr, config), "hipModuleLaunchKernel");
+        };
+        if (row.wg[0] == 0 || row.wg[1] == 0 || row.wg[2] == 0) { ++res.skipped; (void)hipModuleUnload(mod); continue; }
+        for (uint32_t i = 0; i < opt.warmup; ++i) launch();
+        hipCheck(hipStreamSynchronize(s), "hipStreamSynchronize");
+        uint32_t taken = 0;
+        while (!converged(row, opt) && taken < opt.maxSamples) {
+          for (uint32_t i = 0; i < opt.batch; ++i, ++taken) {
+            hipCheck(hipEventRecord(e0, s), "hipEventRecord");
+            launch();
+            hipCheck(hipEventRecord(e1, s), "hipEventRecord");
+            hipCheck(hipEventSynchronize(e1), "hipEventSynchronize");
+            float ms = 0.0f;
+            hipCheck(hipEventElapsedTime(&ms, e0, e1), "hipEventElapsedTime");
+            db.add_dispatch_benchmark_result(r, static_cast<double>(ms) * 1e6);
+          }
+        }
+        ++res.benchmarked;
+        if (converged(row, opt)) ++res.converged;
+      } catch (...) {
+        (void)hipModuleUnload(mod);
+        throw;
+      }
+      hipCheck(hipModuleUnload(mod), "hipModuleUnload");
+      if (opt.saveProgress && ++sinceWriteback >= opt.epochSize) { db.atomic_writeback(); sinceWriteback = 0; }
+    }
+    if (opt.saveProgress && !db.path().empty()) db.atomic_writeback();
+  } catch (...) {
+    cleanup();
+    throw;
+  }
+  cleanup();
+  return res;
+}
+
+} // namespace denox::runtime

@@ -1,0 +1,342 @@
+#include "runtime.hpp"
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+
+namespace denox::runtime {
+
+void hipCheck(hipError_t e, const char *what) {
+  if (e != hipSuccess) fail(Status::HipError, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+// ---------------------------------------------------------------- Context
+Context::Context(int device) : m_device(device) {
+  int n = 0;
+  hipCheck(hipGetDeviceCount(&n), "hipGetDeviceCount");
+  if (device < 0 || device >= n) fail(Status::InvalidArgument, "no HIP device with index " + std::to_string(device));
+  hipCheck(hipSetDevice(device), "hipSetDevice");
+  hipCheck(hipGetDeviceProperties(&m_props, device), "hipGetDeviceProperties");
+  // default priority, non-blocking with respect to the null stream
+  hipCheck(hipStreamCreateWithFlags(&m_stream, hipStreamNonBlocking), "hipStreamCreateWithFlags");
+}
+
+Context::~Context() {
+  if (m_stream) (void)hipStreamDestroy(m_stream);
+}
+
+void Context::makeCurrent() const { hipCheck(hipSetDevice(m_device), "hipSetDevice"); }
+
+// ---------------------------------------------------------------- Model
+Model::Model(ContextHandle ctx, const void *dnxbuf, size_t size) : m_ctx(std::move(ctx)), m_dnx(dnx::deserialize(dnxbuf, size)) {
+  m_ctx->makeCurrent();
+  m_modules.resize(m_dnx.shader_binaries.size(), nullptr);
+  try {
+    for (size_t i = 0; i < m_modules.size(); ++i) {
+      if (m_dnx.shader_binaries[i].code_object.empty()) fail(Status::InvalidModel, "empty shader binary");
+      hipCheck(hipModuleLoadData(&m_modules[i], m_dnx.shader_binaries[i].code_object.data()), "hipModuleLoadData");
+    }
+    m_dispatches.reserve(m_dnx.dispatches.size());
+    for (const auto &d : m_dnx.dispatches) {
+      ModelDispatch md;
+      md.dnx = &d;
+      hipCheck(hipModuleGetFunction(&md.function, m_modules[d.binary_id], d.entry_point.c_str()), "hipModuleGetFunction");
+      // kernel arguments follow (set, binding) order
+      std::vector<const dnx::DescriptorSetBinding *> sets;
+      for (const auto &s : d.bindings) sets.push_back(&s);
+      std::sort(sets.begin(), sets.end(), [](auto *a, auto *b) { return a->set < b->set; });
+      for (const auto *s : sets) {
+        std::vector<dnx::DescriptorBinding> bs = s->bindings;
+        std::sort(bs.begin(), bs.end(), [](const auto &a, const auto &b) { return a.binding < b.binding; });
+        for (const auto &b : bs) md.tensors.emplace_back(b.tensor, b.access);
+      }
+      // On one in-order stream program order resolves every RAW/WAW/WAR hazard the
+      // reference inserts barriers for; what remains to check is that no single
+      // dispatch reads a tensor through one binding and writes it through another.
+      for (size_t a = 0; a < md.tensors.size(); ++a)
+        for (size_t b = a + 1; b < md.tensors.size(); ++b)
+          if (md.tensors[a].first == md.tensors[b].first &&
+              (md.tensors[a].second != dnx::Access::ReadOnly || md.tensors[b].second != dnx::Access::ReadOnly))
+            fail(Status::InvalidModel, "dispatch '" + d.info.name + "' binds a tensor it writes more than once");
+      m_dispatches.push_back(std::move(md));
+    }
+  } catch (...) {
+    for (auto m : m_modules) if (m) (void)hipModuleUnload(m);
+    throw;
+  }
+}
+
+Model::~Model() {
+  for (auto m : m_modules) if (m) (void)hipModuleUnload(m);
+}
+
+// ---------------------------------------------------------------- Instance
+static void putScalar(std::vector<uint8_t> &buf, size_t off, dnx::ScalarType t, int64_t v) {
+  switch (t) {
+  case dnx::ScalarType::I16: { int16_t x = static_cast<int16_t>(v); std::memcpy(buf.data() + off, &x, 2); break; }
+  case dnx::ScalarType::U16: { uint16_t x = static_cast<uint16_t>(v); std::memcpy(buf.data() + off, &x, 2); break; }
+  case dnx::ScalarType::I32: { int32_t x = static_cast<int32_t>(v); std::memcpy(buf.data() + off, &x, 4); break; }
+  case dnx::ScalarType::U32: { uint32_t x = static_cast<uint32_t>(v); std::memcpy(buf.data() + off, &x, 4); break; }
+  case dnx::ScalarType::I64: std::memcpy(buf.data() + off, &v, 8); break;
+  case dnx::ScalarType::U64: { uint64_t x = static_cast<uint64_t>(v); std::memcpy(buf.data() + off, &x, 8); break; }
+  default: fail(Status::Unsupported, "floating-point push constants are not supported"); // instance.cpp:196-199 of the reference
+  }
+}
+
+Instance::Instance(ModelHandle model, const std::vector<ValueSpec> &specs) : m_model(std::move(model)) {
+  const dnx::Model &m = m_model->dnx();
+  m_model->context()->makeCurrent();
+  // name -> variable, unknown names are ignored (instance.cpp:308-318 of the reference)
+  std::vector<int64_t> vars(m.sym_ir.varCount, 0);
+  std::vector<bool> set(m.sym_ir.varCount, false);
+  for (const auto &spec : specs)
+    for (const auto &vn : m.value_names)
+      if (vn.name == spec.name && vn.value.symbolic && vn.value.value >= 0 && static_cast<uint64_t>(vn.value.value) < vars.size()) {
+        vars[static_cast<size_t>(vn.value.value)] = spec.value;
+        set[static_cast<size_t>(vn.value.value)] = true;
+      }
+  // every named variable needs a value (unnamed table slots are unused)
+  for (const auto &vn : m.value_names)
+    if (vn.value.symbolic && vn.value.value >= 0 && static_cast<uint64_t>(vn.value.value) < vars.size() && !set[static_cast<size_t>(vn.value.value)])
+      fail(Status::InvalidArgument, "no value given for dynamic extent '" + vn.name + "'");
+  m_sym = m.sym_ir.eval(vars);
+
+  // tensors must fit their buffers
+  m_bufferSizes.resize(m.buffers.size());
+  for (size_t i = 0; i < m.buffers.size(); ++i) {
+    const int64_t sz = m.buffers[i].size.eval(m_sym);
+    if (sz < 0 || sz > (int64_t(1) << 40)) fail(Status::InvalidArgument, "buffer " + std::to_string(i) + " evaluates to an unusable size (" + std::to_string(sz) + " bytes)");
+    m_bufferSizes[i] = static_cast<uint64_t>(sz);
+  }
+  for (const auto &t : m.tensors) {
+    const int64_t off = t.offset.eval(m_sym), sz = t.size.eval(m_sym);
+    if (off < 0 || sz < 0 || static_cast<uint64_t>(off) + static_cast<uint64_t>(sz) > m_bufferSizes[t.buffer])
+      fail(Status::InvalidModel, "tensor '" + t.info.name + "' does not fit its buffer");
+  }
+  try {
+    m_buffers.assign(m.buffers.size(), nullptr);
+    for (size_t i = 0; i < m.buffers.size(); ++i) {
+      // slack so that 16-byte vector accesses at the very end of a tensor stay inside the allocation
+      const uint64_t bytes = std::max<uint64_t>(m_bufferSizes[i], 16) + 256;
+      hipCheck(hipMalloc(&m_buffers[i], bytes), "hipMalloc");
+      m_deviceBytes += bytes;
+    }
+    // parameters (instance.cpp:65-113 of the reference)
+    hipStream_t s = m_model->context()->stream();
+    for (const auto &init : m.initializers) {
+      const auto &t = m.tensors[init.tensor];
+      const uint64_t sz = static_cast<uint64_t>(t.size.eval(m_sym));
+      if (init.data.size() > sz) fail(Status::InvalidModel, "initializer larger than its tensor");
+      hipCheck(hipMemcpyAsync(tensorPtr(init.tensor), init.data.data(), init.data.size(), hipMemcpyHostToDevice, s), "hipMemcpyAsync(initializer)");
+    }
+    hipCheck(hipStreamSynchronize(s), "hipStreamSynchronize");
+
+    // launches (instance.cpp:121-229 of the reference)
+    for (const auto &md : m_model->dispatches()) {
+      const dnx::ComputeDispatch &d = *md.dnx;
+      Launch l;
+      l.fn = md.function;
+      const int64_t g[3] = {d.workgroup_count_x.eval(m_sym), d.workgroup_count_y.eval(m_sym), d.workgroup_count_z.eval(m_sym)};
+      for (int i = 0; i < 3; ++i) {
+        if (g[i] < 0 || g[i] > 0x7FFFFFFF) fail(Status::InvalidArgument, "dispatch '" + d.info.name + "' workgroup count out of range");
+        l.grid[i] = static_cast<unsigned>(g[i]);
+        l.block[i] = d.workgroup_size[i];
+      }
+      const size_t ptrBytes = md.tensors.size() * sizeof(void *);
+      // push constants start at the next multiple of their strictest field alignment (at most 8)
+      size_t pcAlign = 4;
+      for (const auto &f : d.push_constant.fields) pcAlign = std::max(pcAlign, dnx::scalarSize(f.dtype));
+      const size_t pcOff = (ptrBytes + pcAlign - 1) / pcAlign * pcAlign;
+      l.args.assign(pcOff + d.push_constant.size, 0);
+      for (size_t i = 0; i < md.tensors.size(); ++i) {
+        void *p = tensorPtr(md.tensors[i].first);
+        std::memcpy(l.args.data() + i * sizeof(void *), &p, sizeof(void *));
+        l.ptrSlots.emplace_back(i * sizeof(void *), md.tensors[i].first);
+      }
+      for (const auto &f : d.push_constant.fields) putScalar(l.args, pcOff + f.offset, f.dtype, f.source.eval(m_sym));
+      m_launches.push_back(std::move(l));
+    }
+    m_boundInputs.assign(m.inputs.size(), nullptr);
+    m_boundOutputs.assign(m.outputs.size(), nullptr);
+    if (!std::getenv("DENOX_HIP_NO_GRAPH")) buildGraph();
+  } catch (...) {
+    for (void *b : m_buffers) if (b) (void)hipFree(b);
+    if (m_graphExec) (void)hipGraphExecDestroy(m_graphExec);
+    if (m_graph) (void)hipGraphDestroy(m_graph);
+    throw;
+  }
+}
+
+Instance::~Instance() {
+  if (m_model) {
+    (void)hipSetDevice(m_model->context()->device());
+    (void)hipStreamSynchronize(m_model->context()->stream());
+  }
+  if (m_graphExec) (void)hipGraphExecDestroy(m_graphExec);
+  if (m_graph) (void)hipGraphDestroy(m_graph);
+  for (void *b : m_buffers) if (b) (void)hipFree(b);
+}
+
+void *Instance::tensorPtr(uint32_t tensor) const {
+  const auto &t = m_model->dnx().tensors.at(tensor);
+  return static_cast<uint8_t *>(m_buffers[t.buffer]) + t.offset.eval(m_sym);
+}
+
+TensorDesc Instance::describe(uint32_t tensor) const {
+  const auto &t = m_model->dnx().tensors.at(tensor);
+  TensorDesc d;
+  if (t.info.has_extent) {
+    d.width = t.info.width.eval(m_sym);
+    d.height = t.info.height.eval(m_sym);
+    d.channels = t.info.channels.eval(m_sym);
+  }
+  d.format = t.info.format;
+  d.dtype = t.info.type;
+  d.byteSize = static_cast<uint64_t>(t.size.eval(m_sym));
+  d.name = t.info.name;
+  return d;
+}
+
+static void launchOne(hipFunction_t fn, const unsigned grid[3], const unsigned block[3], std::vector<uint8_t> &args, hipStream_t s) {
+  if (grid[0] == 0 || grid[1] == 0 || grid[2] == 0) return; // empty extent: nothing to do
+  size_t size = args.size();
+  void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, args.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+  hipCheck(hipModuleLaunchKernel(fn, grid[0], grid[1], grid[2], block[0], block[1], block[2], 0, s, nullptr, config), "hipModuleLaunchKernel");
+}
+
+void Instance::launchAll(hipStream_t s) {
+  for (auto &l : m_launches) launchOne(l.fn, l.grid, l.block, l.args, s);
+}
+
+void Instance::buildGraph() {
+  // Whole-network capture: one graph launch per frame instead of one driver
+  // call per dispatch.
+  hipStream_t s = m_model->context()->stream();
+  hipCheck(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
+  try {
+    launchAll(s);
+  } catch (...) {
+    hipGraph_t g = nullptr;
+    (void)hipStreamEndCapture(s, &g);
+    if (g) (void)hipGraphDestroy(g);
+    throw;
+  }
+  hipCheck(hipStreamEndCapture(s, &m_graph), "hipStreamEndCapture");
+  hipCheck(hipGraphInstantiate(&m_graphExec, m_graph, nullptr, nullptr, 0), "hipGraphInstantiate");
+}
+
+void Instance::rebind(const void *const *inputs, void *const *outputs) {
+  // Patch external input/output addresses into the argument buffers.  The graph
+  // is rebuilt only when an address differs from the last call's.
+  const dnx::Model &m = m_model->dnx();
+  bool changed = false;
+  std::vector<std::pair<uint32_t, void *>> over; // tensor -> address
+  for (size_t i = 0; i < m.inputs.size(); ++i) {
+    void *p = inputs ? const_cast<void *>(inputs[i]) : nullptr;
+    if (p != m_boundInputs[i]) { changed = true; m_boundInputs[i] = p; }
+    over.emplace_back(m.inputs[i], p ? p : tensorPtr(m.inputs[i]));
+  }
+  for (size_t i = 0; i < m.outputs.size(); ++i) {
+    void *p = outputs ? outputs[i] : nullptr;
+    if (p != m_boundOutputs[i]) { changed = true; m_boundOutputs[i] = p; }
+    over.emplace_back(m.outputs[i], p ? p : tensorPtr(m.outputs[i]));
+  }
+  if (!changed) return;
+  for (auto &l : m_launches)
+    for (const auto &[off, tensor] : l.ptrSlots)
+      for (const auto &[t, p] : over)
+        if (t == tensor) std::memcpy(l.args.data() + off, &p, sizeof(void *));
+  if (m_graphExec) {
+    (void)hipGraphExecDestroy(m_graphExec);
+    (void)hipGraphDestroy(m_graph);
+    m_graphExec = nullptr;
+    m_graph = nullptr;
+    buildGraph();
+  }
+}
+
+void Instance::inferDevice(const void *const *inputs, void *const *outputs) {
+  m_model->context()->makeCurrent();
+  rebind(inputs, outputs);
+  hipStream_t s = m_model->context()->stream();
+  if (m_graphExec)
+    hipCheck(hipGraphLaunch(m_graphExec, s), "hipGraphLaunch");
+  else
+    launchAll(s);
+}
+
+void Instance::synchronize() {
+  m_model->context()->makeCurrent();
+  hipCheck(hipStreamSynchronize(m_model->context()->stream()), "hipStreamSynchronize");
+}
+
+void Instance::infer(const void *const *inputs, void *const *outputs) {
+  const dnx::Model &m = m_model->dnx();
+  if (!inputs || !outputs) fail(Status::InvalidArgument, "infer: null pointer array");
+  m_model->context()->makeCurrent();
+  hipStream_t s = m_model->context()->stream();
+  for (size_t i = 0; i < m.inputs.size(); ++i) {
+    if (!inputs[i]) fail(Status::InvalidArgument, "infer: null input pointer");
+    const uint64_t sz = static_cast<uint64_t>(m.tensors[m.inputs[i]].size.eval(m_sym));
+    hipCheck(hipMemcpyAsync(tensorPtr(m.inputs[i]), inputs[i], sz, hipMemcpyHostToDevice, s), "hipMemcpyAsync(input)");
+  }
+  inferDevice(nullptr, nullptr);
+  for (size_t i = 0; i < m.outputs.size(); ++i) {
+    if (!outputs[i]) fail(Status::InvalidArgument, "infer: null output pointer");
+    const uint64_t sz = static_cast<uint64_t>(m.tensors[m.outputs[i]].size.eval(m_sym));
+    hipCheck(hipMemcpyAsync(outputs[i], tensorPtr(m.outputs[i]), sz, hipMemcpyDeviceToHost, s), "hipMemcpyAsync(output)");
+  }
+  hipCheck(hipStreamSynchronize(s), "hipStreamSynchronize");
+}
+
+std::vector<DispatchTiming> Instance::bench(int warmup) {
+  const dnx::Model &m = m_model->dnx();
+  m_model->context()->makeCurrent();
+  rebind(nullptr, nullptr);
+  hipStream_t s = m_model->context()->stream();
+  for (int i = 0; i < warmup; ++i) {
+    if (m_graphExec) hipCheck(hipGraphLaunch(m_graphExec, s), "hipGraphLaunch");
+    else launchAll(s);
+  }
+  hipCheck(hipStreamSynchronize(s), "hipStreamSynchronize");
+  std::vector<hipEvent_t> ev(m_launches.size() + 1, nullptr);
+  std::vector<DispatchTiming> out;
+  try {
+    for (auto &e : ev) hipCheck(hipEventCreate(&e), "hipEventCreate");
+    hipCheck(hipEventRecord(ev[0], s), "hipEventRecord");
+    for (size_t i = 0; i < m_launches.size(); ++i) {
+      auto &l = m_launches[i];
+      launchOne(l.fn, l.grid, l.block, l.args, s);
+      hipCheck(hipEventRecord(ev[i + 1], s), "hipEventRecord");
+    }
+    hipCheck(hipStreamSynchronize(s), "hipStreamSynchronize");
+    auto fmt = [&](uint32_t t) {
+      const auto &ti = m.tensors[t].info;
+      const char *f = ti.format == dnx::TensorFormat::SSBO_HWC ? "HWC" : ti.format == dnx::TensorFormat::SSBO_CHW ? "CHW" : ti.format == dnx::TensorFormat::SSBO_CHWC8 ? "CHWC8" : "?";
+      return std::string(f) + "[" + (ti.has_extent ? std::to_string(ti.channels.eval(m_sym)) : std::string("-")) + "]";
+    };
+    for (size_t i = 0; i < m_launches.size(); ++i) {
+      const auto &md = m_model->dispatches()[i];
+      const auto &d = *md.dnx;
+      DispatchTiming t;
+      t.name = d.info.name;
+      for (const auto &[tensor, access] : md.tensors) {
+        const bool param = std::any_of(m.initializers.begin(), m.initializers.end(), [&](const auto &in) { return in.tensor == tensor; });
+        if (param) continue;
+        if (access == dnx::Access::ReadOnly) t.input += (t.input.empty() ? "" : "+") + fmt(tensor);
+        else t.output += (t.output.empty() ? "" : "+") + fmt(tensor);
+      }
+      if (d.info.has_reads) t.memoryReads = static_cast<uint64_t>(d.info.memory_reads.eval(m_sym));
+      if (d.info.has_writes) t.memoryWrites = static_cast<uint64_t>(d.info.memory_writes.eval(m_sym));
+      if (d.info.has_flops) t.flops = static_cast<uint64_t>(d.info.flops.eval(m_sym));
+      hipCheck(hipEventElapsedTime(&t.latencyMs, ev[i], ev[i + 1]), "hipEventElapsedTime");
+      out.push_back(std::move(t));
+    }
+  } catch (...) {
+    for (auto e : ev) if (e) (void)hipEventDestroy(e);
+    throw;
+  }
+  for (auto e : ev) if (e) (void)hipEventDestroy(e);
+  return out;
+}
+
+} // namespace denox::runtime

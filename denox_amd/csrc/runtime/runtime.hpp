@@ -1,0 +1,135 @@
+// Run-time half of the backend: load a compiled model, bind it to concrete
+// image extents, execute it on one HIP stream.
+//
+// Same object model as the reference runtime --
+//   Context  : runtime/src/denox/runtime/context.hpp:113-252 (device + queue)
+//   Model    : runtime/src/denox/runtime/model.hpp:107-170, model.cpp:80-239,637-659
+//   Instance : runtime/src/denox/runtime/instance.hpp:44-63, instance.cpp:25-430
+// -- with Vulkan replaced by the HIP module API: one hipModule_t per shader
+// binary, one hipFunction_t per dispatch, kernel arguments = bound tensor
+// addresses in (set, binding) order followed by the push-constant bytes, all
+// launches in program order on a single stream (which makes the reference's
+// barrier insertion, model.cpp:247-340, unnecessary), and the whole dispatch
+// list captured once per Instance into a hipGraph.
+#pragma once
+#include "../common/dnx.hpp"
+#include <hip/hip_runtime_api.h>
+#include <memory>
+#include <string>
+#include <vector>
+
+namespace denox::runtime {
+
+void hipCheck(hipError_t e, const char *what);
+
+class Context {
+public:
+  explicit Context(int device);
+  ~Context();
+  Context(const Context &) = delete;
+  Context &operator=(const Context &) = delete;
+  int device() const { return m_device; }
+  hipStream_t stream() const { return m_stream; }
+  void makeCurrent() const;
+  const hipDeviceProp_t &props() const { return m_props; }
+
+private:
+  int m_device;
+  hipStream_t m_stream = nullptr;
+  hipDeviceProp_t m_props;
+};
+using ContextHandle = std::shared_ptr<Context>;
+
+struct ModelDispatch {
+  const dnx::ComputeDispatch *dnx = nullptr;
+  hipFunction_t function = nullptr;
+  std::vector<std::pair<uint32_t, dnx::Access>> tensors; // flattened in (set, binding) order
+};
+
+class Model {
+public:
+  Model(ContextHandle ctx, const void *dnxbuf, size_t size);
+  ~Model();
+  Model(const Model &) = delete;
+  Model &operator=(const Model &) = delete;
+  const ContextHandle &context() const { return m_ctx; }
+  const dnx::Model &dnx() const { return m_dnx; }
+  const std::vector<ModelDispatch> &dispatches() const { return m_dispatches; }
+
+private:
+  ContextHandle m_ctx;
+  dnx::Model m_dnx;
+  std::vector<hipModule_t> m_modules;
+  std::vector<ModelDispatch> m_dispatches;
+};
+using ModelHandle = std::shared_ptr<Model>;
+
+struct ValueSpec { std::string name; int64_t value; };
+
+struct TensorDesc {
+  int64_t width = 0, height = 0, channels = 0;
+  dnx::TensorFormat format = dnx::TensorFormat::UNKNOWN;
+  dnx::ScalarType dtype = dnx::ScalarType::F16;
+  uint64_t byteSize = 0;
+  std::string name;
+};
+
+struct DispatchTiming {
+  std::string name, input, output;
+  uint64_t memoryReads = 0, memoryWrites = 0, flops = 0;
+  float latencyMs = 0.0f;
+};
+
+class Instance {
+public:
+  Instance(ModelHandle model, const std::vector<ValueSpec> &specs);
+  ~Instance();
+  Instance(const Instance &) = delete;
+  Instance &operator=(const Instance &) = delete;
+
+  // Host pointers, arrays in model input / output order, tightly packed in the
+  // tensor's declared format; blocking (instance.cpp:322-430 of the reference).
+  void infer(const void *const *inputs, void *const *outputs);
+  // Device pointers (inputs already resident in HBM); enqueues on the context's
+  // stream and returns without synchronising.  A null entry means "use the
+  // instance's own buffer for that tensor" (see inputDevicePtr/outputDevicePtr).
+  void inferDevice(const void *const *inputs, void *const *outputs);
+  void synchronize();
+  // Per-dispatch timings with hipEvents after warm-up passes (instance.cpp:432-654).
+  std::vector<DispatchTiming> bench(int warmup);
+
+  size_t inputCount() const { return m_model->dnx().inputs.size(); }
+  size_t outputCount() const { return m_model->dnx().outputs.size(); }
+  TensorDesc inputDesc(size_t i) const { return describe(m_model->dnx().inputs.at(i)); }
+  TensorDesc outputDesc(size_t i) const { return describe(m_model->dnx().outputs.at(i)); }
+  void *inputDevicePtr(size_t i) const { return tensorPtr(m_model->dnx().inputs.at(i)); }
+  void *outputDevicePtr(size_t i) const { return tensorPtr(m_model->dnx().outputs.at(i)); }
+  uint64_t deviceBytes() const { return m_deviceBytes; }
+  bool usesGraph() const { return m_graphExec != nullptr; }
+
+private:
+  struct Launch {
+    hipFunction_t fn;
+    unsigned grid[3], block[3];
+    std::vector<uint8_t> args;              // pointers then push constants
+    std::vector<std::pair<size_t, uint32_t>> ptrSlots; // (byte offset in args, tensor id)
+    hipGraphNode_t node = nullptr;
+  };
+  TensorDesc describe(uint32_t tensor) const;
+  void *tensorPtr(uint32_t tensor) const;
+  void launchAll(hipStream_t s);
+  void buildGraph();
+  void rebind(const void *const *inputs, void *const *outputs);
+
+  ModelHandle m_model;
+  std::vector<int64_t> m_sym;
+  std::vector<void *> m_buffers;
+  std::vector<uint64_t> m_bufferSizes;
+  std::vector<Launch> m_launches;
+  std::vector<void *> m_boundInputs, m_boundOutputs; // external overrides currently patched in
+  hipGraph_t m_graph = nullptr;
+  hipGraphExec_t m_graphExec = nullptr;
+  uint64_t m_deviceBytes = 0;
+};
+
+} // namespace denox::runtime

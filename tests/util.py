@@ -1,0 +1,34 @@
+"""Helpers shared by the GPU parity tests: seeded tensors and the parity bar."""
+import numpy as np
+
+# north-star tolerance for conv outputs, on the final fp16 output against an fp32 evaluation
+CONV_MAX_ABS = 2e-2
+CONV_MEAN_ABS = 2e-3
+
+
+def he_weights(rng, K, C, R=3, S=3):
+    return (rng.standard_normal((K, C, R, S)) * np.sqrt(2.0 / (R * S * C))).astype(np.float16)
+
+
+def small_bias(rng, K):
+    return (rng.standard_normal(K) * 0.01).astype(np.float16)
+
+
+def assert_conv_close(got_f16, want_f32, what=""):
+    got = np.asarray(got_f16, np.float32)
+    want = np.asarray(want_f32, np.float32)
+    assert got.shape == want.shape, (got.shape, want.shape)
+    assert np.isfinite(got).all(), f"{what}: non-finite output"
+    err = np.abs(got - want)
+    # the bar is absolute on outputs of O(1) magnitude; scale it for layers whose outputs are larger
+    scale = max(1.0, float(np.abs(want).max()))
+    assert err.max() <= CONV_MAX_ABS * scale, f"{what}: max abs err {err.max():.4g} (scale {scale:.3g}) at {np.unravel_index(err.argmax(), err.shape)}"
+    assert err.mean() <= CONV_MEAN_ABS * scale, f"{what}: mean abs err {err.mean():.4g}"
+
+
+def assert_bits_equal(got, want, what=""):
+    g = np.ascontiguousarray(got, np.float16).view(np.uint16)
+    w = np.ascontiguousarray(want, np.float16).view(np.uint16)
+    assert g.shape == w.shape, (g.shape, w.shape)
+    bad = np.argwhere(g != w)
+    assert bad.size == 0, f"{what}: {len(bad)} differing elements, first at {tuple(bad[0])}: got {g[tuple(bad[0])]:#06x} want {w[tuple(bad[0])]:#06x}"
