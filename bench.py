@@ -1,0 +1,156 @@
+#!/usr/bin/env python3
+"""Headline benchmark: OIDN-style 9->3 U-Net, fp16 HWC, 1920x1080, one MI355X.
+
+A "step" is one whole-network inference of one synthetic frame that is already
+resident in HBM (device pointers in, device pointer out), launched through the
+C ABI (denox_hip_instance_infer_device) as one hipGraph on the library's stream.
+
+Prints ONE JSON line: Mpix/s (= 1920*1080 / time per frame) with ms/frame in
+`ms_per_step`, a `roofline` object for the dominant kernel (per-dispatch
+hipEvent timing on the launch stream) and a `cpu_baseline` object (the CPU
+oracle timed on a bounded crop of the same workload).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP16_MFMA_TFLOPS = 2500.0  # MI355X dense fp16, published
+PEAK_HBM_GBPS = 8000.0          # MI355X HBM3E, published
+
+
+def lavapipe_probe() -> str:
+    """The reference's own CPU route (its SPIR-V on Mesa lavapipe) needs a Vulkan loader, the
+    lavapipe ICD and a built denox; report why it is unavailable rather than inventing a number."""
+    import ctypes.util
+    if ctypes.util.find_library("vulkan") is None:
+        return "unavailable (no Vulkan loader on this machine)"
+    if ctypes.util.find_library("vulkan_lvp") is None:
+        return "unavailable (no lavapipe ICD on this machine)"
+    return "unavailable (denox itself cannot be built here: needs glslang, SPIRV-Tools, FlatBuffers)"
+
+
+def cpu_baseline(seed: int, budget_h: int = 272, budget_w: int = 480) -> dict:
+    """CPU oracle (fp32, OpenMP) on a crop of the benchmark frame, same network and weights."""
+    import numpy as np
+    import oracle
+    from denox_amd import networks
+    oracle.build()
+    model, _ = networks.build("oidn_unet", seed=seed)
+    x = networks.synthetic_input("oidn_unet", budget_h, budget_w, seed=seed)
+    ops = model.to_ops({"H": budget_h, "W": budget_w})
+    t0 = time.perf_counter()
+    oracle.run_graph(ops, {"input": x}, "f16")
+    dt = time.perf_counter() - t0
+    return {"value": budget_h * budget_w / dt * 1e-6, "unit": "Mpix/s", "cores": oracle.num_threads(), "kind": "port",
+            "sample": f"one {budget_w}x{budget_h} frame of the same U-Net (1/16 of the 1080p pixels), {dt:.1f} s wall",
+            "lavapipe_baseline": lavapipe_probe()}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--height", type=int, default=1080)
+    ap.add_argument("--width", type=int, default=1920)
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--per-dispatch", action="store_true", help="print the per-dispatch report to stderr")
+    ap.add_argument("--conv-config", default=None)
+    ap.add_argument("--db", default=None, help="timing table to select the schedule with")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path runs on exactly one GPU (independent frames shard trivially across GPUs; "
+              "nothing in this build uses a second one). Run with --gpus 1.", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+    import denox_amd as dx
+    from denox_amd import networks
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+    H, W = args.height, args.width
+    model, _ = networks.build("oidn_unet", seed=args.seed)
+    db = dx.Db(args.db) if args.db else None
+    blob = dx.compile_model(model, assume={"H": H, "W": W}, conv_config=args.conv_config, db=db)
+    mod = dx.Module.load(blob)
+    inst = mod.instance(H=H, W=W)
+
+    x = networks.synthetic_input("oidn_unet", H, W, seed=args.seed)
+    d_in = torch.from_numpy(x).cuda()
+    d_out = torch.empty((H, W, 3), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    ins, outs = [d_in.data_ptr()], [d_out.data_ptr()]
+
+    for _ in range(args.warmup):
+        inst.infer_device(ins, outs)
+    inst.synchronize()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        inst.infer_device(ins, outs)
+    inst.synchronize()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms = dt / args.steps * 1e3
+    out_host = d_out.cpu().numpy()
+    if not np.isfinite(out_host).all():
+        print("bench.py: non-finite output", file=sys.stderr)
+        return 1
+
+    # per-dispatch hipEvent timings on the launch stream, averaged over several passes
+    passes = 5
+    acc = None
+    for _ in range(passes):
+        t = inst.bench(warmup=2)
+        if acc is None:
+            acc = t
+        else:
+            for a, b in zip(acc, t):
+                a["latency_ms"] += b["latency_ms"]
+    for a in acc:
+        a["latency_ms"] /= passes
+        a["GBps"] = (a["memory_reads"] + a["memory_writes"]) / a["latency_ms"] * 1e-6
+        a["TFLOPs"] = a["flops"] / a["latency_ms"] * 1e-9
+    if args.per_dispatch:
+        print(dx.report(acc), file=sys.stderr)
+    dom = max(acc, key=lambda a: a["latency_ms"])
+    conv = [a for a in acc if a["flops"] > 0 and "conv" in a["name"]]
+    conv_ms = sum(a["latency_ms"] for a in conv)
+    conv_flops = sum(a["flops"] for a in conv)
+    other = [a for a in acc if a not in conv]
+    other_ms = sum(a["latency_ms"] for a in other)
+    other_bytes = sum(a["memory_reads"] + a["memory_writes"] for a in other)
+    roofline = {"bound": "mfma", "kernel": dom["name"], "achieved": dom["TFLOPs"], "peak": PEAK_FP16_MFMA_TFLOPS, "unit": "TFLOP/s",
+                "frac": dom["TFLOPs"] / PEAK_FP16_MFMA_TFLOPS, "traffic": None,
+                "kernel_ms": dom["latency_ms"], "kernel_GBps": dom["GBps"],
+                "all_conv_TFLOPs": conv_flops / conv_ms * 1e-9 if conv_ms else None,
+                "all_conv_frac": conv_flops / conv_ms * 1e-9 / PEAK_FP16_MFMA_TFLOPS if conv_ms else None,
+                "non_conv_GBps": other_bytes / other_ms * 1e-6 if other_ms else None,
+                "non_conv_frac_of_hbm": other_bytes / other_ms * 1e-6 / PEAK_HBM_GBPS if other_ms else None,
+                "sum_dispatch_ms": sum(a["latency_ms"] for a in acc)}
+
+    line = {
+        "metric": "oidn_unet_fp16_hwc_1080p_throughput", "value": H * W / (ms * 1e-3) * 1e-6, "unit": "Mpix/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"OIDN-style U-Net 9->3, fp16 HWC, {W}x{H}, replicate-pad to multiple of 16 + crop included, "
+                               f"{mod.runtime_model.dispatch_count} dispatches in one hipGraph", "device_bytes": inst.device_bytes},
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(args.seed)
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
