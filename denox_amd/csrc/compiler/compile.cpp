@@ -1,8 +1,11 @@
 #include "compile.hpp"
 #include <algorithm>
 #include <cstring>
+#include <atomic>
 #include <map>
 #include <set>
+#include <mutex>
+#include <thread>
 
 namespace denox::compiler {
 
@@ -328,7 +331,7 @@ std::vector<uint8_t> compile(const Model &modelIn, const hip::HipCompiler &hipc,
   return dnx::serialize(out);
 }
 
-size_t populate(Db &db, const Model &modelIn, const hip::HipCompiler &hipc, const CompileOptions &opt) {
+size_t populate(Db &db, const Model &modelIn, const hip::HipCompiler &hipc, const CompileOptions &opt, bool compileKernels) {
   Model model = modelIn;
   SymGraph &sym = model.symGraph();
   const auto shaders = get_all_shaders(&hipc);
@@ -359,6 +362,33 @@ size_t populate(Db &db, const Model &modelIn, const hip::HipCompiler &hipc, cons
       db.insert_dispatch(row);
       if (db.rows().size() > before) ++added;
     }
+  if (compileKernels) {
+    // every distinct kernel variant, on all host threads (populate.cpp:70-99 of the reference);
+    // the code objects land in the compiler's cache, where compile() and the benchmark find them
+    std::map<std::string, const hip::HipCompilerInstance *> distinct;
+    for (const auto &edge : g.edges)
+      for (const auto &d : edge.dispatches) distinct.emplace(d.kernel.sha256(), &d.kernel);
+    std::vector<const hip::HipCompilerInstance *> work;
+    for (const auto &kv : distinct) work.push_back(kv.second);
+    std::atomic<size_t> next{0};
+    std::mutex errMutex;
+    std::string firstError;
+    const unsigned nthreads = std::max(1u, std::min<unsigned>(std::thread::hardware_concurrency(), 16u));
+    std::vector<std::thread> pool;
+    for (unsigned t = 0; t < nthreads; ++t)
+      pool.emplace_back([&] {
+        for (size_t i = next++; i < work.size(); i = next++) {
+          try {
+            (void)work[i]->compile();
+          } catch (const std::exception &e) {
+            std::lock_guard<std::mutex> lock(errMutex);
+            if (firstError.empty()) firstError = e.what();
+          }
+        }
+      });
+    for (auto &th : pool) th.join();
+    if (!firstError.empty()) fail(Status::CompileError, firstError);
+  }
   return added;
 }
 

@@ -49,7 +49,7 @@ Db Db::open(const std::string &path) {
     std::stringstream ss(line);
     std::string cell;
     while (std::getline(ss, cell, '\t')) c.push_back(cell);
-    if (c.size() != 22) fail(Status::IoError, "db: malformed row in " + path);
+    if (c.size() != 21) fail(Status::IoError, "db: malformed row in " + path);
     DbDispatch d;
     size_t i = 0;
     d.sha256 = c[i++]; d.pushConstants = unhex(c[i++]);

@@ -100,7 +100,7 @@ std::vector<uint8_t> HipCompilerInstance::compile() const {
     if (f) {
       std::vector<uint8_t> code((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
       if (!code.empty()) {
-        ++m_compiler->m_stats.cacheHits;
+        ++m_compiler->m_cacheHits;
         return code;
       }
     }
@@ -129,7 +129,7 @@ std::vector<uint8_t> HipCompilerInstance::compile() const {
   std::vector<uint8_t> code(size);
   hiprtcGetCode(prog, reinterpret_cast<char *>(code.data()));
   hiprtcDestroyProgram(&prog);
-  ++m_compiler->m_stats.compiled;
+  ++m_compiler->m_compiled;
   if (!cachePath.empty()) { // temp file + rename: concurrent compilers never see a partial file
     const std::string tmp = cachePath + ".tmp." + std::to_string(getpid());
     std::ofstream f(tmp, std::ios::binary);

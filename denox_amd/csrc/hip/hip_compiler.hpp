@@ -7,6 +7,7 @@
 // the SPIR-V cache keyed by source hash in
 //   compiler/src/denox/compiler/compile_shaders/compile_shaders.cpp:35-48,80-83.
 #pragma once
+#include <atomic>
 #include <cstdint>
 #include <map>
 #include <memory>
@@ -49,13 +50,13 @@ public:
   const std::string &arch() const { return m_arch; }
 
   struct Stats { uint64_t compiled = 0, cacheHits = 0; };
-  Stats stats() const { return m_stats; }
+  Stats stats() const { return Stats{m_compiled.load(), m_cacheHits.load()}; }
 
 private:
   friend class HipCompilerInstance;
   std::string m_kernelDir, m_cacheDir, m_arch;
   std::string m_headerDigest; // text of every *.h in the kernel directory
-  mutable Stats m_stats;
+  mutable std::atomic<uint64_t> m_compiled{0}, m_cacheHits{0};
 };
 
 // Directory of the shared library this code is linked into (for default paths).

@@ -99,30 +99,69 @@ load_src8(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B,
   }
 }
 
+// Staging is split in two so that the global loads of the next chunk are in
+// flight while the matrix cores work on the current one: fetch_chunk issues the
+// loads into registers, commit_chunk writes them to LDS after the barrier.
+#define NV_IN ((HALO_PIX * (CK / 8) + NT - 1) / NT)
+#define NV_W ((9 * KT * (CK / 8) + NT - 1) / NT)
+
+struct Staged {
+  uint4v in[NV_IN];
+  uint4v w[NV_W];
+};
+
 template <int L>
 __device__ DNX_INLINE void
-stage_chunk(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B,
-            const _Float16 *__restrict__ wchunk, _Float16 *sIn, _Float16 *sW,
-            int c0, int y0, int x0, unsigned W, unsigned H, int tid) {
+fetch_chunk(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B,
+            const _Float16 *__restrict__ wchunk, Staged &st, int c0, int y0,
+            int x0, unsigned W, unsigned H, int tid) {
   constexpr int VPP = L / 8; // 16-byte vectors per pixel
-  for (int i = tid; i < HALO_PIX * VPP; i += NT) {
-    const int pix = i / VPP;
-    const int v = i - pix * VPP;
-    const int hy = pix / HALO_W;
-    const int hx = pix - hy * HALO_W;
-    const int gy = y0 + hy - 1;
-    const int gx = x0 + hx - 1;
+#pragma unroll
+  for (int it = 0; it < NV_IN; ++it) {
+    const int i = tid + it * NT;
     uint4v val = {0u, 0u, 0u, 0u};
-    if (gy >= 0 && gy < (int)H && gx >= 0 && gx < (int)W)
-      val = load_src8(A, B, gy, gx, c0 + v * 8, W);
-    *reinterpret_cast<uint4v *>(sIn + pix * CKP + v * 8) = val;
+    if (i < HALO_PIX * VPP) {
+      const int pix = i / VPP;
+      const int v = i - pix * VPP;
+      const int hy = pix / HALO_W;
+      const int hx = pix - hy * HALO_W;
+      const int gy = y0 + hy - 1;
+      const int gx = x0 + hx - 1;
+      if (gy >= 0 && gy < (int)H && gx >= 0 && gx < (int)W)
+        val = load_src8(A, B, gy, gx, c0 + v * 8, W);
+    }
+    st.in[it] = val;
   }
-  // weight slice for these channels: global [tap][KT rows][L] -> LDS [tap][KT][CKP]
-  for (int i = tid; i < 9 * KT * VPP; i += NT) {
-    const int row = i / VPP;
-    const int v = i - row * VPP;
-    *reinterpret_cast<uint4v *>(sW + row * CKP + v * 8) =
-        ld16(wchunk + (size_t)row * L + v * 8);
+  // weight slice for these channels: global [tap][KT rows][L]
+#pragma unroll
+  for (int it = 0; it < NV_W; ++it) {
+    const int i = tid + it * NT;
+    if (i < 9 * KT * VPP)
+      st.w[it] = ld16(wchunk + (size_t)i * 8);
+  }
+}
+
+template <int L>
+__device__ DNX_INLINE void commit_chunk(const Staged &st, _Float16 *sIn,
+                                        _Float16 *sW, int tid) {
+  constexpr int VPP = L / 8;
+#pragma unroll
+  for (int it = 0; it < NV_IN; ++it) {
+    const int i = tid + it * NT;
+    if (i < HALO_PIX * VPP) {
+      const int pix = i / VPP;
+      const int v = i - pix * VPP;
+      *reinterpret_cast<uint4v *>(sIn + pix * CKP + v * 8) = st.in[it];
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < NV_W; ++it) {
+    const int i = tid + it * NT;
+    if (i < 9 * KT * VPP) {
+      const int row = i / VPP;
+      const int v = i - row * VPP;
+      *reinterpret_cast<uint4v *>(sW + row * CKP + v * 8) = st.w[it];
+    }
   }
 }
 
@@ -210,18 +249,30 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void conv3x3_mfma(
 
   // packed filter: [kt][chunk][tap][KT][len(chunk)]
   const _Float16 *wbase = FILT + (size_t)kt * 9 * KT * CPAD;
+  Staged st;
+  if (NCHUNK > 1 || TAIL == CK)
+    fetch_chunk<CK>(A, B, wbase, st, 0, y0, x0, W, H, tid);
+  else
+    fetch_chunk<TAIL>(A, B, wbase, st, 0, y0, x0, W, H, tid);
   for (int chunk = 0; chunk < NCHUNK; ++chunk) {
-    const int c0 = chunk * CK;
-    const _Float16 *wchunk = wbase + (size_t)9 * KT * c0;
-    if (TAIL == CK || chunk < NCHUNK - 1) {
-      stage_chunk<CK>(A, B, wchunk, sIn, sW, c0, y0, x0, W, H, tid);
-      DNX_SYNC();
-      mma_chunk<CK>(sIn, sW, acc, wv, lane);
-    } else {
-      stage_chunk<TAIL>(A, B, wchunk, sIn, sW, c0, y0, x0, W, H, tid);
-      DNX_SYNC();
-      mma_chunk<TAIL>(sIn, sW, acc, wv, lane);
+    const bool fullNow = (TAIL == CK) || (chunk < NCHUNK - 1);
+    if (fullNow)
+      commit_chunk<CK>(st, sIn, sW, tid);
+    else
+      commit_chunk<TAIL>(st, sIn, sW, tid);
+    DNX_SYNC();
+    if (chunk + 1 < NCHUNK) { // loads for the next chunk fly during the MFMAs below
+      const int c1 = (chunk + 1) * CK;
+      const _Float16 *wnext = wbase + (size_t)9 * KT * c1;
+      if (TAIL == CK || chunk + 1 < NCHUNK - 1)
+        fetch_chunk<CK>(A, B, wnext, st, c1, y0, x0, W, H, tid);
+      else
+        fetch_chunk<TAIL>(A, B, wnext, st, c1, y0, x0, W, H, tid);
     }
+    if (fullNow)
+      mma_chunk<CK>(sIn, sW, acc, wv, lane);
+    else
+      mma_chunk<TAIL>(sIn, sW, acc, wv, lane);
     DNX_SYNC();
   }
 
