@@ -85,6 +85,9 @@ SIGNATURES = {
     "denox_hip_compile": (c_int, [c_void_p, POINTER(CompileOptions), c_void_p, POINTER(c_void_p), POINTER(c_size_t)]),
     "denox_hip_last_compile_report": (c_char_p, []),
     "denox_hip_free": (None, [c_void_p]),
+    "denox_hip_dnx_describe": (c_int, [c_void_p, c_size_t, POINTER(c_char_p), POINTER(c_int64), c_uint32, POINTER(c_void_p)]),
+    "denox_hip_min_cost_subgraph": (c_int, [c_uint32, c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_void_p,
+                                            c_void_p, POINTER(c_uint32), POINTER(c_double)]),
     "denox_hip_db_open": (c_int, [c_char_p, POINTER(c_void_p)]),
     "denox_hip_db_close": (None, [c_void_p]),
     "denox_hip_db_row_count": (c_int, [c_void_p, POINTER(c_uint64)]),

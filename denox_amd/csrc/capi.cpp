@@ -224,6 +224,99 @@ int denox_hip_compile(const denox_hip_builder *b, const denox_hip_compile_option
   });
 }
 const char *denox_hip_last_compile_report(void) { return g_lastReport.c_str(); }
+
+int denox_hip_min_cost_subgraph(uint32_t node_count, const uint8_t *is_input, uint32_t edge_count, const uint32_t *edge_input_offsets,
+                                 const int32_t *edge_inputs, const int32_t *edge_outputs, const double *edge_costs, uint32_t output_count,
+                                 const int32_t *outputs, uint32_t *out_chosen, uint32_t *out_chosen_count, double *out_total) {
+  return guarded([&] {
+    need(is_input, "is_input"); need(edge_input_offsets, "edge_input_offsets"); need(edge_outputs, "edge_outputs"); need(edge_costs, "edge_costs");
+    need(outputs, "outputs"); need(out_chosen, "out_chosen"); need(out_chosen_count, "out_chosen_count");
+    std::vector<bool> isIn(node_count);
+    for (uint32_t i = 0; i < node_count; ++i) isIn[i] = is_input[i] != 0;
+    std::vector<compiler::HyperEdge> edges(edge_count);
+    std::vector<double> costs(edge_costs, edge_costs + edge_count);
+    for (uint32_t e = 0; e < edge_count; ++e) {
+      if (edge_input_offsets[e + 1] < edge_input_offsets[e]) fail(Status::InvalidArgument, "edge_input_offsets must be non-decreasing");
+      if (edge_input_offsets[e + 1] > edge_input_offsets[e]) need(edge_inputs, "edge_inputs");
+      edges[e].inputs.assign(edge_inputs + edge_input_offsets[e], edge_inputs + edge_input_offsets[e + 1]);
+      edges[e].output = edge_outputs[e];
+    }
+    double total = 0.0;
+    const std::vector<size_t> chosen = compiler::minimum_cost_subgraph(isIn, edges, costs, std::vector<int>(outputs, outputs + output_count), &total);
+    for (size_t i = 0; i < chosen.size(); ++i) out_chosen[i] = static_cast<uint32_t>(chosen[i]);
+    *out_chosen_count = static_cast<uint32_t>(chosen.size());
+    if (out_total) *out_total = total;
+  });
+}
+
+static void jsonEscape(std::ostringstream &o, const std::string &s) {
+  o << '"';
+  for (char c : s) {
+    if (c == '"' || c == '\\') o << '\\' << c;
+    else if (static_cast<unsigned char>(c) < 0x20) o << ' ';
+    else o << c;
+  }
+  o << '"';
+}
+
+int denox_hip_dnx_describe(const void *dnxbuf, size_t size, const char *const *names, const int64_t *values, uint32_t n, char **out_json) {
+  return guarded([&] {
+    need(dnxbuf, "dnx"); need(out_json, "out_json");
+    const dnx::Model m = dnx::deserialize(dnxbuf, size);
+    std::vector<int64_t> vars(m.sym_ir.varCount, 0);
+    for (uint32_t i = 0; i < n; ++i) {
+      need(names, "names"); need(values, "values");
+      for (const auto &vn : m.value_names)
+        if (vn.name == names[i] && vn.value.symbolic && static_cast<uint64_t>(vn.value.value) < vars.size()) vars[static_cast<size_t>(vn.value.value)] = values[i];
+    }
+    const std::vector<int64_t> dp = m.sym_ir.eval(vars);
+    std::ostringstream o;
+    o << "{\"producer\":"; jsonEscape(o, m.info.producer);
+    o << ",\"var_count\":" << m.sym_ir.varCount << ",\"sym_ops\":" << m.sym_ir.ops.size();
+    o << ",\"value_names\":[";
+    for (size_t i = 0; i < m.value_names.size(); ++i) { if (i) o << ','; jsonEscape(o, m.value_names[i].name); }
+    o << "],\"inputs\":[";
+    for (size_t i = 0; i < m.inputs.size(); ++i) o << (i ? "," : "") << m.inputs[i];
+    o << "],\"outputs\":[";
+    for (size_t i = 0; i < m.outputs.size(); ++i) o << (i ? "," : "") << m.outputs[i];
+    o << "],\"buffers\":[";
+    for (size_t i = 0; i < m.buffers.size(); ++i) o << (i ? "," : "") << "{\"size\":" << m.buffers[i].size.eval(dp) << ",\"alignment\":" << m.buffers[i].alignment << "}";
+    o << "],\"tensors\":[";
+    std::vector<bool> isParam(m.tensors.size(), false);
+    for (const auto &in : m.initializers) isParam[in.tensor] = true;
+    for (size_t i = 0; i < m.tensors.size(); ++i) {
+      const auto &t = m.tensors[i];
+      o << (i ? "," : "") << "{\"buffer\":" << t.buffer << ",\"offset\":" << t.offset.eval(dp) << ",\"size\":" << t.size.eval(dp) << ",\"format\":" << static_cast<int>(t.info.format)
+        << ",\"param\":" << (isParam[i] ? "true" : "false") << ",\"name\":";
+      jsonEscape(o, t.info.name);
+      if (t.info.has_extent) o << ",\"width\":" << t.info.width.eval(dp) << ",\"height\":" << t.info.height.eval(dp) << ",\"channels\":" << t.info.channels.eval(dp);
+      o << "}";
+    }
+    o << "],\"binaries\":" << m.shader_binaries.size() << ",\"dispatches\":[";
+    for (size_t i = 0; i < m.dispatches.size(); ++i) {
+      const auto &d = m.dispatches[i];
+      o << (i ? "," : "") << "{\"name\":"; jsonEscape(o, d.info.name);
+      o << ",\"entry_point\":"; jsonEscape(o, d.entry_point);
+      o << ",\"src_path\":"; jsonEscape(o, d.info.src_path);
+      o << ",\"debug_info\":"; jsonEscape(o, d.info.debug_info);
+      o << ",\"binary_id\":" << d.binary_id << ",\"workgroup_count\":[" << d.workgroup_count_x.eval(dp) << ',' << d.workgroup_count_y.eval(dp) << ',' << d.workgroup_count_z.eval(dp)
+        << "],\"workgroup_size\":[" << d.workgroup_size[0] << ',' << d.workgroup_size[1] << ',' << d.workgroup_size[2] << "],\"bindings\":[";
+      bool first = true;
+      for (const auto &sb : d.bindings)
+        for (const auto &b : sb.bindings) { o << (first ? "" : ",") << "{\"set\":" << sb.set << ",\"binding\":" << b.binding << ",\"access\":" << static_cast<int>(b.access) << ",\"tensor\":" << b.tensor << "}"; first = false; }
+      o << "],\"push_constants\":[";
+      for (size_t f = 0; f < d.push_constant.fields.size(); ++f) o << (f ? "," : "") << d.push_constant.fields[f].source.eval(dp);
+      o << "],\"memory_reads\":" << (d.info.has_reads ? d.info.memory_reads.eval(dp) : 0) << ",\"memory_writes\":" << (d.info.has_writes ? d.info.memory_writes.eval(dp) : 0)
+        << ",\"flops\":" << (d.info.has_flops ? d.info.flops.eval(dp) : 0) << "}";
+    }
+    o << "]}";
+    const std::string s = o.str();
+    char *p = static_cast<char *>(std::malloc(s.size() + 1));
+    if (!p) fail(Status::Internal, "out of host memory");
+    std::memcpy(p, s.c_str(), s.size() + 1);
+    *out_json = p;
+  });
+}
 void denox_hip_free(void *p) { std::free(p); }
 
 // ---------------------------------------------------------------- database

@@ -74,27 +74,32 @@ double edge_cost_ms(const SuperGraphEdge &e, const std::vector<int64_t> &dp, con
 
 namespace {
 struct Selector {
-  const Model &model;
-  const SuperGraph &g;
+  const std::vector<bool> &isInput;
+  const std::vector<HyperEdge> &edges;
   const std::vector<double> &cost;
   std::vector<std::vector<size_t>> producers;
   std::map<std::vector<int>, std::pair<double, long>> memo; // needed set -> (cost, edge chosen for its largest member)
+
+  std::vector<int> after(const std::vector<int> &needed, size_t e) const {
+    std::vector<int> sub(needed.begin(), needed.end() - 1);
+    for (int in : edges[e].inputs)
+      if (!isInput[static_cast<size_t>(in)]) sub.push_back(in);
+    std::sort(sub.begin(), sub.end());
+    sub.erase(std::unique(sub.begin(), sub.end()), sub.end());
+    return sub;
+  }
 
   double solve(const std::vector<int> &needed) {
     if (needed.empty()) return 0.0;
     auto it = memo.find(needed);
     if (it != memo.end()) return it->second.first;
-    const int t = needed.back(); // largest handle: nothing else still needed depends on it being produced later
-    std::vector<int> rest(needed.begin(), needed.end() - 1);
-    double best = 1e300;
+    // the largest node id: node ids are topologically ordered, so no other node
+    // still needed can require it to be produced later
+    const int t = needed.back();
+    double best = kInfiniteCost;
     long bestEdge = -1;
-    for (size_t e : producers[t]) {
-      std::vector<int> sub = rest;
-      for (int in : g.edges[e].inputs)
-        if (!model.tensors()[in].isInput) sub.push_back(in);
-      std::sort(sub.begin(), sub.end());
-      sub.erase(std::unique(sub.begin(), sub.end()), sub.end());
-      const double c = cost[e] + solve(sub);
+    for (size_t e : producers[static_cast<size_t>(t)]) {
+      const double c = cost[e] + solve(after(needed, e));
       if (c < best) { best = c; bestEdge = static_cast<long>(e); }
     }
     memo[needed] = {best, bestEdge};
@@ -103,38 +108,48 @@ struct Selector {
 };
 } // namespace
 
-std::vector<size_t> select_schedule(const Model &model, const SuperGraph &g, const std::vector<double> &edgeCost) {
-  Selector s{model, g, edgeCost, {}, {}};
-  s.producers.resize(model.tensors().size());
-  for (size_t e = 0; e < g.edges.size(); ++e) {
-    const auto &edge = g.edges[e];
+std::vector<size_t> minimum_cost_subgraph(const std::vector<bool> &isInput, const std::vector<HyperEdge> &edges, const std::vector<double> &edgeCost,
+                                          const std::vector<int> &outputs, double *totalCost) {
+  if (edges.size() != edgeCost.size()) fail(Status::InvalidArgument, "one cost per edge expected");
+  Selector s{isInput, edges, edgeCost, {}, {}};
+  s.producers.resize(isInput.size());
+  for (size_t e = 0; e < edges.size(); ++e) {
+    const auto &edge = edges[e];
+    if (edge.output < 0 || static_cast<size_t>(edge.output) >= isInput.size()) fail(Status::InvalidArgument, "edge output out of range");
     for (int in : edge.inputs)
-      if (in >= edge.output) fail(Status::Internal, "super-graph edge is not topologically ordered");
-    s.producers[edge.output].push_back(e);
+      if (in < 0 || in >= edge.output) fail(Status::InvalidArgument, "hyper-graph nodes must be numbered in topological order");
+    s.producers[static_cast<size_t>(edge.output)].push_back(e);
   }
   std::vector<int> needed;
-  for (TensorHandle o : model.outputs())
-    if (!model.tensors()[o].isInput) needed.push_back(o);
+  for (int o : outputs) {
+    if (o < 0 || static_cast<size_t>(o) >= isInput.size()) fail(Status::InvalidArgument, "output out of range");
+    if (!isInput[static_cast<size_t>(o)]) needed.push_back(o);
+  }
   std::sort(needed.begin(), needed.end());
   needed.erase(std::unique(needed.begin(), needed.end()), needed.end());
   const double total = s.solve(needed);
-  if (total >= 1e299) fail(Status::Unsupported, "no kernel implements part of this graph (a layer has no matching shader)");
-  // walk the memo to recover the chosen edges
+  if (totalCost) *totalCost = total;
   std::vector<size_t> chosen;
+  if (total >= kInfiniteCost) return chosen;
   std::vector<int> cur = needed;
   while (!cur.empty()) {
-    const auto &entry = s.memo.at(cur);
-    const size_t e = static_cast<size_t>(entry.second);
+    const size_t e = static_cast<size_t>(s.memo.at(cur).second);
     chosen.push_back(e);
-    std::vector<int> sub(cur.begin(), cur.end() - 1);
-    for (int in : g.edges[e].inputs)
-      if (!model.tensors()[in].isInput) sub.push_back(in);
-    std::sort(sub.begin(), sub.end());
-    sub.erase(std::unique(sub.begin(), sub.end()), sub.end());
-    cur = std::move(sub);
+    cur = s.after(cur, e);
   }
-  // producers come before consumers when sorted by output handle
-  std::sort(chosen.begin(), chosen.end(), [&](size_t a, size_t b) { return g.edges[a].output < g.edges[b].output; });
+  // producers come before consumers when sorted by output node
+  std::sort(chosen.begin(), chosen.end(), [&](size_t a, size_t b) { return edges[a].output < edges[b].output; });
+  return chosen;
+}
+
+std::vector<size_t> select_schedule(const Model &model, const SuperGraph &g, const std::vector<double> &edgeCost) {
+  std::vector<bool> isInput(model.tensors().size());
+  for (size_t i = 0; i < isInput.size(); ++i) isInput[i] = model.tensors()[i].isInput;
+  std::vector<HyperEdge> edges;
+  for (const auto &e : g.edges) edges.push_back(HyperEdge{e.inputs, e.output});
+  double total = 0.0;
+  std::vector<size_t> chosen = minimum_cost_subgraph(isInput, edges, edgeCost, model.outputs(), &total);
+  if (total >= kInfiniteCost) fail(Status::Unsupported, "no kernel implements part of this graph (a layer has no matching shader)");
   return chosen;
 }
 

@@ -33,8 +33,20 @@ std::vector<int64_t> assumed_symeval(const Model &model, const SymGraph &sym, co
 // database where every dispatch of the edge has one, else a roofline estimate.
 double edge_cost_ms(const SuperGraphEdge &e, const std::vector<int64_t> &dp, const Db *db, const CompileOptions &opt, bool *measured);
 
-// Minimum-cost set of edges producing every model output from the model
-// inputs; returns edge indices in execution order.
+// Minimum-cost sub-hypergraph (common/src/denox/algorithm/minimum_const_subgraph.hpp:45-49 of
+// the reference): nodes are numbered in topological order, an edge produces its
+// output node from all of its input nodes at a cost, every node is produced at
+// most once.  Returns the edges of a cheapest set that derives every requested
+// output from the input nodes, in execution order; empty with *totalCost >=
+// kInfiniteCost when some output cannot be produced.  Exact: memoised search over
+// the set of nodes still to be produced.
+struct HyperEdge { std::vector<int> inputs; int output; };
+constexpr double kInfiniteCost = 1e300;
+std::vector<size_t> minimum_cost_subgraph(const std::vector<bool> &isInput, const std::vector<HyperEdge> &edges, const std::vector<double> &edgeCost,
+                                          const std::vector<int> &outputs, double *totalCost);
+
+// Minimum-cost set of super-graph edges producing every model output from the
+// model inputs; returns edge indices in execution order.
 std::vector<size_t> select_schedule(const Model &model, const SuperGraph &g, const std::vector<double> &edgeCost);
 
 std::vector<uint8_t> compile(const Model &model, const hip::HipCompiler &hipc, const Db *db, const CompileOptions &opt, CompileReport *report);

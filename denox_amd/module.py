@@ -110,6 +110,19 @@ def compile_model(model: Model, *, features: Optional[dict] = None, input_layout
         _capi.lib().denox_hip_free(blob)
 
 
+def describe(dnx: bytes, **extents: int) -> dict:
+    """Decode a compiled model (no GPU needed), symbolic quantities evaluated at `extents`."""
+    import json
+    names = (c_char_p * len(extents))(*[k.encode() for k in extents])
+    vals = (c_int64 * len(extents))(*[int(v) for v in extents.values()])
+    p = c_void_p()
+    _capi.check(_capi.lib().denox_hip_dnx_describe(dnx, len(dnx), names, vals, len(extents), byref(p)))
+    try:
+        return json.loads(ctypes.string_at(p.value).decode())
+    finally:
+        _capi.lib().denox_hip_free(p)
+
+
 def last_compile_report() -> str:
     return (_capi.lib().denox_hip_last_compile_report() or b"").decode()
 

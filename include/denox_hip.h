@@ -138,6 +138,22 @@ int denox_hip_compile(const denox_hip_builder *b, const denox_hip_compile_option
 /* one line per selected dispatch of the most recent compile on this thread */
 const char *denox_hip_last_compile_report(void);
 void denox_hip_free(void *p);
+/* JSON description of a compiled model with every symbolic quantity evaluated
+ * at the given extents: tensors, buffers, dispatches (workgroup counts, push
+ * constants, bindings, bytes and FLOPs).  Needs no GPU.  The role of reading
+ * a dnx file back (runtime/src/denox/runtime/model.cpp:637-659).  Release the
+ * string with denox_hip_free. */
+int denox_hip_dnx_describe(const void *dnx, size_t size, const char *const *names, const int64_t *values, uint32_t n, char **out_json);
+
+/* minimum_cost_subgraph (common/src/denox/algorithm/minimum_const_subgraph.hpp:45-49), the search
+ * behind schedule selection (compiler/src/denox/compiler/selection/selection.cpp:23-266), on a
+ * caller-supplied hyper-graph.  Nodes 0..node_count-1 are numbered in topological order; edge e
+ * produces edge_outputs[e] from edge_inputs[edge_input_offsets[e] .. edge_input_offsets[e+1]).
+ * Writes the chosen edge indices in execution order (out_chosen has room for edge_count entries).
+ * *out_total >= 1e300 and zero chosen edges mean that an output cannot be produced. */
+int denox_hip_min_cost_subgraph(uint32_t node_count, const uint8_t *is_input, uint32_t edge_count, const uint32_t *edge_input_offsets,
+                                const int32_t *edge_inputs, const int32_t *edge_outputs, const double *edge_costs, uint32_t output_count,
+                                const int32_t *outputs, uint32_t *out_chosen, uint32_t *out_chosen_count, double *out_total);
 
 /* ------------------------------------------------------------------ database
  * Db::open / populate / bench / query / dumpcsv

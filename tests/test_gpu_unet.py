@@ -1,0 +1,178 @@
+"""GPU parity of whole networks through the C ABI.
+
+Small extents are compared with the oracle's fp32 evaluation of the whole network.
+At the benchmark's full extents the oracle would take minutes, so the comparison
+uses what the domain offers: a 3x3 conv output depends on a 3x3 neighbourhood, so
+random output pixels of the full-size layer are checked against the oracle run on
+crops; the U-Net's receptive field is under 96 pixels, so the centre of an oracle
+evaluation of a 16-aligned crop equals the full-frame result there; and data-movement
+kernels are bit-exact against closed forms at full size."""
+import numpy as np
+import pytest
+
+import denox_amd as dx
+from denox_amd import networks
+from util import assert_bits_equal, assert_conv_close
+
+pytestmark = pytest.mark.gpu
+
+
+def oracle_net(oracle, model, x, H, W, mode="fp32"):
+    return oracle.run_graph(model.to_ops({"H": H, "W": W}), {"input": x}, mode)[model.outputs[0].name]
+
+
+@pytest.mark.parametrize("H,W", [(128, 128), (37, 61), (2, 2)])
+def test_tiny_unet(oracle, H, W):
+    H2, W2 = H // 2 * 2, W // 2 * 2  # the un-wrapped tiny net needs even extents
+    m, _ = networks.build("tiny_unet", seed=3)
+    x = networks.synthetic_input("tiny_unet", H2, W2, seed=3)
+    got = dx.Module.compile(m).instance(H=H2, W=W2).infer(x)[0]
+    assert_conv_close(got, oracle_net(oracle, m, x, H2, W2), f"tiny {H2}x{W2}")
+
+
+@pytest.mark.parametrize("H,W", [(64, 96), (75, 101), (16, 16), (1, 1), (33, 250)])
+def test_oidn_unet_small_extents(oracle, H, W):
+    m, _ = networks.build("oidn_unet", seed=1)
+    x = networks.synthetic_input("oidn_unet", H, W, seed=1)
+    mod = dx.Module.compile(m, assume={"H": H, "W": W})
+    inst = mod.instance(H=H, W=W)
+    got = inst.infer(x)[0]
+    assert got.shape == (H, W, 3)
+    assert_conv_close(got, oracle_net(oracle, m, x, H, W), f"oidn {H}x{W}")
+    # a second frame through the same instance (graph replay) and determinism
+    again = inst.infer(x)[0]
+    assert_bits_equal(again, got, "replay")
+
+
+def test_oidn_unet_one_model_many_extents(oracle):
+    """Dynamic extents: one compiled model, instances at several sizes."""
+    m, _ = networks.build("oidn_unet", seed=2)
+    mod = dx.Module.compile(m)
+    for H, W in [(48, 80), (50, 70), (80, 48)]:
+        x = networks.synthetic_input("oidn_unet", H, W, seed=H)
+        got = mod.instance(H=H, W=W).infer(x)[0]
+        assert_conv_close(got, oracle_net(oracle, m, x, H, W), f"oidn dyn {H}x{W}")
+    with pytest.raises(dx.DenoxHipError):
+        mod.instance(H=48)  # W missing
+
+
+def test_double_width_unet_chw_interface(oracle):
+    """Channel widths doubled, CHW in and out, extents that are not multiples of 16."""
+    H, W = 45, 77
+    m, _ = networks.build("oidn_unet", seed=4, width_mult=2)
+    x = networks.synthetic_input("oidn_unet", H, W, seed=4)
+    mod = dx.Module.compile(m, input_layout=dx.Layout.CHW, output_layout=dx.Layout.CHW, assume={"H": H, "W": W})
+    inst = mod.instance(H=H, W=W)
+    assert inst.input_desc()["layout"] == dx.Layout.CHW and inst.output_desc()["layout"] == dx.Layout.CHW
+    got = inst.infer(np.ascontiguousarray(x.transpose(2, 0, 1)))[0]
+    assert got.shape == (3, H, W)
+    assert_conv_close(got.transpose(1, 2, 0), oracle_net(oracle, m, x, H, W), "2x width CHW")
+
+
+def test_chwc8_interface_bit_exact(oracle):
+    H, W, C = 19, 23, 16
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((H, W, C)).astype(np.float16)
+    m = dx.Model()
+    m.output(m.pool(m.input("input", "W", "H", C)))
+    mod = dx.Module.compile(m, input_layout=dx.Layout.CHWC8, output_layout=dx.Layout.CHWC8)
+    xin = oracle.relayout(x, oracle.LAYOUT_HWC, oracle.LAYOUT_CHWC8, H, W, C).reshape(C // 8, H, W, 8)
+    got = mod.instance(H=H, W=W).infer(xin)[0]
+    want = oracle.relayout(oracle.maxpool(x), oracle.LAYOUT_HWC, oracle.LAYOUT_CHWC8, H // 2, W // 2, C)
+    assert_bits_equal(got.reshape(-1), want, "CHWC8 pool")
+
+
+def test_device_pointer_path_matches_host_path():
+    torch = pytest.importorskip("torch")
+    H, W = 40, 56
+    m, _ = networks.build("oidn_unet", seed=5)
+    x = networks.synthetic_input("oidn_unet", H, W, seed=5)
+    inst = dx.Module.compile(m).instance(H=H, W=W)
+    want = inst.infer(x)[0]
+    d_in = torch.from_numpy(x).cuda()
+    outs = [torch.zeros((H, W, 3), dtype=torch.float16, device="cuda") for _ in range(2)]
+    torch.cuda.synchronize()
+    for o in outs + [outs[0]]:  # new addresses re-bind the graph; a repeated address reuses it
+        inst.infer_device([d_in.data_ptr()], [o.data_ptr()])
+        inst.synchronize()
+        assert_bits_equal(o.cpu().numpy(), want, "device-pointer path")
+    inst.infer_device(None, None)  # the instance's own buffers still work afterwards
+    inst.synchronize()
+
+
+# ----------------------------------------------------------------------------- full size
+FULL_H, FULL_W = 1080, 1920
+
+
+def test_full_size_conv64_against_oracle_on_crops(oracle):
+    """conv3x3 64->64 + bias + ReLU at 1080 x 1920: 64 random 9x9 output patches (every
+    border included) against the oracle evaluated on the matching 11x11 input crops."""
+    rng = np.random.default_rng(11)
+    m, _ = networks.build("single_conv", seed=11)
+    x = networks.synthetic_input("single_conv", FULL_H, FULL_W, seed=11)
+    got = dx.Module.compile(m, assume={"H": FULL_H, "W": FULL_W}).instance(H=FULL_H, W=FULL_W).infer(x)[0]
+    ops = m.to_ops({"H": 0, "W": 0})
+    corners = [(0, 0), (0, FULL_W - 9), (FULL_H - 9, 0), (FULL_H - 9, FULL_W - 9), (0, 1000), (FULL_H - 9, 31), (500, 0), (7, FULL_W - 9)]
+    spots = corners + [(int(rng.integers(0, FULL_H - 9)), int(rng.integers(0, FULL_W - 9))) for _ in range(56)]
+    for y, xx in spots:
+        y0, y1, x0, x1 = max(y - 1, 0), min(y + 10, FULL_H), max(xx - 1, 0), min(xx + 10, FULL_W)
+        crop = np.ascontiguousarray(x[y0:y1, x0:x1])
+        want = oracle.run_graph(ops, {"input": crop}, "fp32")[m.outputs[0].name]
+        # rows/cols of the crop that are true image borders keep their zero padding; interior cuts are dropped
+        want = want[y - y0:y - y0 + 9, xx - x0:xx - x0 + 9]
+        assert_conv_close(got[y:y + 9, xx:xx + 9], want, f"patch at {(y, xx)}")
+    assert (got >= 0).all()
+
+
+def test_full_size_conv64_closed_forms():
+    C = 64
+    ones = np.ones((FULL_H, FULL_W, C), np.float16)
+    m = dx.Model()
+    m.output(m.conv2d(m.input("input", "W", "H", C), np.ones((C, C, 3, 3), np.float16)))
+    got = dx.Module.compile(m, assume={"H": FULL_H, "W": FULL_W}).instance(H=FULL_H, W=FULL_W).infer(ones)[0]
+    assert (got[1:-1, 1:-1] == 9 * C).all() and (got[0, 1:-1] == 6 * C).all() and (got[-1, 1:-1] == 6 * C).all()
+    assert (got[1:-1, 0] == 6 * C).all() and (got[1:-1, -1] == 6 * C).all()
+    assert (got[[0, 0, -1, -1], [0, -1, 0, -1]] == 4 * C).all()
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((FULL_H, FULL_W, C)).astype(np.float16)
+    w = np.zeros((C, C, 3, 3), np.float16)
+    w[np.arange(C), np.arange(C), 1, 1] = 1
+    m = dx.Model()
+    m.output(m.conv2d(m.input("input", "W", "H", C), w))
+    got = dx.Module.compile(m, assume={"H": FULL_H, "W": FULL_W}).instance(H=FULL_H, W=FULL_W).infer(x)[0]
+    assert_bits_equal(got, x, "identity conv at full size")
+
+
+def test_full_size_bandwidth_kernels_bit_exact():
+    rng = np.random.default_rng(6)
+    C = 32
+    x = rng.standard_normal((FULL_H, FULL_W, C)).astype(np.float16)
+    m = dx.Model()
+    i = m.input("input", "W", "H", C)
+    p = m.pad_to_multiple(i, 16)
+    m.output(m.slice(m.concat(m.upsample(m.pool(p)), p), 0, i.width, 0, i.height))
+    got = dx.Module.compile(m).instance(H=FULL_H, W=FULL_W).infer(x)[0]
+    xp = np.pad(x, ((0, 8), (0, 0), (0, 0)), mode="edge")
+    pooled = xp.reshape(544, 2, 960, 2, C).max(axis=(1, 3))
+    up = np.repeat(np.repeat(pooled, 2, axis=0), 2, axis=1)
+    want = np.concatenate([up, xp], axis=2)[:FULL_H, :FULL_W]
+    assert_bits_equal(got, want, "pad/pool/upsample/concat/slice at 1080p")
+
+
+def test_full_size_oidn_unet_centre_of_crop(oracle):
+    """OIDN U-Net at 1920 x 1080 against the oracle on 16-aligned 272 x 272 crops: the receptive
+    field is below 96 pixels, so the central 80 x 80 of a crop evaluation equals the full-frame result."""
+    m, _ = networks.build("oidn_unet", seed=0)
+    x = networks.synthetic_input("oidn_unet", FULL_H, FULL_W, seed=0)
+    got = dx.Module.compile(m, assume={"H": FULL_H, "W": FULL_W}).instance(H=FULL_H, W=FULL_W).infer(x)[0]
+    assert got.shape == (FULL_H, FULL_W, 3) and np.isfinite(got).all()
+    S, Mg = 272, 96
+    for y0, x0 in [(0, 0), (400, 800), (FULL_H - S + 8, FULL_W - S)]:  # last crop reaches the replicate-padded bottom rows
+        y0 -= y0 % 16
+        x0 -= x0 % 16
+        h = min(S, FULL_H - y0)
+        crop = np.ascontiguousarray(x[y0:y0 + h, x0:x0 + S])
+        want = oracle_net(oracle, m, crop, h, S)
+        ys = slice(0 if y0 == 0 else Mg, h if y0 + h >= FULL_H else h - Mg)
+        xs = slice(0 if x0 == 0 else Mg, S if x0 + S >= FULL_W else S - Mg)
+        assert_conv_close(got[y0:y0 + h, x0:x0 + S][ys, xs], want[ys, xs], f"crop at {(y0, x0)}")
