@@ -34,7 +34,7 @@ def lavapipe_probe() -> str:
     return "unavailable (denox itself cannot be built here: needs glslang, SPIRV-Tools, FlatBuffers)"
 
 
-def cpu_baseline(seed: int, budget_h: int = 272, budget_w: int = 480) -> dict:
+def cpu_baseline(seed: int, budget_h: int = 1080, budget_w: int = 1920) -> dict:
     """CPU oracle (fp32, OpenMP) on a crop of the benchmark frame, same network and weights."""
     import numpy as np
     import oracle
@@ -47,7 +47,7 @@ def cpu_baseline(seed: int, budget_h: int = 272, budget_w: int = 480) -> dict:
     oracle.run_graph(ops, {"input": x}, "f16")
     dt = time.perf_counter() - t0
     return {"value": budget_h * budget_w / dt * 1e-6, "unit": "Mpix/s", "cores": oracle.num_threads(), "kind": "port",
-            "sample": f"one {budget_w}x{budget_h} frame of the same U-Net (1/16 of the 1080p pixels), {dt:.1f} s wall",
+            "sample": f"one {budget_w}x{budget_h} frame of the same U-Net, fp32 accumulation, {dt:.1f} s wall",
             "lavapipe_baseline": lavapipe_probe()}
 
 
@@ -62,7 +62,8 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--per-dispatch", action="store_true", help="print the per-dispatch report to stderr")
     ap.add_argument("--conv-config", default=None)
-    ap.add_argument("--db", default=None, help="timing table to select the schedule with")
+    ap.add_argument("--db", default=None, help="timing table to select the schedule with (default: measure one now)")
+    ap.add_argument("--no-tune", action="store_true", help="skip the timing table; select by roofline estimates")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on exactly one GPU (independent frames shard trivially across GPUs; "
@@ -79,7 +80,18 @@ def main() -> int:
         return 1
     H, W = args.height, args.width
     model, _ = networks.build("oidn_unet", seed=args.seed)
-    db = dx.Db(args.db) if args.db else None
+    # The reference workflow: populate the table with every candidate dispatch, time them on
+    # this GPU, then compile against the measured latencies (README.md:112-199 of the reference:
+    # `denox populate`, `denox bench`, `denox compile --db`).
+    db = None
+    tune_s = 0.0
+    if not args.no_tune:
+        import tempfile
+        t0 = time.perf_counter()
+        db = dx.Db(args.db or os.path.join(tempfile.mkdtemp(prefix="denox_hip_"), "gpu.db"))
+        db.populate(model, assume={"H": H, "W": W}, conv_config=args.conv_config)
+        db.bench(min_samples=10, max_relative_error=0.03, max_samples=50, save_progress=bool(args.db))
+        tune_s = time.perf_counter() - t0
     blob = dx.compile_model(model, assume={"H": H, "W": W}, conv_config=args.conv_config, db=db)
     mod = dx.Module.load(blob)
     inst = mod.instance(H=H, W=W)
@@ -143,7 +155,9 @@ def main() -> int:
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": f"OIDN-style U-Net 9->3, fp16 HWC, {W}x{H}, replicate-pad to multiple of 16 + crop included, "
-                               f"{mod.runtime_model.dispatch_count} dispatches in one hipGraph", "device_bytes": inst.device_bytes},
+                               f"{mod.runtime_model.dispatch_count} dispatches in one hipGraph", "device_bytes": inst.device_bytes,
+                   "schedule": "min-cost over measured dispatch latencies" if db is not None else "min-cost over roofline estimates",
+                   "tuning_seconds": round(tune_s, 2)},
         "roofline": roofline,
     }
     if not args.no_cpu_baseline:

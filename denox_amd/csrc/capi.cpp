@@ -201,6 +201,9 @@ void denox_hip_compile_options_default(denox_hip_compile_options *o) {
   std::memset(o, 0, sizeof(*o));
   o->enable_conv_relu_fusion = o->enable_concat_conv_fusion = o->enable_upsample_fusion = o->enable_pool_fusion = 1;
   o->device = -1;
+  o->populate_compile_kernels = 1;
+  o->kernel_shard_index = 0;
+  o->kernel_shard_count = 1;
 }
 
 int denox_hip_compile(const denox_hip_builder *b, const denox_hip_compile_options *o, const denox_hip_db *db, void **out_dnx, size_t *out_size) {
@@ -331,7 +334,7 @@ int denox_hip_db_populate(denox_hip_db *db, const denox_hip_builder *b, const de
   return guarded([&] {
     need(db, "db"); need(b, "builder");
     const hip::HipCompiler hipc = makeCompiler();
-    const size_t n = compiler::populate(db->db, b->model, hipc, toOptions(o));
+    const size_t n = compiler::populate(db->db, b->model, hipc, toOptions(o), !o || o->populate_compile_kernels != 0, o ? o->kernel_shard_index : 0, o ? o->kernel_shard_count : 1);
     if (out_added) *out_added = n;
   });
 }

@@ -275,7 +275,8 @@ std::vector<uint8_t> compile(const Model &modelIn, const hip::HipCompiler &hipc,
     ComputeDispatch d;
     d.kernel = hipc.read("relayout.hip");
     d.kernel.define("CH", n.channels); d.kernel.define("SRC_LAYOUT", layoutId(from)); d.kernel.define("DST_LAYOUT", layoutId(to));
-    d.entryPoint = "relayout";
+    d.entryPoint = "relayout_c" + std::to_string(n.channels) + "_" + std::to_string(layoutId(from)) + "to" + std::to_string(layoutId(to));
+    d.kernel.define("KERNEL_NAME", d.entryPoint);
     d.workgroupCountX = sym.cdiv(sym.mul(n.width, n.height), 256);
     d.workgroupCountY = d.workgroupCountZ = Sym::Const(1);
     d.workgroupSize[0] = 256;
@@ -346,7 +347,7 @@ std::vector<uint8_t> compile(const Model &modelIn, const hip::HipCompiler &hipc,
   return dnx::serialize(out);
 }
 
-size_t populate(Db &db, const Model &modelIn, const hip::HipCompiler &hipc, const CompileOptions &opt, bool compileKernels) {
+size_t populate(Db &db, const Model &modelIn, const hip::HipCompiler &hipc, const CompileOptions &opt, bool compileKernels, unsigned shardIndex, unsigned shardCount) {
   Model model = modelIn;
   SymGraph &sym = model.symGraph();
   const auto shaders = get_all_shaders(&hipc);
@@ -384,7 +385,12 @@ size_t populate(Db &db, const Model &modelIn, const hip::HipCompiler &hipc, cons
     for (const auto &edge : g.edges)
       for (const auto &d : edge.dispatches) distinct.emplace(d.kernel.sha256(), &d.kernel);
     std::vector<const hip::HipCompilerInstance *> work;
-    for (const auto &kv : distinct) work.push_back(kv.second);
+    {
+      // several processes can split the work: hiprtc serialises compilations inside one process
+      size_t idx = 0;
+      for (const auto &kv : distinct)
+        if (shardCount <= 1 || idx++ % shardCount == shardIndex) work.push_back(kv.second);
+    }
     std::atomic<size_t> next{0};
     std::mutex errMutex;
     std::string firstError;

@@ -53,7 +53,8 @@ std::vector<uint8_t> compile(const Model &model, const hip::HipCompiler &hipc, c
 
 // Insert one row per candidate dispatch (all matches, all configurations),
 // evaluated at the assumed extents; returns the number of new rows.
-size_t populate(Db &db, const Model &model, const hip::HipCompiler &hipc, const CompileOptions &opt, bool compileKernels = true);
+size_t populate(Db &db, const Model &model, const hip::HipCompiler &hipc, const CompileOptions &opt, bool compileKernels = true,
+                unsigned shardIndex = 0, unsigned shardCount = 1);
 
 std::vector<uint8_t> push_constant_bytes(const ComputeDispatch &d, const std::vector<int64_t> &dp, std::vector<uint16_t> *offsets = nullptr);
 

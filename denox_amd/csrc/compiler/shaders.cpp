@@ -220,9 +220,12 @@ public:
     k.define("POOL", pool ? 1 : 0); k.define("HAS_BIAS", conv.hasBias ? 1 : 0);
     k.define("WAVES", cfg.waves); k.define("RPW", cfg.rpw); k.define("CK", cfg.ck);
 
+    std::string entry = "conv3x3_c" + std::to_string(CA) + (up ? "u" : "") + (CB ? "p" + std::to_string(CB) : "") + "_k" + std::to_string(conv.K) +
+                        (act == 1 ? "_relu" : act == 2 ? "_lrelu" : "") + (pool ? "_pool" : "") + "_" + cfg.name;
+    k.define("KERNEL_NAME", entry);
     const Sym W = convIn.width, H = convIn.height;
     const unsigned th = cfg.waves * cfg.rpw;
-    auto d = impl.registerDispatch(k, "conv3x3_mfma", sym.cdiv(W, 32), sym.cdiv(H, th), Sym::Const(g.KOUTP / g.KT), cfg.waves * 64);
+    auto d = impl.registerDispatch(k, entry, sym.cdiv(W, 32), sym.cdiv(H, th), Sym::Const(g.KOUTP / g.KT), cfg.waves * 64);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     if (CB) d.addBinding(dnx::Access::ReadOnly, m.inputs[1]);
     d.addBinding(dnx::Access::WriteOnly, m.output);
@@ -306,7 +309,9 @@ public:
     const unsigned vec = in.channels % 8 == 0 ? 8 : 1;
     auto k = m_compiler->read("pool.hip");
     k.define("CH", in.channels); k.define("KX", op.kernelX); k.define("KY", op.kernelY); k.define("VEC", vec);
-    auto d = impl.registerDispatch(k, "pool_max", linearGrid(sym, out.width, out.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
+    const std::string entry = "pool_max_c" + std::to_string(in.channels) + "v" + std::to_string(vec);
+    k.define("KERNEL_NAME", entry);
+    auto d = impl.registerDispatch(k, entry, linearGrid(sym, out.width, out.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     d.addBinding(dnx::Access::WriteOnly, m.output);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
@@ -325,7 +330,9 @@ public:
     const unsigned vec = in.channels % 8 == 0 ? 8 : 1;
     auto k = m_compiler->read("upsample.hip");
     k.define("CH", in.channels); k.define("SCALE", op.scale); k.define("VEC", vec);
-    auto d = impl.registerDispatch(k, "upsample_nearest", linearGrid(sym, in.width, in.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
+    const std::string entry = "upsample_c" + std::to_string(in.channels) + "v" + std::to_string(vec);
+    k.define("KERNEL_NAME", entry);
+    auto d = impl.registerDispatch(k, entry, linearGrid(sym, in.width, in.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     d.addBinding(dnx::Access::WriteOnly, m.output);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
@@ -351,7 +358,9 @@ public:
       auto k = m_compiler->read("copy_transform.hip");
       k.define("IN_CH", in.channels); k.define("IN_CH_OFFSET", 0); k.define("OUT_CH", out.channels); k.define("OUT_CH_OFFSET", off);
       k.define("COUNT", in.channels); k.define("VEC", vec);
-      auto d = impl.registerDispatch(k, "copy_transform", linearGrid(sym, in.width, in.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
+      const std::string entry = "copy_c" + std::to_string(in.channels) + "_to_c" + std::to_string(out.channels) + "o" + std::to_string(off) + "v" + std::to_string(vec);
+      k.define("KERNEL_NAME", entry);
+      auto d = impl.registerDispatch(k, entry, linearGrid(sym, in.width, in.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
       d.addBinding(dnx::Access::ReadOnly, m.inputs[s]);
       d.addBinding(dnx::Access::WriteOnly, m.output);
       d.addPushConstant(in.width); d.addPushConstant(in.height);
@@ -373,7 +382,9 @@ public:
     auto k = m_compiler->read("activation.hip");
     k.define("CH", in.channels); k.define("VEC", vec); k.define("ACT", op.func == ActivationFunction::ReLU ? 1 : 2);
     if (op.func == ActivationFunction::LeakyReLU) k.define("ALPHA", fmtFloat(op.alpha));
-    auto d = impl.registerDispatch(k, "activation", linearGrid(sym, in.width, in.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
+    const std::string entry = std::string(op.func == ActivationFunction::ReLU ? "relu_c" : "leaky_relu_c") + std::to_string(in.channels) + "v" + std::to_string(vec);
+    k.define("KERNEL_NAME", entry);
+    auto d = impl.registerDispatch(k, entry, linearGrid(sym, in.width, in.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     d.addBinding(dnx::Access::WriteOnly, m.output);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
@@ -394,7 +405,9 @@ public:
     const unsigned vec = in.channels % 8 == 0 ? 8 : 1;
     auto k = m_compiler->read("pad.hip");
     k.define("CH", in.channels); k.define("VEC", vec);
-    auto d = impl.registerDispatch(k, "memory_pad", linearGrid(sym, out.width, out.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
+    const std::string entry = "memory_pad_c" + std::to_string(in.channels) + "v" + std::to_string(vec);
+    k.define("KERNEL_NAME", entry);
+    auto d = impl.registerDispatch(k, entry, linearGrid(sym, out.width, out.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     d.addBinding(dnx::Access::WriteOnly, m.output);
     d.addPushConstant(out.width); d.addPushConstant(out.height);
@@ -414,7 +427,9 @@ public:
     const unsigned vec = in.channels % 8 == 0 ? 8 : 1;
     auto k = m_compiler->read("slice.hip");
     k.define("CH", in.channels); k.define("VEC", vec);
-    auto d = impl.registerDispatch(k, "memory_slice", linearGrid(sym, out.width, out.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
+    const std::string entry = "memory_slice_c" + std::to_string(in.channels) + "v" + std::to_string(vec);
+    k.define("KERNEL_NAME", entry);
+    auto d = impl.registerDispatch(k, entry, linearGrid(sym, out.width, out.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     d.addBinding(dnx::Access::WriteOnly, m.output);
     d.addPushConstant(op.top); d.addPushConstant(op.left);

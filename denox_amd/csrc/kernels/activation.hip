@@ -6,6 +6,10 @@
 #ifndef ALPHA
 #define ALPHA 0.0f
 #endif
+// The entry point is named per variant (KERNEL_NAME) so that profilers tell variants apart.
+#ifndef KERNEL_NAME
+#define KERNEL_NAME activation
+#endif
 struct PushConstants { unsigned int W, H; };
 __device__ DNX_INLINE _Float16 act1(_Float16 v) {
 #if ACT == 1
@@ -15,7 +19,7 @@ __device__ DNX_INLINE _Float16 act1(_Float16 v) {
   return v > av ? v : av;
 #endif
 }
-extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void activation(
+extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
     const ushort_t *__restrict__ IN, ushort_t *__restrict__ OUT, PushConstants pc) {
   constexpr unsigned CV = CH / VEC;
   const unsigned long long idx = (unsigned long long)DNX_BID_X * WG + DNX_TID;

@@ -56,6 +56,10 @@ typedef unsigned short ushort_t;
 #define NT (WAVES * 64)
 #define KOUTP (((KOUT) + 31) / 32 * 32)
 
+// The entry point is named per variant (KERNEL_NAME) so that profilers tell variants apart.
+#ifndef KERNEL_NAME
+#define KERNEL_NAME conv3x3_mfma
+#endif
 struct PushConstants {
   unsigned int IN_W;
   unsigned int IN_H;
@@ -215,7 +219,7 @@ __device__ DNX_INLINE ushort_t dpp_xor1(ushort_t v) {
   return (ushort_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xF, 0xF, true);
 }
 
-extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void conv3x3_mfma(
+extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     const _Float16 *__restrict__ A,
 #if CB > 0
     const _Float16 *__restrict__ B,

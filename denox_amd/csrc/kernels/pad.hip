@@ -3,8 +3,12 @@
 //   out[ho, wo, c] = in[clamp(ho - PAD_T, 0, IN_H-1), clamp(wo - PAD_L, 0, IN_W-1), c].
 // Definitions: CH, VEC.
 #include "common.h"
+// The entry point is named per variant (KERNEL_NAME) so that profilers tell variants apart.
+#ifndef KERNEL_NAME
+#define KERNEL_NAME memory_pad
+#endif
 struct PushConstants { unsigned int OUT_W, OUT_H, PAD_L, PAD_R, PAD_T, PAD_B; };
-extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void memory_pad(
+extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
     const ushort_t *__restrict__ IN, ushort_t *__restrict__ OUT, PushConstants pc) {
   constexpr unsigned CV = CH / VEC;
   const unsigned long long idx = (unsigned long long)DNX_BID_X * WG + DNX_TID;

@@ -4,8 +4,12 @@
 //   output extent floor(H/KY) x floor(W/KX).
 // Definitions: CH, KX, KY, VEC.  One thread per output vector.
 #include "common.h"
+// The entry point is named per variant (KERNEL_NAME) so that profilers tell variants apart.
+#ifndef KERNEL_NAME
+#define KERNEL_NAME pool_max
+#endif
 struct PushConstants { unsigned int W, H; };
-extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void pool_max(
+extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
     const ushort_t *__restrict__ IN, ushort_t *__restrict__ OUT, PushConstants pc) {
   constexpr unsigned CV = CH / VEC;
   const unsigned W2 = pc.W / KX, H2 = pc.H / KY;

@@ -10,13 +10,17 @@ typedef unsigned short ushort_t;
 #ifndef WG
 #define WG 256
 #endif
+// The entry point is named per variant (KERNEL_NAME) so that profilers tell variants apart.
+#ifndef KERNEL_NAME
+#define KERNEL_NAME relayout
+#endif
 struct PushConstants { unsigned int W, H; };
 __device__ DNX_INLINE size_t lidx(int layout, size_t HW, size_t pix, unsigned c) {
   if (layout == 0) return pix * CH + c;
   if (layout == 1) return (size_t)c * HW + pix;
   return (size_t)(c >> 3) * (HW * 8) + pix * 8 + (c & 7);
 }
-extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void relayout(
+extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
     const ushort_t *__restrict__ IN, ushort_t *__restrict__ OUT, PushConstants pc) {
   const size_t HW = (size_t)pc.W * pc.H;
   const size_t pix = (size_t)DNX_BID_X * WG + DNX_TID;

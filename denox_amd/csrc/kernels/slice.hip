@@ -3,8 +3,12 @@
 //   out[h, w, c] = in[h + IN_TOP, w + IN_LEFT, c].
 // Definitions: CH, VEC.
 #include "common.h"
+// The entry point is named per variant (KERNEL_NAME) so that profilers tell variants apart.
+#ifndef KERNEL_NAME
+#define KERNEL_NAME memory_slice
+#endif
 struct PushConstants { unsigned int IN_TOP, IN_LEFT, IN_W, IN_H, OUT_W, OUT_H; };
-extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void memory_slice(
+extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
     const ushort_t *__restrict__ IN, ushort_t *__restrict__ OUT, PushConstants pc) {
   constexpr unsigned CV = CH / VEC;
   const unsigned long long idx = (unsigned long long)DNX_BID_X * WG + DNX_TID;

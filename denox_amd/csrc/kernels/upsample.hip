@@ -4,8 +4,12 @@
 // Definitions: CH, SCALE, VEC.  One thread per *input* vector; it writes the
 // SCALE x SCALE replicas, so every input byte is fetched once.
 #include "common.h"
+// The entry point is named per variant (KERNEL_NAME) so that profilers tell variants apart.
+#ifndef KERNEL_NAME
+#define KERNEL_NAME upsample_nearest
+#endif
 struct PushConstants { unsigned int W, H; }; // input extent
-extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void upsample_nearest(
+extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
     const ushort_t *__restrict__ IN, ushort_t *__restrict__ OUT, PushConstants pc) {
   constexpr unsigned CV = CH / VEC;
   const unsigned long long idx = (unsigned long long)DNX_BID_X * WG + DNX_TID;

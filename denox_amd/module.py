@@ -148,6 +148,8 @@ class Db:
     def populate(self, model: Model, **kw) -> int:
         o, _keep = _options(kw.get("features"), kw.get("input_layout", Layout.HWC), kw.get("output_layout", Layout.HWC),
                             kw.get("assume"), kw.get("conv_config"), kw.get("device", -1))
+        o.populate_compile_kernels = int(kw.get("compile_kernels", True))
+        o.kernel_shard_index, o.kernel_shard_count = kw.get("shard", (0, 1))
         n = c_uint64()
         _capi.check(_capi.lib().denox_hip_db_populate(self._h, model._h, byref(o), byref(n)))
         return n.value

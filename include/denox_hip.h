@@ -129,6 +129,12 @@ typedef struct denox_hip_compile_options {
   const int64_t *assumption_values;
   const char *force_conv_config;     /* NULL / "" = choose; else one named conv configuration */
   int32_t device;                    /* >= 0: prune configurations with that device's limits; < 0: CDNA4 table */
+  /* denox_hip_db_populate only: compile every candidate kernel into the code-object cache
+   * (compiler/src/denox/compiler/populate.cpp:70-99); shard index/count let several processes
+   * split that work (this call compiles the kernels whose ordinal % count == index). */
+  int32_t populate_compile_kernels;
+  uint32_t kernel_shard_index;
+  uint32_t kernel_shard_count;
 } denox_hip_compile_options;
 void denox_hip_compile_options_default(denox_hip_compile_options *opt);
 /* db may be NULL (roofline estimates drive the selection).  The blob is
