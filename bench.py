@@ -93,6 +93,8 @@ def main() -> int:
         db.bench(min_samples=10, max_relative_error=0.03, max_samples=50, save_progress=bool(args.db))
         tune_s = time.perf_counter() - t0
     blob = dx.compile_model(model, assume={"H": H, "W": W}, conv_config=args.conv_config, db=db)
+    if args.per_dispatch:
+        print(dx.last_compile_report(), file=sys.stderr)
     mod = dx.Module.load(blob)
     inst = mod.instance(H=H, W=W)
 

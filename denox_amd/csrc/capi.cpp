@@ -76,6 +76,8 @@ compiler::CompileOptions toOptions(const denox_hip_compile_options *o) {
   opt.features.enableConcatConvFusion = o->enable_concat_conv_fusion != 0;
   opt.features.enableUpsampleFusion = o->enable_upsample_fusion != 0;
   opt.features.enablePoolFusion = o->enable_pool_fusion != 0;
+  opt.features.enablePadFusion = o->enable_pad_fusion != 0;
+  opt.features.enableSliceFusion = o->enable_slice_fusion != 0;
   auto fmt = [](int f) {
     switch (f) {
     case 0: case DENOX_HIP_FORMAT_HWC: return dnx::TensorFormat::SSBO_HWC;
@@ -200,6 +202,7 @@ void denox_hip_compile_options_default(denox_hip_compile_options *o) {
   if (!o) return;
   std::memset(o, 0, sizeof(*o));
   o->enable_conv_relu_fusion = o->enable_concat_conv_fusion = o->enable_upsample_fusion = o->enable_pool_fusion = 1;
+  o->enable_pad_fusion = o->enable_slice_fusion = 1;
   o->device = -1;
   o->populate_compile_kernels = 1;
   o->kernel_shard_index = 0;

@@ -15,6 +15,8 @@ struct Features {
   bool enableConcatConvFusion = true; // conv reads its two concat sources      (reference: ConcatConvCMShader)
   bool enableUpsampleFusion = true;   // conv reads a half-resolution source at (y/2, x/2)
   bool enablePoolFusion = true;       // conv stores the 2x2 max only
+  bool enablePadFusion = true;        // conv reads an un-padded source through the replicate clamp
+  bool enableSliceFusion = true;      // conv stores only the cropped window
   bool enableImplicitConcat = true;   // memory-aliasing concat where layouts allow it
 };
 

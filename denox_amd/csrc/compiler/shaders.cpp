@@ -38,44 +38,55 @@ std::string fmtFloat(float v) {
 }
 
 // ------------------------------------------------------------------ conv
-struct ConvConfig { unsigned waves, rpw, ck; const char *name; };
+// Two kernel sources share one configuration table: conv3x3_mfma.hip streams the
+// weight slice of every reduction step through LDS (any layer size), conv3x3_mfma_ws.hip
+// keeps the whole slice resident and runs persistently (layers whose weights fit LDS).
+struct ConvConfig { unsigned waves, rpw, ck; bool resident; const char *name; };
 const ConvConfig kConvConfigs[] = {
-    {4, 2, 16, "w4r2k16"}, {4, 2, 32, "w4r2k32"}, {4, 4, 16, "w4r4k16"}, {4, 4, 32, "w4r4k32"},
-    {8, 2, 16, "w8r2k16"}, {8, 2, 32, "w8r2k32"}, {4, 2, 64, "w4r2k64"}, {8, 1, 16, "w8r1k16"},
+    {4, 2, 16, false, "w4r2k16"}, {4, 2, 32, false, "w4r2k32"}, {4, 4, 16, false, "w4r4k16"}, {4, 4, 32, false, "w4r4k32"},
+    {8, 2, 16, false, "w8r2k16"}, {8, 2, 32, false, "w8r2k32"}, {4, 2, 64, false, "w4r2k64"}, {8, 1, 16, false, "w8r1k16"},
+    {8, 1, 16, true, "p8r1k16"},  {8, 1, 32, true, "p8r1k32"},  {16, 1, 16, true, "p16r1k16"}, {16, 1, 32, true, "p16r1k32"},
+    {8, 2, 16, true, "p8r2k16"},  {8, 2, 32, true, "p8r2k32"},  {16, 2, 16, true, "p16r2k16"}, {4, 2, 32, true, "p4r2k32"},
 };
 constexpr unsigned kNumConvConfigs = sizeof(kConvConfigs) / sizeof(kConvConfigs[0]);
 
-enum ConvPatternBits : unsigned { PAT_CONCAT = 1, PAT_UPSAMPLE = 2, PAT_ACT = 4, PAT_POOL = 8 };
+enum ConvPatternBits : unsigned { PAT_CONCAT = 1, PAT_UPSAMPLE = 2, PAT_ACT = 4, PAT_POOL = 8, PAT_PADA = 16, PAT_PADB = 32, PAT_CROP = 64 };
 
 struct ConvGeometry {
-  unsigned CA, CB, C, CPAD, K, KOUTP, KT;
+  unsigned CA, CB, C, CPAD, K, KOUTP, KT, slots;
   size_t ldsBytes;
 };
 
 // Output channels per workgroup: the largest divisor of KOUTP (in blocks of 32)
-// whose weight slice fits LDS next to the halo and whose accumulators fit the
+// whose weights fit LDS next to the halo(s) and whose accumulators fit the
 // register file.
-bool chooseKT(const ConvConfig &cfg, unsigned CA, unsigned CB, unsigned K, unsigned ldsLimit, ConvGeometry &g) {
+bool chooseKT(const ConvConfig &cfg, unsigned CA, unsigned CB, unsigned K, const DeviceInfo &dev, ConvGeometry &g) {
   g.CA = CA; g.CB = CB; g.C = CA + CB; g.CPAD = (g.C + 15) / 16 * 16; g.K = K; g.KOUTP = (K + 31) / 32 * 32;
   const unsigned th = cfg.waves * cfg.rpw;
   const unsigned haloPix = (th + 2) * 34;
   const unsigned ckp = cfg.ck + 8;
   const unsigned blocks = g.KOUTP / 32;
+  // registers per lane: 512 shared by the waves of one SIMD; a workgroup of `waves` waves puts waves/4 on each
+  const unsigned regBudget = cfg.waves >= 16 ? 128 : 256;
   for (unsigned kb = blocks; kb >= 1; --kb) {
     if (blocks % kb) continue;
-    if (kb * cfg.rpw > 8) continue; // <= 128 accumulator registers per lane
-    const size_t lds = (static_cast<size_t>(haloPix) + 9u * kb * 32u) * ckp * 2u;
-    if (lds > ldsLimit) continue;
+    if (kb * cfg.rpw * 16 + 64 > regBudget) continue;
+    const size_t lds = cfg.resident ? static_cast<size_t>(9u * kb * 32u) * (g.CPAD + 8) * 2u + 2u * static_cast<size_t>(haloPix) * ckp * 2u
+                                    : (static_cast<size_t>(haloPix) + 9u * kb * 32u) * ckp * 2u;
+    if (lds > dev.maxComputeSharedMemory) continue;
     g.KT = kb * 32;
     g.ldsBytes = lds;
+    const unsigned nkt = blocks / kb;
+    g.slots = std::max(1u, dev.computeUnits / (dev.xcdCount * nkt));
     return true;
   }
   return false;
 }
 
-// Weight layout the kernel reads: [kt][chunk][tap r*3+s][KT rows][len(chunk)], rows
+// Weight layout the kernels read: [kt][chunk][tap r*3+s][KT rows][len(chunk)], rows
 // permuted so that MFMA row rho of a 32-block holds output channel
 // 16*((rho>>2)&1) + 4*(rho>>3) + (rho&3) of that block; zero for c >= C or k >= K.
+// (The resident kernel uses one chunk spanning the whole reduction.)
 std::vector<uint8_t> packConvWeights(const Op &conv, const ConvGeometry &g, unsigned ck) {
   std::vector<uint16_t> out(static_cast<size_t>(g.KOUTP) * 9 * g.CPAD, 0);
   const unsigned nkt = g.KOUTP / g.KT;
@@ -105,6 +116,20 @@ public:
   explicit ConvMfmaShader(const hip::HipCompiler *c) : m_compiler(c) {}
   std::string name() const override { return "conv3x3_mfma"; }
 
+  // A source of the conv after looking through one optional upsample or pad.
+  struct Source { unsigned bits; std::vector<int> ops; int tensor; };
+  static std::vector<Source> sourcesOf(const Model &model, TensorHandle t, bool allowUpsample, unsigned padBit, const CompileOptions &opt) {
+    std::vector<Source> out;
+    out.push_back(Source{0, {}, t});
+    const int prod = model.tensors()[t].producer;
+    if (prod >= 0) {
+      const Op &p = model.ops()[prod];
+      if (allowUpsample && p.kind == OpKind::Upsample && p.scale == 2 && opt.features.enableUpsampleFusion) out.push_back(Source{PAT_UPSAMPLE, {prod}, p.inputs[0]});
+      if (p.kind == OpKind::Pad && opt.features.enablePadFusion) out.push_back(Source{padBit, {prod}, p.inputs[0]});
+    }
+    return out;
+  }
+
   std::vector<Match> matchAll(const Model &model, const CompileOptions &opt) const override {
     std::vector<Match> out;
     const auto &ops = model.ops();
@@ -112,38 +137,40 @@ public:
       const Op &conv = ops[i];
       if (conv.kind != OpKind::Conv) continue;
       if (conv.R != 3 || conv.S != 3 || conv.strideX != 1 || conv.strideY != 1 || conv.padX != 1 || conv.padY != 1 || conv.dilX != 1 || conv.dilY != 1) continue;
+      // A fused-away tensor may have other consumers: whoever needs it materialised gets it
+      // from another edge, and the selection weighs both.
       struct Pro { unsigned bits; std::vector<int> ops; std::vector<int> inputs; };
       std::vector<Pro> pros;
       const TensorHandle in = conv.inputs[0];
-      pros.push_back(Pro{0, {}, {in}});
+      for (const Source &s : sourcesOf(model, in, true, PAT_PADA, opt)) pros.push_back(Pro{s.bits, s.ops, {s.tensor}});
       const int prod = model.tensors()[in].producer;
-      if (prod >= 0 && singleUse(model, in)) {
-        const Op &p = ops[prod];
-        if (p.kind == OpKind::Concat && opt.features.enableConcatConvFusion) {
-          pros.push_back(Pro{PAT_CONCAT, {prod}, {p.inputs[0], p.inputs[1]}});
-          const TensorHandle a = p.inputs[0];
-          const int ap = model.tensors()[a].producer;
-          if (ap >= 0 && singleUse(model, a) && ops[ap].kind == OpKind::Upsample && ops[ap].scale == 2 && opt.features.enableUpsampleFusion)
-            pros.push_back(Pro{PAT_CONCAT | PAT_UPSAMPLE, {ap, prod}, {ops[ap].inputs[0], p.inputs[1]}});
-        } else if (p.kind == OpKind::Upsample && p.scale == 2 && opt.features.enableUpsampleFusion) {
-          pros.push_back(Pro{PAT_UPSAMPLE, {prod}, {p.inputs[0]}});
-        }
+      if (prod >= 0 && ops[prod].kind == OpKind::Concat && opt.features.enableConcatConvFusion) {
+        const Op &cat = ops[prod];
+        for (const Source &a : sourcesOf(model, cat.inputs[0], true, PAT_PADA, opt))
+          for (const Source &b : sourcesOf(model, cat.inputs[1], false, PAT_PADB, opt)) {
+            if ((a.bits & PAT_PADA) && (b.bits & PAT_PADB)) continue; // one padded source per dispatch
+            Pro p{PAT_CONCAT | a.bits | b.bits, a.ops, {a.tensor, b.tensor}};
+            p.ops.insert(p.ops.end(), b.ops.begin(), b.ops.end());
+            p.ops.push_back(prod);
+            pros.push_back(std::move(p));
+          }
       }
       struct Epi { unsigned bits; std::vector<int> ops; int output; };
       std::vector<Epi> epis;
       epis.push_back(Epi{0, {}, conv.output});
       auto poolOk = [](const Op &q) { return q.kind == OpKind::Pool && q.kernelX == 2 && q.kernelY == 2 && q.poolStrideX == 2 && q.poolStrideY == 2 && q.poolPadX == 0 && q.poolPadY == 0; };
+      auto tails = [&](TensorHandle t, unsigned bits, std::vector<int> chain) {
+        if (!singleUse(model, t)) return;
+        const int c = model.tensors()[t].consumers[0];
+        if (poolOk(ops[c]) && opt.features.enablePoolFusion) { auto ch = chain; ch.push_back(c); epis.push_back(Epi{bits | PAT_POOL, ch, ops[c].output}); }
+        if (ops[c].kind == OpKind::Slice && opt.features.enableSliceFusion) { auto ch = chain; ch.push_back(c); epis.push_back(Epi{bits | PAT_CROP, ch, ops[c].output}); }
+      };
+      tails(conv.output, 0, {});
       if (singleUse(model, conv.output)) {
         const int c1 = model.tensors()[conv.output].consumers[0];
-        const Op &n1 = ops[c1];
-        if (n1.kind == OpKind::Activation && opt.features.enableConvReluFusion) {
-          epis.push_back(Epi{PAT_ACT, {c1}, n1.output});
-          if (singleUse(model, n1.output)) {
-            const int c2 = model.tensors()[n1.output].consumers[0];
-            if (poolOk(ops[c2]) && opt.features.enablePoolFusion) epis.push_back(Epi{PAT_ACT | PAT_POOL, {c1, c2}, ops[c2].output});
-          }
-        } else if (poolOk(n1) && opt.features.enablePoolFusion) {
-          epis.push_back(Epi{PAT_POOL, {c1}, n1.output});
+        if (ops[c1].kind == OpKind::Activation && opt.features.enableConvReluFusion) {
+          epis.push_back(Epi{PAT_ACT, {c1}, ops[c1].output});
+          tails(ops[c1].output, PAT_ACT, {c1});
         }
       }
       for (const auto &p : pros)
@@ -161,13 +188,13 @@ public:
     return out;
   }
 
-  const Op &convOf(const Model &model, const Match &m) const {
-    for (int o : m.ops) if (model.ops()[o].kind == OpKind::Conv) return model.ops()[o];
-    fail(Status::Internal, "conv match without conv");
+  const Op &opOf(const Model &model, const Match &m, OpKind kind) const {
+    for (int o : m.ops) if (model.ops()[o].kind == kind) return model.ops()[o];
+    fail(Status::Internal, "conv match lacks an expected operation");
   }
 
   std::vector<unsigned> acceptMatch(const Model &model, const Match &m, const CompileOptions &opt) const override {
-    const Op &conv = convOf(model, m);
+    const Op &conv = opOf(model, m, OpKind::Conv);
     const unsigned CA = model.tensors()[m.inputs[0]].channels;
     const unsigned CB = m.inputs.size() > 1 ? model.tensors()[m.inputs[1]].channels : 0;
     const unsigned cpad = (CA + CB + 15) / 16 * 16;
@@ -179,58 +206,62 @@ public:
       if ((m.pattern & PAT_POOL) && (cfg.rpw % 2)) continue;
       if (cfg.waves * 64 > opt.deviceInfo.maxComputeWorkGroupInvocations) continue;
       ConvGeometry g;
-      if (!chooseKT(cfg, CA, CB, conv.K, ldsLimit(opt), g)) continue;
+      if (!chooseKT(cfg, CA, CB, conv.K, opt.deviceInfo, g)) continue;
       out.push_back(c);
     }
     if (out.empty() && !opt.forceConvConfig.empty()) fail(Status::Unsupported, "conv configuration '" + opt.forceConvConfig + "' is not valid for this layer");
     return out;
   }
 
-  static unsigned ldsLimit(const CompileOptions &opt) { return opt.deviceInfo.maxComputeSharedMemory; }
-
   size_t parameterMemorySize(const Model &model, const Match &m) const override {
-    const Op &conv = convOf(model, m);
+    const Op &conv = opOf(model, m, OpKind::Conv);
     const unsigned C = conv.C, cpad = (C + 15) / 16 * 16, kp = (conv.K + 31) / 32 * 32;
     return static_cast<size_t>(kp) * 9 * cpad * 2 + static_cast<size_t>(kp) * 2;
   }
 
   void implement(OpImpl &impl, const Model &model, const Match &m, unsigned config, SymGraph &sym, const CompileOptions &opt) const override {
     const ConvConfig &cfg = kConvConfigs[config];
-    const Op &conv = convOf(model, m);
+    const Op &conv = opOf(model, m, OpKind::Conv);
     const TensorNode &convIn = model.tensors()[conv.inputs[0]];
     const TensorNode &tA = model.tensors()[m.inputs[0]];
     const unsigned CA = tA.channels;
     const unsigned CB = m.inputs.size() > 1 ? model.tensors()[m.inputs[1]].channels : 0;
     ConvGeometry g;
-    if (!chooseKT(cfg, CA, CB, conv.K, ldsLimit(opt), g)) fail(Status::Internal, "conv config rejected at implement time");
+    if (!chooseKT(cfg, CA, CB, conv.K, opt.deviceInfo, g)) fail(Status::Internal, "conv config rejected at implement time");
     int act = 0;
     float alpha = 0.0f;
-    for (int o : m.ops)
-      if (model.ops()[o].kind == OpKind::Activation) {
-        act = model.ops()[o].func == ActivationFunction::ReLU ? 1 : 2;
-        alpha = model.ops()[o].alpha;
-      }
-    const bool pool = (m.pattern & PAT_POOL) != 0, up = (m.pattern & PAT_UPSAMPLE) != 0;
+    if (m.pattern & PAT_ACT) {
+      const Op &a = opOf(model, m, OpKind::Activation);
+      act = a.func == ActivationFunction::ReLU ? 1 : 2;
+      alpha = a.alpha;
+    }
+    const bool pool = (m.pattern & PAT_POOL) != 0, up = (m.pattern & PAT_UPSAMPLE) != 0, crop = (m.pattern & PAT_CROP) != 0;
+    const bool padA = (m.pattern & PAT_PADA) != 0, padB = (m.pattern & PAT_PADB) != 0;
 
-    hip::HipCompilerInstance k = m_compiler->read("conv3x3_mfma.hip");
+    hip::HipCompilerInstance k = m_compiler->read(cfg.resident ? "conv3x3_mfma_ws.hip" : "conv3x3_mfma.hip");
     k.define("CA", CA); k.define("CB", CB); k.define("UPA", up ? 1 : 0);
     k.define("KOUT", conv.K); k.define("KT", g.KT);
     k.define("ACT", act);
     if (act == 2) k.define("ALPHA", fmtFloat(alpha));
     k.define("POOL", pool ? 1 : 0); k.define("HAS_BIAS", conv.hasBias ? 1 : 0);
+    if (padA) k.define("PADA", 1);
+    if (padB) k.define("PADB", 1);
+    if (crop) k.define("CROP", 1);
     k.define("WAVES", cfg.waves); k.define("RPW", cfg.rpw); k.define("CK", cfg.ck);
-
-    std::string entry = "conv3x3_c" + std::to_string(CA) + (up ? "u" : "") + (CB ? "p" + std::to_string(CB) : "") + "_k" + std::to_string(conv.K) +
-                        (act == 1 ? "_relu" : act == 2 ? "_lrelu" : "") + (pool ? "_pool" : "") + "_" + cfg.name;
+    if (cfg.resident) k.define("SLOTS", g.slots);
+    std::string entry = "conv3x3_c" + std::to_string(CA) + (up ? "u" : "") + (padA ? "e" : "") + (CB ? "p" + std::to_string(CB) + (padB ? "e" : "") : "") + "_k" +
+                        std::to_string(conv.K) + (act == 1 ? "_relu" : act == 2 ? "_lrelu" : "") + (pool ? "_pool" : "") + (crop ? "_crop" : "") + "_" + cfg.name;
     k.define("KERNEL_NAME", entry);
     const Sym W = convIn.width, H = convIn.height;
     const unsigned th = cfg.waves * cfg.rpw;
-    auto d = impl.registerDispatch(k, entry, sym.cdiv(W, 32), sym.cdiv(H, th), Sym::Const(g.KOUTP / g.KT), cfg.waves * 64);
+    const unsigned nkt = g.KOUTP / g.KT;
+    auto d = cfg.resident ? impl.registerDispatch(k, entry, Sym::Const(opt.deviceInfo.xcdCount * nkt * g.slots), Sym::Const(1), Sym::Const(1), cfg.waves * 64)
+                          : impl.registerDispatch(k, entry, sym.cdiv(W, 32), sym.cdiv(H, th), Sym::Const(nkt), cfg.waves * 64);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     if (CB) d.addBinding(dnx::Access::ReadOnly, m.inputs[1]);
     d.addBinding(dnx::Access::WriteOnly, m.output);
     const Op convCopy = conv; // the lazy packers outlive the model reference
-    const unsigned ck = cfg.ck;
+    const unsigned ck = cfg.resident ? g.CPAD : cfg.ck;
     TensorId wt = impl.createParameter(static_cast<size_t>(g.KOUTP) * 9 * g.CPAD * 2, dnx::ScalarType::F16,
                                        [convCopy, g, ck]() { return packConvWeights(convCopy, g, ck); });
     d.addParamBinding(wt);
@@ -245,17 +276,29 @@ public:
     }
     d.addPushConstant(W, dnx::ScalarType::U32);
     d.addPushConstant(H, dnx::ScalarType::U32);
+    if (padA || padB) {
+      const Op &pad = opOf(model, m, OpKind::Pad);
+      const TensorNode &src = model.tensors()[pad.inputs[0]];
+      d.addPushConstant(src.width); d.addPushConstant(src.height); d.addPushConstant(pad.left); d.addPushConstant(pad.top);
+    }
+    if (crop) {
+      const Op &sl = opOf(model, m, OpKind::Slice);
+      const TensorNode &o = model.tensors()[m.output];
+      d.addPushConstant(o.width); d.addPushConstant(o.height); d.addPushConstant(sl.left); d.addPushConstant(sl.top);
+    }
 
     std::string nm = "conv3x3";
     if (up) nm = "upsample+" + nm;
+    if (padA || padB) nm = "pad+" + nm;
     if (m.pattern & PAT_CONCAT) nm = "concat+" + nm;
     if (act == 1) nm += "+relu"; else if (act == 2) nm += "+leaky_relu";
     if (pool) nm += "+maxpool";
+    if (crop) nm += "+slice";
     d.setName(nm);
     d.setOperation(nm);
     d.setConfig(std::string(cfg.name) + "/kt" + std::to_string(g.KT));
     impl.edge().config = cfg.name;
-    // bytes that cross HBM: sources at their stored resolution, weights, bias; the (pooled) output
+    // bytes that cross HBM: sources at their stored resolution, weights, bias; the (pooled / cropped) output
     Sym reads = bytesOf(sym, tA);
     if (CB) reads = sym.add(reads, bytesOf(sym, model.tensors()[m.inputs[1]]));
     reads = sym.add(reads, static_cast<int64_t>(conv.K) * conv.C * 9 * 2 + (conv.hasBias ? conv.K * 2 : 0));

@@ -1,0 +1,270 @@
+// Shared pieces of the conv3x3 MFMA kernels: the compile-time interface, the
+// source loader (concat / upsample / replicate-pad folded into the addressing)
+// and the epilogue (bias, activation, rounding, 2x2 max pool or crop, store).
+//
+//   out[y,x,k] = act(bias[k] + sum_{r,s,c} src[y+r-1, x+s-1, c] * W[k,c,r,s])       (zero outside the image)
+//   src[y,x,c] = c < CA ? A'[y,x,c] : B'[y,x,c-CA]
+//   A' = UPA ? A[y/2, x/2] : (PADA ? A[clamp(y-PAD_T), clamp(x-PAD_L)] : A[y,x]),   B' likewise with PADB
+//
+// Definitions every variant is compiled with:
+//   CA, CB      channels of source A / source B (CB = 0: single source)
+//   UPA         1: A is stored at half resolution and read at (y>>1, x>>1)
+//   PADA, PADB  1: that source is stored un-padded (SRC_H x SRC_W) and read through a
+//               replicate pad with offsets (PAD_T, PAD_L); IN_H x IN_W is the padded extent
+//   KOUT        output channels;  KT: output channels per workgroup (multiple of 32)
+//   ACT         0 none, 1 ReLU, 2 LeakyReLU(ALPHA);   HAS_BIAS 0/1
+//   POOL        1: store max over 2x2 output windows at (y/2, x/2) only
+//   CROP        1: store only rows/cols inside [CROP_T, CROP_T+OUT_H) x [CROP_L, CROP_L+OUT_W)
+//   WAVES, RPW  waves per workgroup, output rows per wave -> tile = (WAVES*RPW) x 32 pixels
+//   CK          input channels staged in LDS per step (multiple of 16)
+//
+// Mapping onto v_mfma_f32_32x32x16_f16: the weights are the M operand (32 output
+// channels per block, rows permuted so that each lane ends up with 16 consecutive
+// channels), 32 consecutive pixels of one image row are the N operand, and the
+// reduction runs over (tap, input channel) in steps of 16 channels.
+#include "prelude.h"
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
+typedef unsigned short ushort_t;
+
+#ifndef ALPHA
+#define ALPHA 0.0f
+#endif
+#ifndef PADA
+#define PADA 0
+#endif
+#ifndef PADB
+#define PADB 0
+#endif
+#ifndef CROP
+#define CROP 0
+#endif
+
+#define CIN (CA + CB)
+#define CPAD (((CIN) + 15) / 16 * 16)
+#define NCHUNK ((CPAD + CK - 1) / CK)
+#define TAIL (CPAD - (NCHUNK - 1) * CK)
+#define TW 32
+#define TH (WAVES * RPW)
+#define HALO_W (TW + 2)
+#define HALO_H (TH + 2)
+#define HALO_PIX (HALO_W * HALO_H)
+#define CKP (CK + 8)
+#define KB (KT / 32)
+#define NT (WAVES * 64)
+#define KOUTP (((KOUT) + 31) / 32 * 32)
+
+struct PushConstants {
+  unsigned int IN_W;
+  unsigned int IN_H;
+#if PADA || PADB
+  unsigned int SRC_W, SRC_H, PAD_L, PAD_T;
+#endif
+#if CROP
+  unsigned int OUT_W, OUT_H, CROP_L, CROP_T;
+#endif
+};
+
+__device__ DNX_INLINE uint4v ld16(const _Float16 *p) {
+  return *reinterpret_cast<const uint4v *>(p);
+}
+
+__device__ DNX_INLINE int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+// Element offsets of full-resolution pixel (gy, gx) inside A and B.
+__device__ DNX_INLINE void src_offsets(int gy, int gx, const PushConstants &pc, size_t &pa, size_t &pb) {
+  const unsigned W = pc.IN_W;
+#if PADA
+  const int ay = clampi(gy - (int)pc.PAD_T, 0, (int)pc.SRC_H - 1), ax = clampi(gx - (int)pc.PAD_L, 0, (int)pc.SRC_W - 1);
+  const unsigned WA = pc.SRC_W;
+#else
+  const int ay = UPA ? (gy >> 1) : gy, ax = UPA ? (gx >> 1) : gx;
+  const unsigned WA = UPA ? (W >> 1) : W;
+#endif
+#if PADB
+  const int by = clampi(gy - (int)pc.PAD_T, 0, (int)pc.SRC_H - 1), bx = clampi(gx - (int)pc.PAD_L, 0, (int)pc.SRC_W - 1);
+  const unsigned WB = pc.SRC_W;
+#else
+  const int by = gy, bx = gx;
+  const unsigned WB = W;
+#endif
+  pa = ((size_t)ay * WA + (size_t)ax) * CA;
+  pb = ((size_t)by * WB + (size_t)bx) * (CB > 0 ? CB : 1);
+}
+
+// Eight consecutive channels [cc, cc+8) of the concatenated source at the pixel whose
+// element offsets are (pa, pb); channels past CIN read as zero.
+__device__ DNX_INLINE uint4v
+load_src8(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, size_t pa, size_t pb, int cc) {
+  if ((CA % 8 == 0) && (CB % 8 == 0)) {
+    if (cc < CA)
+      return ld16(A + pa + cc);
+    if (CB > 0 && cc < CIN)
+      return ld16(B + pb + (cc - CA));
+    return uint4v{0u, 0u, 0u, 0u};
+  } else {
+    if ((CA % 8 == 0) && cc + 8 <= CA)
+      return ld16(A + pa + cc);
+    half8 v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int ch = cc + e;
+      _Float16 x = (_Float16)0.0f;
+      if (ch < CA)
+        x = A[pa + ch];
+      else if (CB > 0 && ch < CIN)
+        x = B[pb + (ch - CA)];
+      v[e] = x;
+    }
+    return __builtin_bit_cast(uint4v, v);
+  }
+}
+
+// Halo vector i of a chunk of L channels starting at c0, for the tile at (y0, x0).
+template <int L>
+__device__ DNX_INLINE uint4v
+load_halo_vec(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, int i, int c0, int y0, int x0, const PushConstants &pc) {
+  constexpr int VPP = L / 8; // 16-byte vectors per pixel
+  const int pix = i / VPP;
+  const int v = i - pix * VPP;
+  const int hy = pix / HALO_W;
+  const int hx = pix - hy * HALO_W;
+  const int gy = y0 + hy - 1;
+  const int gx = x0 + hx - 1;
+  uint4v val = {0u, 0u, 0u, 0u};
+  if (gy >= 0 && gy < (int)pc.IN_H && gx >= 0 && gx < (int)pc.IN_W) {
+    size_t pa, pb;
+    src_offsets(gy, gx, pc, pa, pb);
+    val = load_src8(A, B, pa, pb, c0 + v * 8);
+  }
+  return val;
+}
+
+__device__ DNX_INLINE float apply_act(float v) {
+#if ACT == 1
+  return v > 0.0f ? v : 0.0f;
+#elif ACT == 2
+  const float av = ALPHA * v;
+  return v > av ? v : av;
+#else
+  return v;
+#endif
+}
+
+__device__ DNX_INLINE ushort_t dpp_xor1(ushort_t v) {
+  // quad_perm [1,0,3,2]: exchange with the neighbouring lane
+  return (ushort_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xF, 0xF, true);
+}
+
+__device__ DNX_INLINE void store16(_Float16 *dst, const half8 (&o)[2], int chb) {
+  if (KOUT % 16 == 0) {
+    if (chb < KOUT) {
+      *reinterpret_cast<half8 *>(dst) = o[0];
+      *reinterpret_cast<half8 *>(dst + 8) = o[1];
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      if (chb + i < KOUT)
+        dst[i] = o[i >> 3][i & 7];
+  }
+}
+
+// Epilogue of one wave: acc[kb][j] holds, for output row y0 + wv*RPW + j and pixel
+// x0 + (lane & 31), the 16 channels kt*KT + kb*32 + (lane >> 5)*16 + i.
+__device__ DNX_INLINE void
+store_tile(const float16v (&acc)[KB][RPW], _Float16 *__restrict__ OUT, const _Float16 *__restrict__ BIAS,
+           int y0, int x0, int kt, int wv, int lane, const PushConstants &pc) {
+  const unsigned W = pc.IN_W, H = pc.IN_H;
+  const int l32 = lane & 31;
+  const int hsel = lane >> 5;
+  const int x = x0 + l32;
+#pragma unroll
+  for (int kb = 0; kb < KB; ++kb) {
+    const int chb = kt * KT + kb * 32 + hsel * 16; // first of this lane's 16 channels
+    float bias[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+#if HAS_BIAS
+      bias[i] = (float)BIAS[chb + i]; // the bias buffer is zero-padded to KOUTP
+#else
+      bias[i] = 0.0f;
+#endif
+    }
+#if POOL
+    const unsigned WP = W >> 1, HP = H >> 1;
+#pragma unroll
+    for (int j = 0; j < RPW; j += 2) {
+      const int y = y0 + wv * RPW + j;
+      half8 o[2];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const _Float16 v0 = (_Float16)apply_act(acc[kb][j][i] + bias[i]);
+        const _Float16 v1 = (_Float16)apply_act(acc[kb][j + 1][i] + bias[i]);
+        const _Float16 n0 = __builtin_bit_cast(_Float16, dpp_xor1(__builtin_bit_cast(ushort_t, v0)));
+        const _Float16 n1 = __builtin_bit_cast(_Float16, dpp_xor1(__builtin_bit_cast(ushort_t, v1)));
+        // window order (0,0) (0,1) (1,0) (1,1); replace only on strictly greater
+        _Float16 m = v0;
+        m = n0 > m ? n0 : m;
+        m = v1 > m ? v1 : m;
+        m = n1 > m ? n1 : m;
+        o[i >> 3][i & 7] = m;
+      }
+      const unsigned py = (unsigned)y >> 1, px = (unsigned)x >> 1;
+      if ((l32 & 1) == 0 && py < HP && px < WP)
+        store16(OUT + ((size_t)py * WP + px) * KOUT + chb, o, chb);
+    }
+#else
+#pragma unroll
+    for (int j = 0; j < RPW; ++j) {
+      const int y = y0 + wv * RPW + j;
+      half8 o[2];
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        o[i >> 3][i & 7] = (_Float16)apply_act(acc[kb][j][i] + bias[i]);
+#if CROP
+      const int oy = y - (int)pc.CROP_T, ox = x - (int)pc.CROP_L;
+      if (y < (int)H && x < (int)W && oy >= 0 && oy < (int)pc.OUT_H && ox >= 0 && ox < (int)pc.OUT_W)
+        store16(OUT + ((size_t)oy * pc.OUT_W + ox) * KOUT + chb, o, chb);
+#else
+      if (y < (int)H && x < (int)W)
+        store16(OUT + ((size_t)y * W + x) * KOUT + chb, o, chb);
+#endif
+    }
+#endif
+  }
+}
+
+// 9 taps x (L/16) reduction steps from one staged halo (row pitch CKP halves) and
+// a weight slice whose rows are WPITCH halves apart; `wofs` selects the channel
+// offset of this chunk inside a weight row.
+template <int L, int WPITCH>
+__device__ DNX_INLINE void
+mma_chunk(const _Float16 *sIn, const _Float16 *sW, int wofs, float16v (&acc)[KB][RPW], int wv, int lane) {
+  const int l32 = lane & 31;
+  const int kq = (lane >> 5) * 8;
+#pragma unroll
+  for (int s = 0; s < 3; ++s) {
+#pragma unroll
+    for (int ks = 0; ks < L / 16; ++ks) {
+      const int kk = ks * 16 + kq;
+      half8 px[RPW + 2];
+#pragma unroll
+      for (int hr = 0; hr < RPW + 2; ++hr)
+        px[hr] = *reinterpret_cast<const half8 *>(sIn + ((wv * RPW + hr) * HALO_W + l32 + s) * CKP + kk);
+#pragma unroll
+      for (int r = 0; r < 3; ++r) {
+        half8 wf[KB];
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+          wf[kb] = *reinterpret_cast<const half8 *>(sW + (((r * 3 + s) * KT) + kb * 32 + l32) * WPITCH + wofs + kk);
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+          for (int j = 0; j < RPW; ++j)
+            acc[kb][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[kb], px[j + r], acc[kb][j], 0, 0, 0);
+      }
+    }
+  }
+}

@@ -90,20 +90,29 @@ def test_oidn_unet_schedule_dispatch_geometry_covers_every_pixel():
     for H, W in [(1080, 1920), (1077, 1917), (16, 16), (17, 33)]:
         d = dx.describe(dx.compile_model(m, assume={"H": H, "W": W}), H=H, W=W)
         Hp, Wp = (H + 15) // 16 * 16, (W + 15) // 16 * 16
-        assert d["dispatches"][0]["name"] == "pad" and d["dispatches"][-1]["name"] == "slice"
-        assert d["dispatches"][0]["push_constants"] == [Wp, Hp, 0, Wp - W, 0, Hp - H]
-        assert d["dispatches"][-1]["push_constants"] == [0, 0, Wp, Hp, W, H]
+        # pad and crop fold into the first / last conv: IN extent, then source extent + offsets or crop window
+        assert d["dispatches"][0]["name"] == "pad+conv3x3+relu" and d["dispatches"][-1]["name"] == "conv3x3+slice"
+        assert d["dispatches"][0]["push_constants"] == [Wp, Hp, W, H, 0, 0]
+        assert d["dispatches"][-1]["push_constants"] == [Wp, Hp, W, H, 0, 0]
+        u = dx.describe(dx.compile_model(m, assume={"H": H, "W": W}, features=dict(pad_fusion=False, slice_fusion=False)), H=H, W=W)
+        assert u["dispatches"][0]["name"] == "pad" and u["dispatches"][-1]["name"] == "slice"
+        assert u["dispatches"][0]["push_constants"] == [Wp, Hp, 0, Wp - W, 0, Hp - H]
+        assert u["dispatches"][-1]["push_constants"] == [0, 0, Wp, Hp, W, H]
         convs = [x for x in d["dispatches"] if "conv3x3" in x["name"]]
-        assert len(convs) == 16
+        assert len(convs) == 16 == len(d["dispatches"])
         assert sum(x["flops"] for x in convs) == pytest.approx(523.9e9 * (Hp * Wp) / (1088 * 1920), rel=2e-3)
         for x in convs:
-            w, h = x["push_constants"]
+            w, h = x["push_constants"][:2]
             rows = x["workgroup_size"][0] // 64 * int(re.search(r"RPW=(\d+)", x["debug_info"]).group(1))
             gx, gy, gz = x["workgroup_count"]
-            assert gx == -(-w // 32) and gy == -(-h // rows)
             kt = int(re.search(r"KT=(\d+)", x["debug_info"]).group(1))
             kout = int(re.search(r"KOUT=(\d+)", x["debug_info"]).group(1))
-            assert gz * kt == (kout + 31) // 32 * 32
+            if "SLOTS=" in x["debug_info"]:  # persistent launch: 8 XCDs x channel tiles x slots workgroups
+                slots = int(re.search(r"SLOTS=(\d+)", x["debug_info"]).group(1))
+                assert (gx, gy, gz) == (8 * ((kout + 31) // 32 * 32 // kt) * slots, 1, 1) and gx <= 256
+            else:
+                assert gx == -(-w // 32) and gy == -(-h // rows)
+                assert gz * kt == (kout + 31) // 32 * 32
         out = d["tensors"][d["outputs"][0]]
         assert (out["height"], out["width"], out["channels"]) == (H, W, 3)
 
