@@ -41,12 +41,22 @@ std::string fmtFloat(float v) {
 // Two kernel sources share one configuration table: conv3x3_mfma.hip streams the
 // weight slice of every reduction step through LDS (any layer size), conv3x3_mfma_ws.hip
 // keeps the whole slice resident and runs persistently (layers whose weights fit LDS).
-struct ConvConfig { unsigned waves, rpw, ck; bool resident; const char *name; };
+// waves: computing waves; pw: extra staging-only waves (wave specialisation, resident kernel only)
+struct ConvConfig { unsigned waves, rpw, ck; bool resident; unsigned pw; unsigned maxKT; const char *name; };
 const ConvConfig kConvConfigs[] = {
-    {4, 2, 16, false, "w4r2k16"}, {4, 2, 32, false, "w4r2k32"}, {4, 4, 16, false, "w4r4k16"}, {4, 4, 32, false, "w4r4k32"},
-    {8, 2, 16, false, "w8r2k16"}, {8, 2, 32, false, "w8r2k32"}, {4, 2, 64, false, "w4r2k64"}, {8, 1, 16, false, "w8r1k16"},
-    {8, 1, 16, true, "p8r1k16"},  {8, 1, 32, true, "p8r1k32"},  {16, 1, 16, true, "p16r1k16"}, {16, 1, 32, true, "p16r1k32"},
-    {8, 2, 16, true, "p8r2k16"},  {8, 2, 32, true, "p8r2k32"},  {16, 2, 16, true, "p16r2k16"}, {4, 2, 32, true, "p4r2k32"},
+    // weights streamed per step
+    {4, 2, 16, false, 0, 0, "w4r2k16"}, {4, 2, 32, false, 0, 0, "w4r2k32"}, {4, 4, 16, false, 0, 0, "w4r4k16"}, {4, 4, 32, false, 0, 0, "w4r4k32"},
+    {8, 2, 16, false, 0, 0, "w8r2k16"}, {8, 2, 32, false, 0, 0, "w8r2k32"}, {4, 2, 64, false, 0, 0, "w4r2k64"}, {8, 1, 16, false, 0, 0, "w8r1k16"},
+    // small tiles / one 32-channel block per workgroup: more workgroups for low-resolution layers
+    {4, 1, 16, false, 0, 0, "w4r1k16"}, {4, 1, 32, false, 0, 0, "w4r1k32"}, {4, 1, 32, false, 0, 32, "w4r1k32n"}, {4, 2, 32, false, 0, 32, "w4r2k32n"},
+    {2, 2, 32, false, 0, 32, "w2r2k32n"}, {2, 2, 32, false, 0, 0, "w2r2k32"},
+    // weights resident, persistent launch
+    {8, 1, 16, true, 0, 0, "p8r1k16"},  {8, 1, 32, true, 0, 0, "p8r1k32"},  {16, 1, 16, true, 0, 0, "p16r1k16"}, {16, 1, 32, true, 0, 0, "p16r1k32"},
+    {8, 2, 16, true, 0, 0, "p8r2k16"},  {8, 2, 32, true, 0, 0, "p8r2k32"},  {16, 2, 16, true, 0, 0, "p16r2k16"}, {4, 2, 32, true, 0, 0, "p4r2k32"},
+    {8, 4, 16, true, 0, 0, "p8r4k16"},  {4, 4, 16, true, 0, 0, "p4r4k16"},  {4, 4, 32, true, 0, 0, "p4r4k32"},   {4, 1, 32, true, 0, 0, "p4r1k32"},
+    {4, 2, 32, true, 0, 32, "p4r2k32n"}, {4, 1, 32, true, 0, 32, "p4r1k32n"},
+    // resident + staging-only waves
+    {8, 2, 16, true, 4, 0, "s8r2k16"},  {12, 1, 16, true, 4, 0, "s12r1k16"},
 };
 constexpr unsigned kNumConvConfigs = sizeof(kConvConfigs) / sizeof(kConvConfigs[0]);
 
@@ -67,9 +77,11 @@ bool chooseKT(const ConvConfig &cfg, unsigned CA, unsigned CB, unsigned K, const
   const unsigned ckp = cfg.ck + 8;
   const unsigned blocks = g.KOUTP / 32;
   // registers per lane: 512 shared by the waves of one SIMD; a workgroup of `waves` waves puts waves/4 on each
-  const unsigned regBudget = cfg.waves >= 16 ? 128 : 256;
+  const unsigned wavesPerSimd = (cfg.waves + cfg.pw + 3) / 4;
+  const unsigned regBudget = std::min(256u, 512u / wavesPerSimd);
   for (unsigned kb = blocks; kb >= 1; --kb) {
     if (blocks % kb) continue;
+    if (cfg.maxKT && kb * 32 > cfg.maxKT) continue;
     if (kb * cfg.rpw * 16 + 64 > regBudget) continue;
     const size_t lds = cfg.resident ? static_cast<size_t>(9u * kb * 32u) * (g.CPAD + 8) * 2u + 2u * static_cast<size_t>(haloPix) * ckp * 2u
                                     : (static_cast<size_t>(haloPix) + 9u * kb * 32u) * ckp * 2u;
@@ -204,7 +216,7 @@ public:
       if (!opt.forceConvConfig.empty() && opt.forceConvConfig != cfg.name) continue;
       if (cfg.ck > cpad && cfg.ck != 16) continue; // a larger stage than the whole reduction adds nothing
       if ((m.pattern & PAT_POOL) && (cfg.rpw % 2)) continue;
-      if (cfg.waves * 64 > opt.deviceInfo.maxComputeWorkGroupInvocations) continue;
+      if ((cfg.waves + cfg.pw) * 64 > opt.deviceInfo.maxComputeWorkGroupInvocations) continue;
       ConvGeometry g;
       if (!chooseKT(cfg, CA, CB, conv.K, opt.deviceInfo, g)) continue;
       out.push_back(c);
@@ -249,13 +261,14 @@ public:
     if (crop) k.define("CROP", 1);
     k.define("WAVES", cfg.waves); k.define("RPW", cfg.rpw); k.define("CK", cfg.ck);
     if (cfg.resident) k.define("SLOTS", g.slots);
+    if (cfg.pw) k.define("PW", cfg.pw);
     std::string entry = "conv3x3_c" + std::to_string(CA) + (up ? "u" : "") + (padA ? "e" : "") + (CB ? "p" + std::to_string(CB) + (padB ? "e" : "") : "") + "_k" +
                         std::to_string(conv.K) + (act == 1 ? "_relu" : act == 2 ? "_lrelu" : "") + (pool ? "_pool" : "") + (crop ? "_crop" : "") + "_" + cfg.name;
     k.define("KERNEL_NAME", entry);
     const Sym W = convIn.width, H = convIn.height;
     const unsigned th = cfg.waves * cfg.rpw;
     const unsigned nkt = g.KOUTP / g.KT;
-    auto d = cfg.resident ? impl.registerDispatch(k, entry, Sym::Const(opt.deviceInfo.xcdCount * nkt * g.slots), Sym::Const(1), Sym::Const(1), cfg.waves * 64)
+    auto d = cfg.resident ? impl.registerDispatch(k, entry, Sym::Const(opt.deviceInfo.xcdCount * nkt * g.slots), Sym::Const(1), Sym::Const(1), (cfg.waves + cfg.pw) * 64)
                           : impl.registerDispatch(k, entry, sym.cdiv(W, 32), sym.cdiv(H, th), Sym::Const(nkt), cfg.waves * 64);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     if (CB) d.addBinding(dnx::Access::ReadOnly, m.inputs[1]);

@@ -67,6 +67,16 @@ HipCompilerInstance HipCompiler::read(const std::string &relPath) const {
   inst.m_compiler = this;
   inst.m_path = relPath;
   inst.m_source = readFile(m_kernelDir + "/" + relPath);
+  // Experiment hook: extra "NAME=value NAME=value" definitions for every kernel (they take
+  // part in the hash, so such code objects never mix with regular ones).
+  if (const char *extra = std::getenv("DENOX_HIP_EXTRA_DEFINES")) {
+    std::istringstream ss(extra);
+    std::string kv;
+    while (ss >> kv) {
+      const size_t eq = kv.find('=');
+      inst.define(eq == std::string::npos ? kv : kv.substr(0, eq), eq == std::string::npos ? std::string("1") : kv.substr(eq + 1));
+    }
+  }
   return inst;
 }
 

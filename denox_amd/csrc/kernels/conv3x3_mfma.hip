@@ -21,55 +21,30 @@
 #define KERNEL_NAME conv3x3_mfma
 #endif
 
-#define NV_IN ((HALO_PIX * (CK / 8) + NT - 1) / NT)
-#define NV_W ((9 * KT * (CK / 8) + NT - 1) / NT)
+#define NV_W ((9 * KT * VPPK + NT - 1) / NT)
 
-struct Staged {
-  uint4v in[NV_IN];
-  uint4v w[NV_W];
-};
-
+// weight slice of one step: global [tap][KT rows][L] -> registers -> LDS rows of CKP
 template <int L>
-__device__ DNX_INLINE void
-fetch_chunk(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, const _Float16 *__restrict__ wchunk,
-            Staged &st, int c0, int y0, int x0, const PushConstants &pc, int tid) {
+__device__ DNX_INLINE void weights_fetch(const _Float16 *__restrict__ wchunk, uint4v (&st)[NV_W], int tid) {
   constexpr int VPP = L / 8;
-#pragma unroll
-  for (int it = 0; it < NV_IN; ++it) {
-    const int i = tid + it * NT;
-    uint4v val = {0u, 0u, 0u, 0u};
-    if (i < HALO_PIX * VPP)
-      val = load_halo_vec<L>(A, B, i, c0, y0, x0, pc);
-    st.in[it] = val;
-  }
-  // weight slice for these channels: global [tap][KT rows][L]
 #pragma unroll
   for (int it = 0; it < NV_W; ++it) {
     const int i = tid + it * NT;
     if (i < 9 * KT * VPP)
-      st.w[it] = ld16(wchunk + (size_t)i * 8);
+      st[it] = ld16(wchunk + (size_t)i * 8);
   }
 }
 
 template <int L>
-__device__ DNX_INLINE void commit_chunk(const Staged &st, _Float16 *sIn, _Float16 *sW, int tid) {
+__device__ DNX_INLINE void weights_commit(const uint4v (&st)[NV_W], _Float16 *sW, int tid) {
   constexpr int VPP = L / 8;
-#pragma unroll
-  for (int it = 0; it < NV_IN; ++it) {
-    const int i = tid + it * NT;
-    if (i < HALO_PIX * VPP) {
-      const int pix = i / VPP;
-      const int v = i - pix * VPP;
-      *reinterpret_cast<uint4v *>(sIn + pix * CKP + v * 8) = st.in[it];
-    }
-  }
 #pragma unroll
   for (int it = 0; it < NV_W; ++it) {
     const int i = tid + it * NT;
     if (i < 9 * KT * VPP) {
       const int row = i / VPP;
       const int v = i - row * VPP;
-      *reinterpret_cast<uint4v *>(sW + row * CKP + v * 8) = st.w[it];
+      *reinterpret_cast<uint4v *>(sW + row * CKP + v * 8) = st[it];
     }
   }
 }
@@ -100,40 +75,39 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   const int kt = DNX_BID_Z; // output-channel tile
 
   float16v acc[KB][RPW];
-#pragma unroll
-  for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-    for (int j = 0; j < RPW; ++j)
-#pragma unroll
-      for (int i = 0; i < 16; ++i)
-        acc[kb][j][i] = 0.0f;
+  zero_acc(acc);
 
   // packed filter: [kt][chunk][tap][KT][len(chunk)]
   const _Float16 *wbase = FILT + (size_t)kt * 9 * KT * CPAD;
-  Staged st;
+  typedef Halo<NT> H;
+  H::Map map;
+  H::Src src;
+  H::map_init(map, tid);
+  H::src_init(src, map, y0, x0, pc);
+  H::Regs stIn;
+  uint4v stW[NV_W];
+  H::fetch_step(A, B, stIn, map, src, 0);
   if (NCHUNK > 1 || TAIL == CK)
-    fetch_chunk<CK>(A, B, wbase, st, 0, y0, x0, pc, tid);
+    weights_fetch<CK>(wbase, stW, tid);
   else
-    fetch_chunk<TAIL>(A, B, wbase, st, 0, y0, x0, pc, tid);
+    weights_fetch<TAIL>(wbase, stW, tid);
   for (int chunk = 0; chunk < NCHUNK; ++chunk) {
     const bool fullNow = (TAIL == CK) || (chunk < NCHUNK - 1);
+    H::commit_step(stIn, sIn, map, chunk);
     if (fullNow)
-      commit_chunk<CK>(st, sIn, sW, tid);
+      weights_commit<CK>(stW, sW, tid);
     else
-      commit_chunk<TAIL>(st, sIn, sW, tid);
+      weights_commit<TAIL>(stW, sW, tid);
     DNX_SYNC();
-    if (chunk + 1 < NCHUNK) { // loads for the next chunk fly during the MFMAs below
-      const int c1 = (chunk + 1) * CK;
-      const _Float16 *wnext = wbase + (size_t)9 * KT * c1;
+    if (chunk + 1 < NCHUNK) { // loads for the next step fly during the MFMAs below
+      const _Float16 *wnext = wbase + (size_t)9 * KT * (chunk + 1) * CK;
+      H::fetch_step(A, B, stIn, map, src, chunk + 1);
       if (TAIL == CK || chunk + 1 < NCHUNK - 1)
-        fetch_chunk<CK>(A, B, wnext, st, c1, y0, x0, pc, tid);
+        weights_fetch<CK>(wnext, stW, tid);
       else
-        fetch_chunk<TAIL>(A, B, wnext, st, c1, y0, x0, pc, tid);
+        weights_fetch<TAIL>(wnext, stW, tid);
     }
-    if (fullNow)
-      mma_chunk<CK, CKP>(sIn, sW, 0, acc, wv, lane);
-    else
-      mma_chunk<TAIL, CKP>(sIn, sW, 0, acc, wv, lane);
+    mma_step<CKP>(sIn, sW, 0, acc, wv, lane, chunk);
     DNX_SYNC();
   }
   store_tile(acc, OUT, BIAS, y0, x0, kt, wv, lane, pc);

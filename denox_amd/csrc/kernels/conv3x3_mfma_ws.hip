@@ -4,9 +4,15 @@
 // The launch is persistent: GRID workgroups, one per compute unit, each keeps the whole
 // 9 x KT x CPAD weight slice of its output-channel tile in LDS for its lifetime and walks
 // over many (WAVES*RPW) x 32 pixel tiles.  Only input halos stream: CK channels at a time
-// through two LDS buffers, the loads of step i+1 issued into registers before the matrix
-// work of step i, one barrier per step.  Compared with streaming the weights per tile this
-// removes most L2 reads, most LDS writes and most address arithmetic of the inner loop.
+// through two LDS buffers, one barrier per step, every global load issued two steps before
+// its data is written to LDS.  Compared with streaming the weights per tile this removes
+// most L2 reads, most LDS writes and most address arithmetic of the inner loop.
+//
+//   PW = 0  every wave stages its share of the halo and then computes;
+//   PW > 0  wave specialisation: WAVES waves only compute (LDS reads + MFMA + epilogue) while
+//           PW further waves only stage halos, so that address arithmetic, load waits and LDS
+//           writes run beside the matrix work instead of in front of it (all waves of a
+//           workgroup meet at the step barrier, so inside one role nothing overlaps).
 //
 // Workgroup b serves XCD b % 8 (workgroups are dealt round-robin to the 8 XCDs), and each
 // XCD walks its own contiguous band of tiles so that neighbouring halos meet in one L2.
@@ -19,37 +25,8 @@
 
 #define NKT (KOUTP / KT)
 #define CPADP (CPAD + 8)
-#define NV_IN ((HALO_PIX * (CK / 8) + NT - 1) / NT)
 #define NXCD 8
-
-template <int L>
-__device__ DNX_INLINE void
-fetch_halo(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, uint4v (&st)[NV_IN], int c0, int y0, int x0,
-           const PushConstants &pc, int tid) {
-  constexpr int VPP = L / 8;
-#pragma unroll
-  for (int it = 0; it < NV_IN; ++it) {
-    const int i = tid + it * NT;
-    uint4v val = {0u, 0u, 0u, 0u};
-    if (i < HALO_PIX * VPP)
-      val = load_halo_vec<L>(A, B, i, c0, y0, x0, pc);
-    st[it] = val;
-  }
-}
-
-template <int L>
-__device__ DNX_INLINE void commit_halo(const uint4v (&st)[NV_IN], _Float16 *sIn, int tid) {
-  constexpr int VPP = L / 8;
-#pragma unroll
-  for (int it = 0; it < NV_IN; ++it) {
-    const int i = tid + it * NT;
-    if (i < HALO_PIX * VPP) {
-      const int pix = i / VPP;
-      const int v = i - pix * VPP;
-      *reinterpret_cast<uint4v *>(sIn + pix * CKP + v * 8) = st[it];
-    }
-  }
-}
+#define NSTAGE ((PW > 0 ? PW : WAVES) * 64) // threads that stage halos
 
 extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     const _Float16 *__restrict__ A,
@@ -70,7 +47,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   const _Float16 *BIAS = nullptr;
 #endif
   const int tid = DNX_TID;
-  const int wv = tid >> 6;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6); // wave-uniform: roles branch on it
   const int lane = tid & 63;
 
   const int b = DNX_BID_X;
@@ -100,60 +77,106 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     }
   }
 
-  uint4v st[NV_IN];
-  int ty = tile / tilesX, tx = tile - ty * tilesX;
-  if (NCHUNK > 1 || TAIL == CK)
-    fetch_halo<CK>(A, B, st, 0, ty * TH, tx * TW, pc, tid);
-  else
-    fetch_halo<TAIL>(A, B, st, 0, ty * TH, tx * TW, pc, tid);
-  int buf = 0;
-  while (true) {
-    const int y0 = ty * TH, x0 = tx * TW;
-    const int ntile = tile + SLOTS;
-    const bool more = ntile < last;
-    const int nty = ntile / tilesX, ntx = ntile - nty * tilesX;
-
-    float16v acc[KB][RPW];
-#pragma unroll
-    for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-      for (int j = 0; j < RPW; ++j)
-#pragma unroll
-        for (int i = 0; i < 16; ++i)
-          acc[kb][j][i] = 0.0f;
-
-    for (int chunk = 0; chunk < NCHUNK; ++chunk) {
-      const bool fullNow = (TAIL == CK) || (chunk < NCHUNK - 1);
-      if (fullNow)
-        commit_halo<CK>(st, sIn[buf], tid);
-      else
-        commit_halo<TAIL>(st, sIn[buf], tid);
-      // One barrier per step: buffer `buf` was last read two steps ago, and every wave
-      // has passed the barrier of the step in between since then.
-      DNX_SYNC();
-      if (chunk + 1 < NCHUNK) {
-        const int c1 = (chunk + 1) * CK;
-        if (TAIL == CK || chunk + 1 < NCHUNK - 1)
-          fetch_halo<CK>(A, B, st, c1, y0, x0, pc, tid);
-        else
-          fetch_halo<TAIL>(A, B, st, c1, y0, x0, pc, tid);
-      } else if (more) {
-        if (NCHUNK > 1 || TAIL == CK)
-          fetch_halo<CK>(A, B, st, 0, nty * TH, ntx * TW, pc, tid);
-        else
-          fetch_halo<TAIL>(A, B, st, 0, nty * TH, ntx * TW, pc, tid);
-      }
-      if (fullNow)
-        mma_chunk<CK, CPADP>(sIn[buf], sW, chunk * CK, acc, wv, lane);
-      else
-        mma_chunk<TAIL, CPADP>(sIn[buf], sW, chunk * CK, acc, wv, lane);
-      buf ^= 1;
+  // The fetch cursor walks the same sequence of steps as the compute cursor (tile by tile,
+  // NCHUNK steps per tile), two steps ahead.
+  typedef Halo<NSTAGE> H;
+  H::Map map;
+  H::Src fsrc;
+  int ftile = tile, fchunk = 0;
+  auto issue = [&](H::Regs &regs) {
+    if (ftile >= last)
+      return;
+    H::fetch_step(A, B, regs, map, fsrc, fchunk);
+    if (++fchunk == NCHUNK) {
+      fchunk = 0;
+      ftile += SLOTS;
+      if (ftile < last)
+        H::src_init(fsrc, map, (ftile / tilesX) * TH, (ftile % tilesX) * TW, pc);
     }
-    store_tile(acc, OUT, BIAS, y0, x0, kt, wv, lane, pc);
-    if (!more)
+  };
+
+#if PW == 0
+  H::map_init(map, tid);
+  H::src_init(fsrc, map, (ftile / tilesX) * TH, (ftile % tilesX) * TW, pc);
+  float16v acc[KB][RPW];
+  int cchunk = 0, buf = 0;
+  auto step = [&](H::Regs &regs) {
+    if (cchunk == 0)
+      zero_acc(acc);
+    H::commit_step(regs, sIn[buf], map, cchunk);
+    // One barrier per step: buffer `buf` was last read two steps ago, and every wave
+    // has passed the barrier of the step in between since then.
+    DNX_SYNC();
+    issue(regs); // refill this register set: the step after next
+    mma_step<CPADP>(sIn[buf], sW, cchunk * CK, acc, wv, lane, cchunk);
+    buf ^= 1;
+    if (++cchunk == NCHUNK) {
+      const int ty = tile / tilesX, tx = tile - ty * tilesX;
+      store_tile(acc, OUT, BIAS, ty * TH, tx * TW, kt, wv, lane, pc);
+      cchunk = 0;
+      tile += SLOTS;
+    }
+  };
+  H::Regs st0, st1;
+  issue(st0);
+  issue(st1);
+  while (true) {
+    step(st0);
+    if (tile >= last)
       break;
-    tile = ntile;
-    ty = nty;
-    tx = ntx;
+    step(st1);
+    if (tile >= last)
+      break;
   }
+#else
+  // number of steps this workgroup runs: both roles execute exactly one barrier per step
+  const int myTiles = (last - tile + SLOTS - 1) / SLOTS;
+  const int steps = myTiles * NCHUNK;
+  if (wv >= WAVES) {
+    // ---- staging waves: step g's halo is written to sIn[g & 1] during step g - 1 ----
+    H::map_init(map, tid - WAVES * 64);
+    H::src_init(fsrc, map, (ftile / tilesX) * TH, (ftile % tilesX) * TW, pc);
+    H::Regs st0, st1;
+    int cchunk = 0; // chunk index of the step being committed
+    auto commit = [&](H::Regs &regs, int g) {
+      H::commit_step(regs, sIn[g & 1], map, cchunk);
+      if (++cchunk == NCHUNK)
+        cchunk = 0;
+    };
+    issue(st0);         // step 0
+    issue(st1);         // step 1
+    commit(st0, 0);
+    issue(st0);         // step 2
+    for (int g = 0; g < steps; g += 2) {
+      DNX_SYNC();       // step g starts: sIn[g & 1] is complete, sIn[(g + 1) & 1] is free
+      if (g + 1 < steps) {
+        commit(st1, g + 1);
+        issue(st1);     // step g + 3
+      }
+      if (g + 1 >= steps)
+        break;
+      DNX_SYNC();       // step g + 1 starts
+      if (g + 2 < steps) {
+        commit(st0, g + 2);
+        issue(st0);     // step g + 4
+      }
+    }
+  } else {
+    // ---- computing waves ----
+    float16v acc[KB][RPW];
+    int cchunk = 0;
+    for (int g = 0; g < steps; ++g) {
+      if (cchunk == 0)
+        zero_acc(acc);
+      DNX_SYNC();
+      mma_step<CPADP>(sIn[g & 1], sW, cchunk * CK, acc, wv, lane, cchunk);
+      if (++cchunk == NCHUNK) {
+        const int ty = tile / tilesX, tx = tile - ty * tilesX;
+        store_tile(acc, OUT, BIAS, ty * TH, tx * TW, kt, wv, lane, pc);
+        cchunk = 0;
+        tile += SLOTS;
+      }
+    }
+  }
+#endif
 }

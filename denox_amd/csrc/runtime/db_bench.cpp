@@ -1,6 +1,8 @@
 #include "db_bench.hpp"
+#include <algorithm>
 #include <cstring>
 #include <sstream>
+#include <vector>
 
 namespace denox::runtime {
 
@@ -58,8 +60,20 @@ DbBenchResult db_bench(Db &db, const ContextHandle &ctx, const hip::HipCompiler 
           scratch = nullptr;
           hipCheck(hipMalloc(&scratch, need), "hipMalloc(scratch)");
           scratchBytes = need;
-          // zeros are as good as any contents and keep fp16 arithmetic away from NaN slow paths
-          hipCheck(hipMemsetAsync(scratch, 0, need, s), "hipMemsetAsync");
+          // Finite binary16 values of mixed sign and magnitude below 2: timings then include the
+          // switching activity of real data (an all-zero buffer lets the chip clock higher than a
+          // frame would) and no arithmetic meets NaN or infinity.
+          std::vector<uint16_t> pattern(1u << 20);
+          uint32_t lcg = 12345u;
+          for (auto &h : pattern) {
+            lcg = lcg * 1664525u + 1013904223u;
+            h = static_cast<uint16_t>(((lcg >> 16) & 0x8000u) | (0x2C00u + ((lcg >> 8) % 0x1000u))); // |x| in [2^-4, 1)
+          }
+          for (uint64_t off = 0; off < need; off += pattern.size() * 2) {
+            const uint64_t n = std::min<uint64_t>(pattern.size() * 2, need - off);
+            hipCheck(hipMemcpyAsync(static_cast<uint8_t *>(scratch) + off, pattern.data(), n, hipMemcpyHostToDevice, s), "hipMemcpyAsync(scratch)");
+          }
+          hipCheck(hipStreamSynchronize(s), "hipStreamSynchronize");
         }
         std::vector<uint8_t> args(row.bindings.size() * sizeof(void *));
         for (size_t i = 0; i < offs.size(); ++i) {

@@ -45,8 +45,9 @@ def test_conv3x3(oracle, C, K, H, W, act):
     assert_conv_close(got, want, f"conv {C}->{K} {H}x{W} {act}")
 
 
-ALL_CONFIGS = ["w4r2k16", "w4r2k32", "w4r4k16", "w4r4k32", "w8r2k16", "w8r2k32", "w4r2k64", "w8r1k16",
-               "p8r1k16", "p8r1k32", "p16r1k16", "p16r1k32", "p8r2k16", "p8r2k32", "p16r2k16", "p4r2k32"]
+ALL_CONFIGS = ["w4r2k16", "w4r2k32", "w4r4k16", "w4r4k32", "w8r2k16", "w8r2k32", "w4r2k64", "w8r1k16", "w4r1k16", "w4r1k32",
+               "w4r1k32n", "w4r2k32n", "w2r2k32n", "w2r2k32", "p8r1k16", "p8r1k32", "p16r1k16", "p16r1k32", "p8r2k16", "p8r2k32",
+               "p16r2k16", "p4r2k32", "p8r4k16", "p4r4k16", "p4r4k32", "p4r1k32", "p4r2k32n", "p4r1k32n", "s8r2k16", "s12r1k16"]
 
 
 @pytest.mark.parametrize("config", ALL_CONFIGS)
@@ -123,7 +124,7 @@ FUSION_FLAGS = [
 ]
 
 
-@pytest.mark.parametrize("config", ["w4r2k16", "p8r1k16", "p16r1k16", "w8r2k16"])
+@pytest.mark.parametrize("config", ["w4r2k16", "p8r1k16", "p16r1k16", "w8r2k16", "s8r2k16", "s12r1k16"])
 @pytest.mark.parametrize("features", [{}, {"pad_fusion": False}, {"slice_fusion": False}, {"pad_fusion": False, "slice_fusion": False}])
 def test_pad_and_slice_fold_into_the_conv(oracle, features, config):
     """pad -> (upsample, pad) concat -> conv -> relu -> slice, with offsets on every side."""

@@ -103,7 +103,7 @@ def test_oidn_unet_schedule_dispatch_geometry_covers_every_pixel():
         assert sum(x["flops"] for x in convs) == pytest.approx(523.9e9 * (Hp * Wp) / (1088 * 1920), rel=2e-3)
         for x in convs:
             w, h = x["push_constants"][:2]
-            rows = x["workgroup_size"][0] // 64 * int(re.search(r"RPW=(\d+)", x["debug_info"]).group(1))
+            rows = int(re.search(r"WAVES=(\d+)", x["debug_info"]).group(1)) * int(re.search(r"RPW=(\d+)", x["debug_info"]).group(1))
             gx, gy, gz = x["workgroup_count"]
             kt = int(re.search(r"KT=(\d+)", x["debug_info"]).group(1))
             kout = int(re.search(r"KOUT=(\d+)", x["debug_info"]).group(1))
