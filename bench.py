@@ -120,6 +120,12 @@ def main() -> int:
         print("bench.py: non-finite output", file=sys.stderr)
         return 1
 
+    # the reference's own entry point (host pointers in and out, blocking): PCIe-inclusive, reported beside, never as `value`
+    t0 = time.perf_counter()
+    for _ in range(3):
+        inst.infer(x)
+    host_ms = (time.perf_counter() - t0) / 3 * 1e3
+
     # per-dispatch hipEvent timings on the launch stream, averaged over several passes
     passes = 5
     acc = None
@@ -152,6 +158,16 @@ def main() -> int:
                 "non_conv_frac_of_hbm": other_bytes / other_ms * 1e-6 / PEAK_HBM_GBPS if other_ms else None,
                 "sum_dispatch_ms": sum(a["latency_ms"] for a in acc)}
 
+    # HBM traffic of the dominant kernel from the committed rocprofv3 --pmc summary, when it covers this kernel
+    try:
+        with open(os.path.join(ROOT, "profiles", "dominant_conv_traffic.json")) as f:
+            tr = json.load(f)
+        if tr["dispatch_name"] == dom["name"] and (H, W) == (tr["height"], tr["width"]):
+            roofline["traffic"] = tr["fetch_bytes"] + tr["write_bytes"]
+            roofline["traffic_unit"] = "bytes per launch (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel)"
+    except (OSError, KeyError, ValueError):
+        pass
+
     line = {
         "metric": "oidn_unet_fp16_hwc_1080p_throughput", "value": H * W / (ms * 1e-3) * 1e-6, "unit": "Mpix/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
@@ -159,7 +175,7 @@ def main() -> int:
         "config": {"workload": f"OIDN-style U-Net 9->3, fp16 HWC, {W}x{H}, replicate-pad to multiple of 16 + crop included, "
                                f"{mod.runtime_model.dispatch_count} dispatches in one hipGraph", "device_bytes": inst.device_bytes,
                    "schedule": "min-cost over measured dispatch latencies" if db is not None else "min-cost over roofline estimates",
-                   "tuning_seconds": round(tune_s, 2)},
+                   "tuning_seconds": round(tune_s, 2), "host_pointer_path_ms_per_frame": round(host_ms, 3)},
         "roofline": roofline,
     }
     if not args.no_cpu_baseline:
