@@ -300,8 +300,12 @@ std::vector<uint8_t> compile(const Model &modelIn, const hip::HipCompiler &hipc,
   }
 
   double total = 0.0;
+  unsigned walk = 0; // alternates the tile walk of consecutive tiled dispatches
   for (size_t e : chosen) {
-    const SuperGraphEdge &edge = g.edges[e];
+    SuperGraphEdge &edge = g.edges[e];
+    if (opt.features.enableAlternatingTraversal)
+      for (auto &d : edge.dispatches)
+        if (d.traversalFlagIndex >= 0) d.pushConstants[static_cast<size_t>(d.traversalFlagIndex)].value = Sym::Const(walk++ & 1u);
     for (const auto &p : edge.parameters) {
       const uint32_t id = place(p.tensor.index);
       dnx::TensorInitializer init;

@@ -28,6 +28,11 @@ void ComputeDispatchBuilder::addParamBinding(TensorId tensor) {
 
 void ComputeDispatchBuilder::addPushConstant(Sym value, dnx::ScalarType dtype) { self().pushConstants.push_back(PushConstantDesc{value, dtype}); }
 
+void ComputeDispatchBuilder::addTraversalFlag() {
+  self().traversalFlagIndex = static_cast<int>(self().pushConstants.size());
+  self().pushConstants.push_back(PushConstantDesc{Sym::Const(0), dnx::ScalarType::U32});
+}
+
 ComputeDispatchBuilder::~ComputeDispatchBuilder() {
   if (!m_impl) return;
   auto &bs = self().bindings;

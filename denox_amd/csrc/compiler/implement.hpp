@@ -51,6 +51,9 @@ struct ComputeDispatch {
   uint32_t workgroupSize[3] = {1, 1, 1};
   std::vector<TensorBinding> bindings;
   ComputeDispatchInfo info;
+  // index of a push constant whose bit 0 selects a reversed tile walk, -1 if the kernel has none;
+  // the compiler alternates it along the selected schedule (it is 0 in every table row)
+  int traversalFlagIndex = -1;
 };
 
 struct SuperTensor {
@@ -90,6 +93,7 @@ public:
   void addBinding(dnx::Access access, TensorHandle modelTensor);
   void addParamBinding(TensorId tensor);
   void addPushConstant(Sym value, dnx::ScalarType dtype = dnx::ScalarType::U32);
+  void addTraversalFlag(); // a U32 push constant, 0 here, set per position in the schedule
   void setName(const std::string &n) { self().info.name = n; }
   void setConfig(const std::string &c) { self().info.config = c; }
   void setOperation(const std::string &o) { self().info.operation = o; }

@@ -50,6 +50,10 @@ const ConvConfig kConvConfigs[] = {
     // small tiles / one 32-channel block per workgroup: more workgroups for low-resolution layers
     {4, 1, 16, false, 0, 0, "w4r1k16"}, {4, 1, 32, false, 0, 0, "w4r1k32"}, {4, 1, 32, false, 0, 32, "w4r1k32n"}, {4, 2, 32, false, 0, 32, "w4r2k32n"},
     {2, 2, 32, false, 0, 32, "w2r2k32n"}, {2, 2, 32, false, 0, 0, "w2r2k32"},
+    // ck = 0: the whole reduction (or half of it, ck = 1) in one step -- a single round of global loads per workgroup,
+    // for layers with so few tiles that load latency, not throughput, is what a workgroup waits for
+    {4, 1, 0, false, 0, 32, "w4r1kfn"}, {4, 1, 1, false, 0, 32, "w4r1khn"}, {4, 2, 0, false, 0, 32, "w4r2kfn"}, {2, 2, 0, false, 0, 32, "w2r2kfn"},
+    {4, 1, 0, false, 0, 64, "w4r1kfm"}, {4, 2, 1, false, 0, 32, "w4r2khn"},
     // weights resident, persistent launch
     {8, 1, 16, true, 0, 0, "p8r1k16"},  {8, 1, 32, true, 0, 0, "p8r1k32"},  {16, 1, 16, true, 0, 0, "p16r1k16"}, {16, 1, 32, true, 0, 0, "p16r1k32"},
     {8, 2, 16, true, 0, 0, "p8r2k16"},  {8, 2, 32, true, 0, 0, "p8r2k32"},  {16, 2, 16, true, 0, 0, "p16r2k16"}, {4, 2, 32, true, 0, 0, "p4r2k32"},
@@ -70,8 +74,18 @@ struct ConvGeometry {
 // Output channels per workgroup: the largest divisor of KOUTP (in blocks of 32)
 // whose weights fit LDS next to the halo(s) and whose accumulators fit the
 // register file.
-bool chooseKT(const ConvConfig &cfg, unsigned CA, unsigned CB, unsigned K, const DeviceInfo &dev, ConvGeometry &g) {
+// channels per LDS step of a configuration for a layer with `cpad` padded input channels
+unsigned stepChannels(const ConvConfig &cfg, unsigned cpad) {
+  if (cfg.ck == 0) return cpad;                                  // everything at once
+  if (cfg.ck == 1) return std::max(16u, (cpad / 2 + 15) / 16 * 16); // two steps
+  return cfg.ck;
+}
+
+bool chooseKT(const ConvConfig &cfgIn, unsigned CA, unsigned CB, unsigned K, const DeviceInfo &dev, ConvGeometry &g) {
   g.CA = CA; g.CB = CB; g.C = CA + CB; g.CPAD = (g.C + 15) / 16 * 16; g.K = K; g.KOUTP = (K + 31) / 32 * 32;
+  ConvConfig cfg = cfgIn;
+  cfg.ck = stepChannels(cfgIn, g.CPAD);
+  if (cfg.ck > 192) return false; // staging registers
   const unsigned th = cfg.waves * cfg.rpw;
   const unsigned haloPix = (th + 2) * 34;
   const unsigned ckp = cfg.ck + 8;
@@ -215,6 +229,7 @@ public:
       const ConvConfig &cfg = kConvConfigs[c];
       if (!opt.forceConvConfig.empty() && opt.forceConvConfig != cfg.name) continue;
       if (cfg.ck > cpad && cfg.ck != 16) continue; // a larger stage than the whole reduction adds nothing
+      if (cfg.ck <= 1 && cpad <= 32) continue;     // "whole / half reduction" duplicates a fixed-size stage for narrow layers
       if ((m.pattern & PAT_POOL) && (cfg.rpw % 2)) continue;
       if ((cfg.waves + cfg.pw) * 64 > opt.deviceInfo.maxComputeWorkGroupInvocations) continue;
       ConvGeometry g;
@@ -259,7 +274,7 @@ public:
     if (padA) k.define("PADA", 1);
     if (padB) k.define("PADB", 1);
     if (crop) k.define("CROP", 1);
-    k.define("WAVES", cfg.waves); k.define("RPW", cfg.rpw); k.define("CK", cfg.ck);
+    k.define("WAVES", cfg.waves); k.define("RPW", cfg.rpw); k.define("CK", stepChannels(cfg, g.CPAD));
     if (cfg.resident) k.define("SLOTS", g.slots);
     if (cfg.pw) k.define("PW", cfg.pw);
     std::string entry = "conv3x3_c" + std::to_string(CA) + (up ? "u" : "") + (padA ? "e" : "") + (CB ? "p" + std::to_string(CB) + (padB ? "e" : "") : "") + "_k" +
@@ -274,7 +289,7 @@ public:
     if (CB) d.addBinding(dnx::Access::ReadOnly, m.inputs[1]);
     d.addBinding(dnx::Access::WriteOnly, m.output);
     const Op convCopy = conv; // the lazy packers outlive the model reference
-    const unsigned ck = cfg.resident ? g.CPAD : cfg.ck;
+    const unsigned ck = cfg.resident ? g.CPAD : stepChannels(cfg, g.CPAD);
     TensorId wt = impl.createParameter(static_cast<size_t>(g.KOUTP) * 9 * g.CPAD * 2, dnx::ScalarType::F16,
                                        [convCopy, g, ck]() { return packConvWeights(convCopy, g, ck); });
     d.addParamBinding(wt);
@@ -299,6 +314,7 @@ public:
       const TensorNode &o = model.tensors()[m.output];
       d.addPushConstant(o.width); d.addPushConstant(o.height); d.addPushConstant(sl.left); d.addPushConstant(sl.top);
     }
+    d.addTraversalFlag();
 
     std::string nm = "conv3x3";
     if (up) nm = "upsample+" + nm;
@@ -325,8 +341,9 @@ private:
 };
 
 // ------------------------------------------------------------------ bandwidth kernels
-Sym linearGrid(SymGraph &sym, Sym w, Sym h, unsigned vectorsPerPixel) {
-  return sym.cdiv(sym.mul(sym.mul(w, h), static_cast<int64_t>(vectorsPerPixel)), WG_BANDWIDTH);
+// grid.x: workgroups covering one row of w * vectorsPerPixel vectors; grid.y: the rows
+Sym rowGrid(SymGraph &sym, Sym w, unsigned vectorsPerPixel) {
+  return sym.cdiv(sym.mul(w, static_cast<int64_t>(vectorsPerPixel)), WG_BANDWIDTH);
 }
 
 class SingleOpShader : public IShader {
@@ -367,7 +384,7 @@ public:
     k.define("CH", in.channels); k.define("KX", op.kernelX); k.define("KY", op.kernelY); k.define("VEC", vec);
     const std::string entry = "pool_max_c" + std::to_string(in.channels) + "v" + std::to_string(vec);
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, linearGrid(sym, out.width, out.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, in.channels / vec), out.height, Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     d.addBinding(dnx::Access::WriteOnly, m.output);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
@@ -388,7 +405,7 @@ public:
     k.define("CH", in.channels); k.define("SCALE", op.scale); k.define("VEC", vec);
     const std::string entry = "upsample_c" + std::to_string(in.channels) + "v" + std::to_string(vec);
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, linearGrid(sym, in.width, in.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, rowGrid(sym, in.width, in.channels / vec), in.height, Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     d.addBinding(dnx::Access::WriteOnly, m.output);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
@@ -416,7 +433,7 @@ public:
       k.define("COUNT", in.channels); k.define("VEC", vec);
       const std::string entry = "copy_c" + std::to_string(in.channels) + "_to_c" + std::to_string(out.channels) + "o" + std::to_string(off) + "v" + std::to_string(vec);
       k.define("KERNEL_NAME", entry);
-      auto d = impl.registerDispatch(k, entry, linearGrid(sym, in.width, in.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
+      auto d = impl.registerDispatch(k, entry, rowGrid(sym, in.width, in.channels / vec), in.height, Sym::Const(1), WG_BANDWIDTH);
       d.addBinding(dnx::Access::ReadOnly, m.inputs[s]);
       d.addBinding(dnx::Access::WriteOnly, m.output);
       d.addPushConstant(in.width); d.addPushConstant(in.height);
@@ -440,7 +457,7 @@ public:
     if (op.func == ActivationFunction::LeakyReLU) k.define("ALPHA", fmtFloat(op.alpha));
     const std::string entry = std::string(op.func == ActivationFunction::ReLU ? "relu_c" : "leaky_relu_c") + std::to_string(in.channels) + "v" + std::to_string(vec);
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, linearGrid(sym, in.width, in.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, rowGrid(sym, in.width, in.channels / vec), in.height, Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     d.addBinding(dnx::Access::WriteOnly, m.output);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
@@ -463,7 +480,7 @@ public:
     k.define("CH", in.channels); k.define("VEC", vec);
     const std::string entry = "memory_pad_c" + std::to_string(in.channels) + "v" + std::to_string(vec);
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, linearGrid(sym, out.width, out.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, in.channels / vec), out.height, Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     d.addBinding(dnx::Access::WriteOnly, m.output);
     d.addPushConstant(out.width); d.addPushConstant(out.height);
@@ -485,7 +502,7 @@ public:
     k.define("CH", in.channels); k.define("VEC", vec);
     const std::string entry = "memory_slice_c" + std::to_string(in.channels) + "v" + std::to_string(vec);
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, linearGrid(sym, out.width, out.height, in.channels / vec), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, in.channels / vec), out.height, Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     d.addBinding(dnx::Access::WriteOnly, m.output);
     d.addPushConstant(op.top); d.addPushConstant(op.left);

@@ -1,12 +1,11 @@
 // activation.hip -- stand-alone elementwise activation in binary16.
 // Replaces compiler/src/denox/compiler/implement/shaders/activation/basic_activation.comp:26-184:
 //   ReLU: max(v, 0);  LeakyReLU: max(v, alpha * v) with alpha and the product in binary16.
-// Definitions: CH, ACT (1 ReLU, 2 LeakyReLU), ALPHA, VEC.
+// Definitions: CH, ACT (1 ReLU, 2 LeakyReLU), ALPHA, VEC.  grid.y = rows.
 #include "common.h"
 #ifndef ALPHA
 #define ALPHA 0.0f
 #endif
-// The entry point is named per variant (KERNEL_NAME) so that profilers tell variants apart.
 #ifndef KERNEL_NAME
 #define KERNEL_NAME activation
 #endif
@@ -22,16 +21,16 @@ __device__ DNX_INLINE _Float16 act1(_Float16 v) {
 extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
     const ushort_t *__restrict__ IN, ushort_t *__restrict__ OUT, PushConstants pc) {
   constexpr unsigned CV = CH / VEC;
-  const unsigned long long idx = (unsigned long long)DNX_BID_X * WG + DNX_TID;
-  const unsigned long long total = (unsigned long long)pc.W * pc.H * CV;
-  if (idx >= total) return;
-  const vec_t v = ldv(IN + idx * VEC);
+  const unsigned i = DNX_ROW_INDEX();
+  if (i >= pc.W * CV) return;
+  const size_t idx = ((size_t)DNX_BID_Y * pc.W * CV + i) * VEC;
+  const vec_t v = ldv(IN + idx);
 #if VEC == 8
   half8 a = __builtin_bit_cast(half8, v);
 #pragma unroll
   for (int e = 0; e < 8; ++e) a[e] = act1(a[e]);
-  stv(OUT + idx * VEC, __builtin_bit_cast(uint4v, a));
+  stv(OUT + idx, __builtin_bit_cast(uint4v, a));
 #else
-  stv(OUT + idx * VEC, __builtin_bit_cast(ushort_t, act1(__builtin_bit_cast(_Float16, v))));
+  stv(OUT + idx, __builtin_bit_cast(ushort_t, act1(__builtin_bit_cast(_Float16, v))));
 #endif
 }

@@ -1,7 +1,11 @@
-#include "prelude.h"
 // Shared helpers for the bandwidth kernels.  Every kernel processes VEC
 // channels per thread: VEC = 8 (one 16-byte access) when all channel counts and
 // offsets involved are multiples of 8, else VEC = 1 (2-byte accesses).
+//
+// Launch geometry (all of them): grid.y = rows of the iteration space, grid.x * WG threads
+// cover one row of width * (channels / VEC) vectors.  Indices inside a row are 32-bit and
+// only divided by compile-time constants; nothing divides by a run-time extent.
+#include "prelude.h"
 typedef unsigned short ushort_t;
 typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -32,3 +36,6 @@ __device__ DNX_INLINE ushort_t max_keep_first(ushort_t acc, ushort_t v) {
   const _Float16 b = __builtin_bit_cast(_Float16, v);
   return b > a ? v : acc;
 }
+
+// position of this thread inside its row: vector index `i` in [0, rowVectors)
+#define DNX_ROW_INDEX() (DNX_BID_X * WG + (unsigned)DNX_TID)

@@ -65,6 +65,10 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   int tile = first + slot;
   if (tile >= last)
     return; // uniform for the workgroup: nothing was staged yet
+  const bool rev = (pc.FLAGS & 1u) != 0;
+  // position of the t-th tile of the walk
+  auto tileY = [&](int t) { return ((rev ? numTiles - 1 - t : t) / tilesX) * TH; };
+  auto tileX = [&](int t) { return ((rev ? numTiles - 1 - t : t) % tilesX) * TW; };
 
   // ---- resident weights: global [tap][KT][CPAD] (one chunk = whole reduction) -> LDS rows of CPADP ----
   {
@@ -91,13 +95,13 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
       fchunk = 0;
       ftile += SLOTS;
       if (ftile < last)
-        H::src_init(fsrc, map, (ftile / tilesX) * TH, (ftile % tilesX) * TW, pc);
+        H::src_init(fsrc, map, tileY(ftile), tileX(ftile), pc);
     }
   };
 
 #if PW == 0
   H::map_init(map, tid);
-  H::src_init(fsrc, map, (ftile / tilesX) * TH, (ftile % tilesX) * TW, pc);
+  H::src_init(fsrc, map, tileY(ftile), tileX(ftile), pc);
   float16v acc[KB][RPW];
   int cchunk = 0, buf = 0;
   auto step = [&](H::Regs &regs) {
@@ -111,8 +115,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     mma_step<CPADP>(sIn[buf], sW, cchunk * CK, acc, wv, lane, cchunk);
     buf ^= 1;
     if (++cchunk == NCHUNK) {
-      const int ty = tile / tilesX, tx = tile - ty * tilesX;
-      store_tile(acc, OUT, BIAS, ty * TH, tx * TW, kt, wv, lane, pc);
+      store_tile(acc, OUT, BIAS, tileY(tile), tileX(tile), kt, wv, lane, pc);
       cchunk = 0;
       tile += SLOTS;
     }
@@ -135,7 +138,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   if (wv >= WAVES) {
     // ---- staging waves: step g's halo is written to sIn[g & 1] during step g - 1 ----
     H::map_init(map, tid - WAVES * 64);
-    H::src_init(fsrc, map, (ftile / tilesX) * TH, (ftile % tilesX) * TW, pc);
+    H::src_init(fsrc, map, tileY(ftile), tileX(ftile), pc);
     H::Regs st0, st1;
     int cchunk = 0; // chunk index of the step being committed
     auto commit = [&](H::Regs &regs, int g) {
@@ -171,8 +174,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
       DNX_SYNC();
       mma_step<CPADP>(sIn[g & 1], sW, cchunk * CK, acc, wv, lane, cchunk);
       if (++cchunk == NCHUNK) {
-        const int ty = tile / tilesX, tx = tile - ty * tilesX;
-        store_tile(acc, OUT, BIAS, ty * TH, tx * TW, kt, wv, lane, pc);
+        store_tile(acc, OUT, BIAS, tileY(tile), tileX(tile), kt, wv, lane, pc);
         cchunk = 0;
         tile += SLOTS;
       }

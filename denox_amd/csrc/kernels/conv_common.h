@@ -67,6 +67,10 @@ struct PushConstants {
 #if CROP
   unsigned int OUT_W, OUT_H, CROP_L, CROP_T;
 #endif
+  // bit 0: walk the tiles in reverse order.  Consecutive layers alternate, so a layer starts
+  // where its producer just finished and finds that part of its input still in the
+  // memory-side cache.
+  unsigned int FLAGS;
 };
 
 __device__ DNX_INLINE uint4v ld16(const _Float16 *p) {
@@ -92,8 +96,13 @@ __device__ DNX_INLINE void src_offsets(int gy, int gx, const PushConstants &pc, 
   const int by = gy, bx = gx;
   const unsigned WB = W;
 #endif
+#ifdef DBG_FETCH_SMALL // timing experiment: same instructions, all loads hit a 4096-pixel window
+  pa = (((size_t)ay * WA + (size_t)ax) & 4095) * CA;
+  pb = (((size_t)by * WB + (size_t)bx) & 4095) * (CB > 0 ? CB : 1);
+#else
   pa = ((size_t)ay * WA + (size_t)ax) * CA;
   pb = ((size_t)by * WB + (size_t)bx) * (CB > 0 ? CB : 1);
+#endif
 }
 
 typedef uint4v __attribute__((aligned(2))) uint4v_u; // global memory is accessed in unaligned mode
@@ -338,8 +347,13 @@ store_tile(const float16v (&acc)[KB][RPW], _Float16 *__restrict__ OUT, const _Fl
       if (y < (int)H && x < (int)W && oy >= 0 && oy < (int)pc.OUT_H && ox >= 0 && ox < (int)pc.OUT_W)
         store16(OUT + ((size_t)oy * pc.OUT_W + ox) * KOUT + chb, o, chb);
 #else
+#ifdef DBG_STORE_SMALL // timing experiment: same instructions, all stores land in a 4096-pixel window
+      if (y < (int)H && x < (int)W)
+        store16(OUT + ((((size_t)y * W + x) & 4095) * KOUT) + chb, o, chb);
+#else
       if (y < (int)H && x < (int)W)
         store16(OUT + ((size_t)y * W + x) * KOUT + chb, o, chb);
+#endif
 #endif
     }
 #endif

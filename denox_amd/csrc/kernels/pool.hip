@@ -2,9 +2,8 @@
 // Replaces compiler/src/denox/compiler/implement/shaders/pool/basic_pool.comp:27-230:
 //   out[oh, ow, c] = max_{r<KY, s<KX} in[oh*KY + r, ow*KX + s, c],
 //   output extent floor(H/KY) x floor(W/KX).
-// Definitions: CH, KX, KY, VEC.  One thread per output vector.
+// Definitions: CH, KX, KY, VEC.  One thread per output vector; grid.y = output rows.
 #include "common.h"
-// The entry point is named per variant (KERNEL_NAME) so that profilers tell variants apart.
 #ifndef KERNEL_NAME
 #define KERNEL_NAME pool_max
 #endif
@@ -12,13 +11,11 @@ struct PushConstants { unsigned int W, H; };
 extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
     const ushort_t *__restrict__ IN, ushort_t *__restrict__ OUT, PushConstants pc) {
   constexpr unsigned CV = CH / VEC;
-  const unsigned W2 = pc.W / KX, H2 = pc.H / KY;
-  const unsigned long long idx = (unsigned long long)DNX_BID_X * WG + DNX_TID;
-  const unsigned long long total = (unsigned long long)W2 * H2 * CV;
-  if (idx >= total) return;
-  const unsigned cv = (unsigned)(idx % CV);
-  const unsigned long long pix = idx / CV;
-  const unsigned ow = (unsigned)(pix % W2), oh = (unsigned)(pix / W2);
+  const unsigned W2 = pc.W / KX;
+  const unsigned oh = DNX_BID_Y;
+  const unsigned i = DNX_ROW_INDEX();
+  if (i >= W2 * CV) return;
+  const unsigned ow = i / CV, cv = i - ow * CV;
   const ushort_t *src = IN + ((size_t)(oh * KY) * pc.W + (size_t)ow * KX) * CH + cv * VEC;
   vec_t acc = ldv(src);
 #pragma unroll
@@ -36,5 +33,5 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
       acc = max_keep_first(acc, v);
 #endif
     }
-  stv(OUT + (size_t)pix * CH + cv * VEC, acc);
+  stv(OUT + ((size_t)oh * W2 + ow) * CH + cv * VEC, acc);
 }

@@ -137,7 +137,7 @@ Instance::Instance(ModelHandle model, const std::vector<ValueSpec> &specs) : m_m
       l.fn = md.function;
       const int64_t g[3] = {d.workgroup_count_x.eval(m_sym), d.workgroup_count_y.eval(m_sym), d.workgroup_count_z.eval(m_sym)};
       for (int i = 0; i < 3; ++i) {
-        if (g[i] < 0 || g[i] > 0x7FFFFFFF) fail(Status::InvalidArgument, "dispatch '" + d.info.name + "' workgroup count out of range");
+        if (g[i] < 0 || g[i] > (i == 0 ? 0x7FFFFFFF : 65535)) fail(Status::InvalidArgument, "dispatch '" + d.info.name + "' workgroup count out of range");
         l.grid[i] = static_cast<unsigned>(g[i]);
         l.block[i] = d.workgroup_size[i];
       }

@@ -63,7 +63,9 @@ def test_tiny_unet_schedule_and_geometry():
     # e0 feeds both the pool and the skip, so the pool stays its own dispatch; upsample+concat fold into the conv
     assert names == ["conv3x3+relu", "maxpool", "conv3x3+relu", "concat+upsample+conv3x3+relu", "conv3x3"]
     conv0 = d["dispatches"][0]
-    assert conv0["push_constants"] == [128, 128] and conv0["flops"] == 2 * 9 * 3 * 16 * 128 * 128
+    # IN_W, IN_H, then the tile-walk flag, which alternates along the schedule
+    assert conv0["push_constants"] == [128, 128, 0] and conv0["flops"] == 2 * 9 * 3 * 16 * 128 * 128
+    assert [x["push_constants"][-1] for x in d["dispatches"] if "conv3x3" in x["name"]] == [0, 1, 0, 1]
     tx, ty, tz = conv0["workgroup_count"]
     rows = conv0["workgroup_size"][0] // 64 * int(re.search(r"RPW=(\d+)", conv0["debug_info"]).group(1))
     assert tx * 32 >= 128 and ty * rows >= 128 and (tx - 1) * 32 < 128 and (ty - 1) * rows < 128 and tz == 1
@@ -92,8 +94,8 @@ def test_oidn_unet_schedule_dispatch_geometry_covers_every_pixel():
         Hp, Wp = (H + 15) // 16 * 16, (W + 15) // 16 * 16
         # pad and crop fold into the first / last conv: IN extent, then source extent + offsets or crop window
         assert d["dispatches"][0]["name"] == "pad+conv3x3+relu" and d["dispatches"][-1]["name"] == "conv3x3+slice"
-        assert d["dispatches"][0]["push_constants"] == [Wp, Hp, W, H, 0, 0]
-        assert d["dispatches"][-1]["push_constants"] == [Wp, Hp, W, H, 0, 0]
+        assert d["dispatches"][0]["push_constants"] == [Wp, Hp, W, H, 0, 0, 0]
+        assert d["dispatches"][-1]["push_constants"] == [Wp, Hp, W, H, 0, 0, 1]
         u = dx.describe(dx.compile_model(m, assume={"H": H, "W": W}, features=dict(pad_fusion=False, slice_fusion=False)), H=H, W=W)
         assert u["dispatches"][0]["name"] == "pad" and u["dispatches"][-1]["name"] == "slice"
         assert u["dispatches"][0]["push_constants"] == [Wp, Hp, 0, Wp - W, 0, Hp - H]
