@@ -23,6 +23,17 @@ PEAK_FP16_MFMA_TFLOPS = 2500.0  # MI355X dense fp16, published
 PEAK_HBM_GBPS = 8000.0          # MI355X HBM3E, published
 
 
+# name -> (network, builder kwargs, H, W, interface layout, description)
+WORKLOADS = {
+    "tiny_128": ("tiny_unet", {}, 128, 128, "HWC", "tiny 2-level U-Net 3->3, fp16 HWC, 128x128"),
+    "conv64_1080p": ("single_conv", {}, 1080, 1920, "HWC", "conv3x3 64->64 + bias + ReLU, fp16 HWC, 1920x1080"),
+    "oidn_1080p": ("oidn_unet", {}, 1080, 1920, "HWC", "OIDN-style U-Net 9->3, fp16 HWC, 1920x1080, replicate-pad to multiple of 16 + crop included"),
+    "oidn_4k": ("oidn_unet", {}, 2160, 3840, "HWC", "OIDN-style U-Net 9->3, fp16 HWC, 3840x2160"),
+    "oidn2x_chw_1077": ("oidn_unet", {"width_mult": 2}, 1077, 1917, "CHW",
+                        "OIDN-style U-Net with doubled widths 9->3, fp16, CHW in/out, 1917x1077, replicate-pad to 1920x1088 + crop included"),
+}
+
+
 def lavapipe_probe() -> str:
     """The reference's own CPU route (its SPIR-V on Mesa lavapipe) needs a Vulkan loader, the
     lavapipe ICD and a built denox; report why it is unavailable rather than inventing a number."""
@@ -34,20 +45,21 @@ def lavapipe_probe() -> str:
     return "unavailable (denox itself cannot be built here: needs glslang, SPIRV-Tools, FlatBuffers)"
 
 
-def cpu_baseline(seed: int, budget_h: int = 1080, budget_w: int = 1920) -> dict:
-    """CPU oracle (fp32, OpenMP) on a crop of the benchmark frame, same network and weights."""
+def cpu_baseline(net: str, kw: dict, seed: int, budget_h: int, budget_w: int) -> dict:
+    """CPU oracle (fp32 accumulation, OpenMP over rows) on one frame of the workload (capped at 1080p), same network and weights."""
     import numpy as np
     import oracle
     from denox_amd import networks
     oracle.build()
-    model, _ = networks.build("oidn_unet", seed=seed)
-    x = networks.synthetic_input("oidn_unet", budget_h, budget_w, seed=seed)
+    budget_h, budget_w = min(budget_h, 1080), min(budget_w, 1920)
+    model, _ = networks.build(net, seed=seed, **kw)
+    x = networks.synthetic_input(net, budget_h, budget_w, seed=seed)
     ops = model.to_ops({"H": budget_h, "W": budget_w})
     t0 = time.perf_counter()
     oracle.run_graph(ops, {"input": x}, "f16")
     dt = time.perf_counter() - t0
     return {"value": budget_h * budget_w / dt * 1e-6, "unit": "Mpix/s", "cores": oracle.num_threads(), "kind": "port",
-            "sample": f"one {budget_w}x{budget_h} frame of the same U-Net, fp32 accumulation, {dt:.1f} s wall",
+            "sample": f"one {budget_w}x{budget_h} frame of the same network, fp32 accumulation, {dt:.1f} s wall",
             "lavapipe_baseline": lavapipe_probe()}
 
 
@@ -56,8 +68,10 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--height", type=int, default=1080)
-    ap.add_argument("--width", type=int, default=1920)
+    ap.add_argument("--workload", default="oidn_1080p", choices=sorted(WORKLOADS),
+                    help="oidn_1080p is the headline configuration; the others are the remaining benchmark configurations")
+    ap.add_argument("--height", type=int, default=None)
+    ap.add_argument("--width", type=int, default=None)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--per-dispatch", action="store_true", help="print the per-dispatch report to stderr")
@@ -78,8 +92,10 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         return 1
-    H, W = args.height, args.width
-    model, _ = networks.build("oidn_unet", seed=args.seed)
+    net, net_kw, H, W, layout, description = WORKLOADS[args.workload]
+    H, W = args.height or H, args.width or W
+    model, _ = networks.build(net, seed=args.seed, **net_kw)
+    lay = dx.Layout[layout]
     # The reference workflow: populate the table with every candidate dispatch, time them on
     # this GPU, then compile against the measured latencies (README.md:112-199 of the reference:
     # `denox populate`, `denox bench`, `denox compile --db`).
@@ -89,18 +105,20 @@ def main() -> int:
         import tempfile
         t0 = time.perf_counter()
         db = dx.Db(args.db or os.path.join(tempfile.mkdtemp(prefix="denox_hip_"), "gpu.db"))
-        db.populate(model, assume={"H": H, "W": W}, conv_config=args.conv_config)
+        db.populate(model, assume={"H": H, "W": W}, conv_config=args.conv_config, input_layout=lay, output_layout=lay)
         db.bench(min_samples=10, max_relative_error=0.03, max_samples=50, save_progress=bool(args.db))
         tune_s = time.perf_counter() - t0
-    blob = dx.compile_model(model, assume={"H": H, "W": W}, conv_config=args.conv_config, db=db)
+    blob = dx.compile_model(model, assume={"H": H, "W": W}, conv_config=args.conv_config, db=db, input_layout=lay, output_layout=lay)
     if args.per_dispatch:
         print(dx.last_compile_report(), file=sys.stderr)
     mod = dx.Module.load(blob)
     inst = mod.instance(H=H, W=W)
 
-    x = networks.synthetic_input("oidn_unet", H, W, seed=args.seed)
+    x = networks.synthetic_input(net, H, W, seed=args.seed)
+    if layout == "CHW":
+        x = np.ascontiguousarray(x.transpose(2, 0, 1))
     d_in = torch.from_numpy(x).cuda()
-    d_out = torch.empty((H, W, 3), dtype=torch.float16, device="cuda")
+    d_out = torch.empty(inst.output_desc()["byte_size"] // 2, dtype=torch.float16, device="cuda")
     torch.cuda.synchronize()
     ins, outs = [d_in.data_ptr()], [d_out.data_ptr()]
 
@@ -169,17 +187,16 @@ def main() -> int:
         pass
 
     line = {
-        "metric": "oidn_unet_fp16_hwc_1080p_throughput", "value": H * W / (ms * 1e-3) * 1e-6, "unit": "Mpix/s",
+        "metric": "oidn_unet_fp16_hwc_1080p_throughput" if args.workload == "oidn_1080p" else f"{args.workload}_throughput", "value": H * W / (ms * 1e-3) * 1e-6, "unit": "Mpix/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-        "config": {"workload": f"OIDN-style U-Net 9->3, fp16 HWC, {W}x{H}, replicate-pad to multiple of 16 + crop included, "
-                               f"{mod.runtime_model.dispatch_count} dispatches in one hipGraph", "device_bytes": inst.device_bytes,
+        "config": {"workload": f"{description}; {mod.runtime_model.dispatch_count} dispatches in one hipGraph", "device_bytes": inst.device_bytes,
                    "schedule": "min-cost over measured dispatch latencies" if db is not None else "min-cost over roofline estimates",
                    "tuning_seconds": round(tune_s, 2), "host_pointer_path_ms_per_frame": round(host_ms, 3)},
         "roofline": roofline,
     }
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(args.seed)
+        line["cpu_baseline"] = cpu_baseline(net, net_kw, args.seed, H, W)
     print(json.dumps(line))
     return 0
 

@@ -122,4 +122,5 @@ CACHE_WARM_CONFIGS = [
     ("tiny_unet", {}),
     ("single_conv", {}),
     ("oidn_unet", {}),
+    ("oidn_unet", {"width_mult": 2}),
 ]

@@ -1,0 +1,130 @@
+"""The reference's own system-test matrix (test/system/*.py), case for case, through the C ABI.
+
+Each reference test wraps a torch module, compiles it, runs a `torch.rand(1, C, 100, 100)` fp16 input and compares with
+torch (test/__init__.py:45-101).  Here the same layers are built with the graph builder, the same shapes and interface
+layouts are used, and the expectation comes from the CPU oracle: bit-exact for data movement, the fp32-evaluation
+tolerance for convs.
+
+  test_conv.py:126-501        conv3x3 'same', (C_in, C_out) below, HWC and CHWC8 interfaces and mixed
+  test_conv_relu.py:20-94     conv3x3 + ReLU
+  test_max_pool.py            MaxPool2d(2, 2), C in {3, 8, 9, 16, 24, 32, 48, 64, 80} HWC, {8..80} CHWC8
+  test_upsampling.py          Upsample(scale_factor=2), same channel sets
+  test_relu.py                ReLU, same channel sets
+  test_pad.py                 F.pad(x, (100, 200, 300, 400), mode="replicate")
+  test_slice.py               x[:, :, 20:40, 10:30]
+  test_concat.py              two convs of one input concatenated, 100x100 and 2x2
+  test_unet.py:16-83          6-level U-Net, replicate-pad to a multiple of 64, crop
+"""
+import numpy as np
+import pytest
+
+import denox_amd as dx
+from util import assert_bits_equal, assert_conv_close, he_weights, small_bias
+
+pytestmark = pytest.mark.gpu
+
+HWC, CHWC8 = dx.Layout.HWC, dx.Layout.CHWC8
+
+
+def to_layout(oracle, x_hwc, layout):
+    H, W, C = x_hwc.shape
+    if layout == CHWC8:
+        return oracle.relayout(x_hwc, oracle.LAYOUT_HWC, oracle.LAYOUT_CHWC8, H, W, C).reshape(C // 8, H, W, 8)
+    return x_hwc
+
+
+def from_layout(oracle, y, layout, H, W, C):
+    if layout == CHWC8:
+        return oracle.relayout(y.reshape(-1), oracle.LAYOUT_CHWC8, oracle.LAYOUT_HWC, H, W, C).reshape(H, W, C)
+    return y
+
+
+def run_case(oracle, build, C, in_layout=HWC, out_layout=HWC, H=100, W=100, exact=True, seed=0):
+    rng = np.random.default_rng(seed + C)
+    x = rng.random((H, W, C), dtype=np.float32).astype(np.float16)  # torch.rand
+    m = dx.Model()
+    t = build(m, m.input("input", "W", "H", C), rng)
+    m.output(t)
+    mod = dx.Module.compile(m, input_layout=in_layout, output_layout=out_layout)
+    inst = mod.instance(H=H, W=W)
+    got = inst.infer(to_layout(oracle, x, in_layout))[0]
+    d = inst.output_desc()
+    got = from_layout(oracle, got, out_layout, d["height"], d["width"], d["channels"])
+    want = oracle.run_graph(m.to_ops({"H": H, "W": W}), {"input": x}, "f16" if exact else "fp32")[t.name]
+    if exact:
+        assert_bits_equal(got, want)
+    else:
+        assert_conv_close(got, want)
+
+
+CONV_SHAPES = [(3, 3), (3, 32), (32, 3), (8, 16), (16, 8), (16, 32), (32, 16), (32, 32), (64, 64), (24, 24), (32, 48), (48, 48),
+               (64, 32), (64, 80), (67, 64), (80, 96), (96, 96), (112, 112), (128, 64), (160, 96), (160, 112)]
+
+
+@pytest.mark.parametrize("cin,cout", CONV_SHAPES)
+def test_conv_hwc(oracle, cin, cout):
+    run_case(oracle, lambda m, x, rng: m.conv2d(x, he_weights(rng, cout, cin), small_bias(rng, cout)), cin, exact=False)
+
+
+@pytest.mark.parametrize("cin,cout,li,lo", [(8, 16, CHWC8, CHWC8), (16, 8, CHWC8, CHWC8), (16, 32, CHWC8, CHWC8), (32, 16, CHWC8, CHWC8),
+                                            (32, 32, CHWC8, CHWC8), (64, 64, CHWC8, CHWC8), (96, 96, CHWC8, CHWC8), (128, 64, CHWC8, CHWC8),
+                                            (8, 16, HWC, CHWC8), (16, 8, CHWC8, HWC), (32, 32, HWC, CHWC8), (64, 64, CHWC8, HWC)])
+def test_conv_chwc8_and_mixed_interfaces(oracle, cin, cout, li, lo):
+    run_case(oracle, lambda m, x, rng: m.conv2d(x, he_weights(rng, cout, cin), small_bias(rng, cout)), cin, li, lo, exact=False)
+
+
+@pytest.mark.parametrize("cin,cout", [(3, 3), (3, 32), (32, 3), (8, 16), (16, 8), (16, 32), (32, 16), (32, 32), (64, 64)])
+def test_conv_relu(oracle, cin, cout):
+    run_case(oracle, lambda m, x, rng: m.relu(m.conv2d(x, he_weights(rng, cout, cin), small_bias(rng, cout))), cin, exact=False)
+
+
+HWC_CHANNELS = [3, 8, 9, 16, 24, 32, 48, 64, 80]
+CHWC8_CHANNELS = [8, 16, 24, 32, 48, 64, 80]
+
+
+@pytest.mark.parametrize("op", ["pool", "upsample", "relu"])
+@pytest.mark.parametrize("C,layout", [(c, HWC) for c in HWC_CHANNELS] + [(c, CHWC8) for c in CHWC8_CHANNELS])
+def test_pool_upsample_relu(oracle, op, C, layout):
+    build = {"pool": lambda m, x, r: m.pool(x), "upsample": lambda m, x, r: m.upsample(x), "relu": lambda m, x, r: m.relu(x)}[op]
+    run_case(oracle, build, C, layout, layout)
+
+
+@pytest.mark.parametrize("C", [3, 8, 9, 16, 24, 32, 48, 64])
+def test_pad_100_200_300_400(oracle, C):
+    run_case(oracle, lambda m, x, r: m.pad(x, 100, 200, 300, 400), C)
+
+
+@pytest.mark.parametrize("C", [3, 8, 9, 16, 24, 32, 48])
+def test_slice_20_40_10_30(oracle, C):
+    run_case(oracle, lambda m, x, r: m.slice(x, 10, 30, 20, 40), C)
+
+
+@pytest.mark.parametrize("ich,ch1,ch2,H,W", [(3, 3, 3, 100, 100), (3, 3, 4, 2, 2)])
+def test_concat_of_two_convs(oracle, ich, ch1, ch2, H, W):
+    def build(m, x, rng):
+        a = m.conv2d(x, he_weights(rng, ch1, ich), small_bias(rng, ch1))
+        b = m.conv2d(x, he_weights(rng, ch2, ich), small_bias(rng, ch2))
+        return m.concat(a, b)
+    run_case(oracle, build, ich, H=H, W=W, exact=False)
+
+
+def test_six_level_unet(oracle):
+    def build(m, inp, rng):
+        def conv(t, K):
+            return m.relu(m.conv2d(t, he_weights(rng, K, t.channels), small_bias(rng, K)))
+        a = m.pad_to_multiple(inp, 64)
+        extr = conv(a, 32)
+        x128 = m.pool(extr)
+        x64 = m.pool(conv(x128, 48))
+        x32 = m.pool(conv(x64, 64))
+        x16 = m.pool(conv(x32, 80))
+        x8 = m.pool(conv(x16, 112))
+        x4 = m.pool(conv(x8, 112))
+        x = conv(conv(m.concat(m.upsample(x4), x8), 112), 112)
+        x = conv(conv(m.concat(m.upsample(x), x16), 80), 80)
+        x = conv(conv(m.concat(m.upsample(x), x32), 64), 64)
+        x = conv(conv(m.concat(m.upsample(x), x64), 48), 48)
+        x = conv(conv(m.concat(m.upsample(x), x128), 16), 16)
+        x = conv(conv(m.concat(m.upsample(x), a), 12), 12)
+        return m.slice(x, 0, inp.width, 0, inp.height)
+    run_case(oracle, build, 3, exact=False)
