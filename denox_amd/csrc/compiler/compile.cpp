@@ -277,7 +277,9 @@ std::vector<uint8_t> compile(const Model &modelIn, const hip::HipCompiler &hipc,
     d.kernel.define("CH", n.channels); d.kernel.define("SRC_LAYOUT", layoutId(from)); d.kernel.define("DST_LAYOUT", layoutId(to));
     d.entryPoint = "relayout_c" + std::to_string(n.channels) + "_" + std::to_string(layoutId(from)) + "to" + std::to_string(layoutId(to));
     d.kernel.define("KERNEL_NAME", d.entryPoint);
-    d.workgroupCountX = sym.cdiv(sym.mul(n.width, n.height), 256);
+    // HWC <-> CHWC8 moves one 16-byte vector per thread, every other pair one pixel per thread (see relayout.hip)
+    const bool blocky = from != dnx::TensorFormat::SSBO_CHW && to != dnx::TensorFormat::SSBO_CHW && n.channels % 8 == 0;
+    d.workgroupCountX = sym.cdiv(sym.mul(sym.mul(n.width, n.height), blocky ? static_cast<int64_t>(n.channels / 8) : 1), 256);
     d.workgroupCountY = d.workgroupCountZ = Sym::Const(1);
     d.workgroupSize[0] = 256;
     TensorBinding in{0, 0, dnx::Access::ReadOnly, TensorId{external_is_source ? extId : static_cast<uint32_t>(t)}, BindingType::Input};

@@ -42,25 +42,34 @@ std::string fmtFloat(float v) {
 // weight slice of every reduction step through LDS (any layer size), conv3x3_mfma_ws.hip
 // keeps the whole slice resident and runs persistently (layers whose weights fit LDS).
 // waves: computing waves; pw: extra staging-only waves (wave specialisation, resident kernel only)
-struct ConvConfig { unsigned waves, rpw, ck; bool resident; unsigned pw; unsigned maxKT; const char *name; };
+// waves: computing waves; rpw: image rows per wave; ck: input channels per LDS step (0 = all, 1 = half);
+// resident: weights stay in LDS (persistent launch); pw: extra staging-only waves; maxKT: cap on output channels
+// per workgroup (0 = none); mf: matrix shape 32 (32x32x16) or 16 (16x16x32); xb: 16-pixel blocks per row (mf 16).
+struct ConvConfig { unsigned waves, rpw, ck; bool resident; unsigned pw; unsigned maxKT; unsigned mf, xb; const char *name; };
 const ConvConfig kConvConfigs[] = {
     // weights streamed per step
-    {4, 2, 16, false, 0, 0, "w4r2k16"}, {4, 2, 32, false, 0, 0, "w4r2k32"}, {4, 4, 16, false, 0, 0, "w4r4k16"}, {4, 4, 32, false, 0, 0, "w4r4k32"},
-    {8, 2, 16, false, 0, 0, "w8r2k16"}, {8, 2, 32, false, 0, 0, "w8r2k32"}, {4, 2, 64, false, 0, 0, "w4r2k64"}, {8, 1, 16, false, 0, 0, "w8r1k16"},
+    {4, 2, 16, false, 0, 0, 32, 1, "w4r2k16"}, {4, 2, 32, false, 0, 0, 32, 1, "w4r2k32"}, {4, 4, 16, false, 0, 0, 32, 1, "w4r4k16"}, {4, 4, 32, false, 0, 0, 32, 1, "w4r4k32"},
+    {8, 2, 16, false, 0, 0, 32, 1, "w8r2k16"}, {8, 2, 32, false, 0, 0, 32, 1, "w8r2k32"}, {4, 2, 64, false, 0, 0, 32, 1, "w4r2k64"}, {8, 1, 16, false, 0, 0, 32, 1, "w8r1k16"},
     // small tiles / one 32-channel block per workgroup: more workgroups for low-resolution layers
-    {4, 1, 16, false, 0, 0, "w4r1k16"}, {4, 1, 32, false, 0, 0, "w4r1k32"}, {4, 1, 32, false, 0, 32, "w4r1k32n"}, {4, 2, 32, false, 0, 32, "w4r2k32n"},
-    {2, 2, 32, false, 0, 32, "w2r2k32n"}, {2, 2, 32, false, 0, 0, "w2r2k32"},
+    {4, 1, 16, false, 0, 0, 32, 1, "w4r1k16"}, {4, 1, 32, false, 0, 0, 32, 1, "w4r1k32"}, {4, 1, 32, false, 0, 32, 32, 1, "w4r1k32n"}, {4, 2, 32, false, 0, 32, 32, 1, "w4r2k32n"},
+    {2, 2, 32, false, 0, 32, 32, 1, "w2r2k32n"}, {2, 2, 32, false, 0, 0, 32, 1, "w2r2k32"},
     // ck = 0: the whole reduction (or half of it, ck = 1) in one step -- a single round of global loads per workgroup,
     // for layers with so few tiles that load latency, not throughput, is what a workgroup waits for
-    {4, 1, 0, false, 0, 32, "w4r1kfn"}, {4, 1, 1, false, 0, 32, "w4r1khn"}, {4, 2, 0, false, 0, 32, "w4r2kfn"}, {2, 2, 0, false, 0, 32, "w2r2kfn"},
-    {4, 1, 0, false, 0, 64, "w4r1kfm"}, {4, 2, 1, false, 0, 32, "w4r2khn"},
+    {4, 1, 0, false, 0, 32, 32, 1, "w4r1kfn"}, {4, 1, 1, false, 0, 32, 32, 1, "w4r1khn"}, {4, 2, 0, false, 0, 32, 32, 1, "w4r2kfn"}, {2, 2, 0, false, 0, 32, 32, 1, "w2r2kfn"},
+    {4, 1, 0, false, 0, 64, 32, 1, "w4r1kfm"}, {4, 2, 1, false, 0, 32, 32, 1, "w4r2khn"},
     // weights resident, persistent launch
-    {8, 1, 16, true, 0, 0, "p8r1k16"},  {8, 1, 32, true, 0, 0, "p8r1k32"},  {16, 1, 16, true, 0, 0, "p16r1k16"}, {16, 1, 32, true, 0, 0, "p16r1k32"},
-    {8, 2, 16, true, 0, 0, "p8r2k16"},  {8, 2, 32, true, 0, 0, "p8r2k32"},  {16, 2, 16, true, 0, 0, "p16r2k16"}, {4, 2, 32, true, 0, 0, "p4r2k32"},
-    {8, 4, 16, true, 0, 0, "p8r4k16"},  {4, 4, 16, true, 0, 0, "p4r4k16"},  {4, 4, 32, true, 0, 0, "p4r4k32"},   {4, 1, 32, true, 0, 0, "p4r1k32"},
-    {4, 2, 32, true, 0, 32, "p4r2k32n"}, {4, 1, 32, true, 0, 32, "p4r1k32n"},
+    {8, 1, 16, true, 0, 0, 32, 1, "p8r1k16"},  {8, 1, 32, true, 0, 0, 32, 1, "p8r1k32"},  {16, 1, 16, true, 0, 0, 32, 1, "p16r1k16"}, {16, 1, 32, true, 0, 0, 32, 1, "p16r1k32"},
+    {8, 2, 16, true, 0, 0, 32, 1, "p8r2k16"},  {8, 2, 32, true, 0, 0, 32, 1, "p8r2k32"},  {16, 2, 16, true, 0, 0, 32, 1, "p16r2k16"}, {4, 2, 32, true, 0, 0, 32, 1, "p4r2k32"},
+    {8, 4, 16, true, 0, 0, 32, 1, "p8r4k16"},  {4, 4, 16, true, 0, 0, 32, 1, "p4r4k16"},  {4, 4, 32, true, 0, 0, 32, 1, "p4r4k32"},   {4, 1, 32, true, 0, 0, 32, 1, "p4r1k32"},
+    {4, 2, 32, true, 0, 32, 32, 1, "p4r2k32n"}, {4, 1, 32, true, 0, 32, 32, 1, "p4r1k32n"},
     // resident + staging-only waves
-    {8, 2, 16, true, 4, 0, "s8r2k16"},  {12, 1, 16, true, 4, 0, "s12r1k16"},
+    {8, 2, 16, true, 4, 0, 32, 1, "s8r2k16"},  {12, 1, 16, true, 4, 0, 32, 1, "s12r1k16"},
+    // 16x16x32 matrix shape: output channels in blocks of 16, tiles of 16 or 32 pixels width
+    {4, 2, 32, false, 0, 0, 16, 2, "m4r2k32x2"}, {4, 2, 64, false, 0, 0, 16, 2, "m4r2k64x2"}, {4, 1, 32, false, 0, 0, 16, 2, "m4r1k32x2"}, {4, 2, 32, false, 0, 0, 16, 1, "m4r2k32x1"},
+    {4, 4, 32, false, 0, 0, 16, 1, "m4r4k32x1"}, {8, 2, 32, false, 0, 0, 16, 2, "m8r2k32x2"}, {4, 2, 0, false, 0, 0, 16, 1, "m4r2kfx1"},  {4, 1, 0, false, 0, 0, 16, 2, "m4r1kfx2"},
+    {4, 2, 32, false, 0, 32, 16, 2, "m4r2k32x2n"}, {4, 2, 0, false, 0, 32, 16, 1, "m4r2kfx1n"}, {4, 1, 0, false, 0, 48, 16, 1, "m4r1kfx1n"}, {4, 2, 32, false, 0, 48, 16, 1, "m4r2k32x1n"},
+    {8, 2, 32, true, 0, 0, 16, 2, "q8r2k32x2"}, {8, 1, 32, true, 0, 0, 16, 2, "q8r1k32x2"}, {4, 2, 32, true, 0, 0, 16, 2, "q4r2k32x2"}, {8, 2, 32, true, 0, 0, 16, 1, "q8r2k32x1"},
+    {8, 2, 64, true, 0, 0, 16, 2, "q8r2k64x2"}, {4, 2, 32, true, 0, 48, 16, 1, "q4r2k32x1n"},
 };
 constexpr unsigned kNumConvConfigs = sizeof(kConvConfigs) / sizeof(kConvConfigs[0]);
 
@@ -76,31 +85,37 @@ struct ConvGeometry {
 // register file.
 // channels per LDS step of a configuration for a layer with `cpad` padded input channels
 unsigned stepChannels(const ConvConfig &cfg, unsigned cpad) {
-  if (cfg.ck == 0) return cpad;                                  // everything at once
-  if (cfg.ck == 1) return std::max(16u, (cpad / 2 + 15) / 16 * 16); // two steps
+  const unsigned kstep = cfg.mf == 32 ? 16 : 32;
+  if (cfg.ck == 0) return cpad;                                              // everything at once
+  if (cfg.ck == 1) return std::max(kstep, (cpad / 2 + kstep - 1) / kstep * kstep); // two steps
   return cfg.ck;
 }
 
+// Output channels per workgroup: the largest divisor of KOUTP (in blocks of mf channels)
+// whose weights fit LDS next to the halo(s) and whose accumulators fit the register file.
 bool chooseKT(const ConvConfig &cfgIn, unsigned CA, unsigned CB, unsigned K, const DeviceInfo &dev, ConvGeometry &g) {
-  g.CA = CA; g.CB = CB; g.C = CA + CB; g.CPAD = (g.C + 15) / 16 * 16; g.K = K; g.KOUTP = (K + 31) / 32 * 32;
+  const unsigned blk = cfgIn.mf, kstep = cfgIn.mf == 32 ? 16 : 32;
+  g.CA = CA; g.CB = CB; g.C = CA + CB; g.CPAD = (g.C + kstep - 1) / kstep * kstep; g.K = K; g.KOUTP = (K + blk - 1) / blk * blk;
   ConvConfig cfg = cfgIn;
   cfg.ck = stepChannels(cfgIn, g.CPAD);
-  if (cfg.ck > 192) return false; // staging registers
+  if (cfg.ck > 192 || cfg.ck % kstep) return false; // staging registers; whole matrix steps only
   const unsigned th = cfg.waves * cfg.rpw;
-  const unsigned haloPix = (th + 2) * 34;
+  const unsigned tw = cfg.mf == 32 ? 32 : 16 * cfg.xb;
+  const unsigned haloPix = (th + 2) * (tw + 2);
   const unsigned ckp = cfg.ck + 8;
-  const unsigned blocks = g.KOUTP / 32;
+  const unsigned blocks = g.KOUTP / blk;
   // registers per lane: 512 shared by the waves of one SIMD; a workgroup of `waves` waves puts waves/4 on each
   const unsigned wavesPerSimd = (cfg.waves + cfg.pw + 3) / 4;
   const unsigned regBudget = std::min(256u, 512u / wavesPerSimd);
   for (unsigned kb = blocks; kb >= 1; --kb) {
     if (blocks % kb) continue;
-    if (cfg.maxKT && kb * 32 > cfg.maxKT) continue;
-    if (kb * cfg.rpw * 16 + 64 > regBudget) continue;
-    const size_t lds = cfg.resident ? static_cast<size_t>(9u * kb * 32u) * (g.CPAD + 8) * 2u + 2u * static_cast<size_t>(haloPix) * ckp * 2u
-                                    : (static_cast<size_t>(haloPix) + 9u * kb * 32u) * ckp * 2u;
+    if (cfg.maxKT && kb * blk > cfg.maxKT) continue;
+    const unsigned accRegs = cfg.mf == 32 ? kb * cfg.rpw * 16 : kb * cfg.rpw * cfg.xb * 4;
+    if (accRegs + 64 + (cfg.mf == 16 ? kb * 4 : 0) > regBudget) continue;
+    const size_t lds = cfg.resident ? static_cast<size_t>(9u * kb * blk) * (g.CPAD + 8) * 2u + 2u * static_cast<size_t>(haloPix) * ckp * 2u
+                                    : (static_cast<size_t>(haloPix) + 9u * kb * blk) * ckp * 2u;
     if (lds > dev.maxComputeSharedMemory) continue;
-    g.KT = kb * 32;
+    g.KT = kb * blk;
     g.ldsBytes = lds;
     const unsigned nkt = blocks / kb;
     g.slots = std::max(1u, dev.computeUnits / (dev.xcdCount * nkt));
@@ -109,11 +124,22 @@ bool chooseKT(const ConvConfig &cfgIn, unsigned CA, unsigned CB, unsigned K, con
   return false;
 }
 
+// Which output channel a weight row of a workgroup's KT rows computes (the inverse of the
+// lane -> channel assignment of the kernels' epilogues).
+unsigned rowChannel(unsigned mf, unsigned KT, unsigned row) {
+  if (mf == 32) {
+    const unsigned rho = row & 31;
+    return (row & ~31u) + 16 * ((rho >> 2) & 1) + 4 * (rho >> 3) + (rho & 3);
+  }
+  const unsigned kb = row / 16, rho = row % 16, grp = rho / 4, jj = rho % 4, nblocks = KT / 16;
+  const bool paired = 2 * (kb / 2) + 1 < nblocks;
+  return paired ? 32 * (kb / 2) + 8 * grp + 4 * (kb % 2) + jj : 16 * kb + 4 * grp + jj;
+}
+
 // Weight layout the kernels read: [kt][chunk][tap r*3+s][KT rows][len(chunk)], rows
-// permuted so that MFMA row rho of a 32-block holds output channel
-// 16*((rho>>2)&1) + 4*(rho>>3) + (rho&3) of that block; zero for c >= C or k >= K.
+// permuted by rowChannel(); zero for c >= C or k >= K.
 // (The resident kernel uses one chunk spanning the whole reduction.)
-std::vector<uint8_t> packConvWeights(const Op &conv, const ConvGeometry &g, unsigned ck) {
+std::vector<uint8_t> packConvWeights(const Op &conv, const ConvGeometry &g, unsigned ck, unsigned mf) {
   std::vector<uint16_t> out(static_cast<size_t>(g.KOUTP) * 9 * g.CPAD, 0);
   const unsigned nkt = g.KOUTP / g.KT;
   size_t pos = 0;
@@ -123,8 +149,7 @@ std::vector<uint8_t> packConvWeights(const Op &conv, const ConvGeometry &g, unsi
       for (unsigned tap = 0; tap < 9; ++tap) {
         const unsigned r = tap / 3, s = tap % 3;
         for (unsigned row = 0; row < g.KT; ++row) {
-          const unsigned rho = row & 31;
-          const unsigned k = kt * g.KT + (row & ~31u) + 16 * ((rho >> 2) & 1) + 4 * (rho >> 3) + (rho & 3);
+          const unsigned k = kt * g.KT + rowChannel(mf, g.KT, row);
           for (unsigned e = 0; e < len; ++e, ++pos) {
             const unsigned c = c0 + e;
             if (k < g.K && c < g.C) out[pos] = conv.weights[((static_cast<size_t>(k) * g.C + c) * 3 + r) * 3 + s];
@@ -223,12 +248,13 @@ public:
     const Op &conv = opOf(model, m, OpKind::Conv);
     const unsigned CA = model.tensors()[m.inputs[0]].channels;
     const unsigned CB = m.inputs.size() > 1 ? model.tensors()[m.inputs[1]].channels : 0;
-    const unsigned cpad = (CA + CB + 15) / 16 * 16;
     std::vector<unsigned> out;
     for (unsigned c = 0; c < kNumConvConfigs; ++c) {
       const ConvConfig &cfg = kConvConfigs[c];
+      const unsigned kstep = cfg.mf == 32 ? 16 : 32;
+      const unsigned cpad = (CA + CB + kstep - 1) / kstep * kstep;
       if (!opt.forceConvConfig.empty() && opt.forceConvConfig != cfg.name) continue;
-      if (cfg.ck > cpad && cfg.ck != 16) continue; // a larger stage than the whole reduction adds nothing
+      if (cfg.ck > cpad && cfg.ck != kstep) continue; // a larger stage than the whole reduction adds nothing
       if (cfg.ck <= 1 && cpad <= 32) continue;     // "whole / half reduction" duplicates a fixed-size stage for narrow layers
       if ((m.pattern & PAT_POOL) && (cfg.rpw % 2)) continue;
       if ((cfg.waves + cfg.pw) * 64 > opt.deviceInfo.maxComputeWorkGroupInvocations) continue;
@@ -242,7 +268,7 @@ public:
 
   size_t parameterMemorySize(const Model &model, const Match &m) const override {
     const Op &conv = opOf(model, m, OpKind::Conv);
-    const unsigned C = conv.C, cpad = (C + 15) / 16 * 16, kp = (conv.K + 31) / 32 * 32;
+    const unsigned C = conv.C, cpad = (C + 31) / 32 * 32, kp = (conv.K + 31) / 32 * 32; // upper bound over configurations
     return static_cast<size_t>(kp) * 9 * cpad * 2 + static_cast<size_t>(kp) * 2;
   }
 
@@ -277,6 +303,7 @@ public:
     k.define("WAVES", cfg.waves); k.define("RPW", cfg.rpw); k.define("CK", stepChannels(cfg, g.CPAD));
     if (cfg.resident) k.define("SLOTS", g.slots);
     if (cfg.pw) k.define("PW", cfg.pw);
+    if (cfg.mf != 32) { k.define("MF", cfg.mf); k.define("XB", cfg.xb); }
     std::string entry = "conv3x3_c" + std::to_string(CA) + (up ? "u" : "") + (padA ? "e" : "") + (CB ? "p" + std::to_string(CB) + (padB ? "e" : "") : "") + "_k" +
                         std::to_string(conv.K) + (act == 1 ? "_relu" : act == 2 ? "_lrelu" : "") + (pool ? "_pool" : "") + (crop ? "_crop" : "") + "_" + cfg.name;
     k.define("KERNEL_NAME", entry);
@@ -284,14 +311,14 @@ public:
     const unsigned th = cfg.waves * cfg.rpw;
     const unsigned nkt = g.KOUTP / g.KT;
     auto d = cfg.resident ? impl.registerDispatch(k, entry, Sym::Const(opt.deviceInfo.xcdCount * nkt * g.slots), Sym::Const(1), Sym::Const(1), (cfg.waves + cfg.pw) * 64)
-                          : impl.registerDispatch(k, entry, sym.cdiv(W, 32), sym.cdiv(H, th), Sym::Const(nkt), cfg.waves * 64);
+                          : impl.registerDispatch(k, entry, sym.cdiv(W, cfg.mf == 32 ? 32 : 16 * cfg.xb), sym.cdiv(H, th), Sym::Const(nkt), cfg.waves * 64);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     if (CB) d.addBinding(dnx::Access::ReadOnly, m.inputs[1]);
     d.addBinding(dnx::Access::WriteOnly, m.output);
     const Op convCopy = conv; // the lazy packers outlive the model reference
     const unsigned ck = cfg.resident ? g.CPAD : stepChannels(cfg, g.CPAD);
     TensorId wt = impl.createParameter(static_cast<size_t>(g.KOUTP) * 9 * g.CPAD * 2, dnx::ScalarType::F16,
-                                       [convCopy, g, ck]() { return packConvWeights(convCopy, g, ck); });
+                                       [convCopy, g, ck, mf = cfg.mf]() { return packConvWeights(convCopy, g, ck, mf); });
     d.addParamBinding(wt);
     if (conv.hasBias) {
       const unsigned koutp = g.KOUTP;

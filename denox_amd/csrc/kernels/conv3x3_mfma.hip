@@ -76,7 +76,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   const int y0 = (rev ? tilesY - 1 - (int)DNX_BID_Y : (int)DNX_BID_Y) * TH;
   const int kt = DNX_BID_Z; // output-channel tile
 
-  float16v acc[KB][RPW];
+  Acc acc;
   zero_acc(acc);
 
   // packed filter: [kt][chunk][tap][KT][len(chunk)]

@@ -65,6 +65,9 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   int tile = first + slot;
   if (tile >= last)
     return; // uniform for the workgroup: nothing was staged yet
+#ifdef DBG_STAGGER // timing experiment: de-synchronise the workgroups at the start
+  for (int i = 0; i < ((b / NXCD) % 8); ++i) __builtin_amdgcn_s_sleep(DBG_STAGGER);
+#endif
   const bool rev = (pc.FLAGS & 1u) != 0;
   // position of the t-th tile of the walk
   auto tileY = [&](int t) { return ((rev ? numTiles - 1 - t : t) / tilesX) * TH; };
@@ -102,7 +105,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
 #if PW == 0
   H::map_init(map, tid);
   H::src_init(fsrc, map, tileY(ftile), tileX(ftile), pc);
-  float16v acc[KB][RPW];
+  Acc acc;
   int cchunk = 0, buf = 0;
   auto step = [&](H::Regs &regs) {
     if (cchunk == 0)
@@ -166,7 +169,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     }
   } else {
     // ---- computing waves ----
-    float16v acc[KB][RPW];
+    Acc acc;
     int cchunk = 0;
     for (int g = 0; g < steps; ++g) {
       if (cchunk == 0)

@@ -25,6 +25,7 @@
 #include "prelude.h"
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float float16v __attribute__((ext_vector_type(16)));
+typedef float float4v __attribute__((ext_vector_type(4)));
 typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
 typedef unsigned short ushort_t;
 
@@ -41,22 +42,33 @@ typedef unsigned short ushort_t;
 #define CROP 0
 #endif
 
+// Matrix-core shape: MF = 32 -> v_mfma_f32_32x32x16_f16 (32 output channels x 32 pixels per block, 16 input
+// channels per step), MF = 16 -> v_mfma_f32_16x16x32_f16 (16 x 16 per block, 32 input channels per step; XB blocks
+// side by side in x).  The 16-wide shape wastes less on output-channel counts like 48, 80, 112 or 3 and makes
+// smaller tiles for low-resolution layers; the 32-wide shape pads input channels less (73 -> 80 instead of 96).
+#ifndef MF
+#define MF 32
+#endif
+#ifndef XB
+#define XB 1
+#endif
+#define KSTEP (MF == 32 ? 16 : 32) // input channels per matrix instruction
 #define CIN (CA + CB)
-#define CPAD (((CIN) + 15) / 16 * 16)
+#define CPAD (((CIN) + KSTEP - 1) / KSTEP * KSTEP)
 #define NCHUNK ((CPAD + CK - 1) / CK)
 #define TAIL (CPAD - (NCHUNK - 1) * CK)
-#define TW 32
+#define TW (MF == 32 ? 32 : 16 * XB)
 #define TH (WAVES * RPW)
 #define HALO_W (TW + 2)
 #define HALO_H (TH + 2)
 #define HALO_PIX (HALO_W * HALO_H)
 #define CKP (CK + 8)
-#define KB (KT / 32)
+#define KB (KT / MF)
 #ifndef PW
 #define PW 0 // extra waves that only stage halos (weight-stationary kernel)
 #endif
 #define NT ((WAVES + PW) * 64)
-#define KOUTP (((KOUT) + 31) / 32 * 32)
+#define KOUTP (((KOUT) + MF - 1) / MF * MF)
 
 struct PushConstants {
   unsigned int IN_W;
@@ -290,10 +302,16 @@ __device__ DNX_INLINE void store16(_Float16 *dst, const half8 (&o)[2], int chb) 
   }
 }
 
+#if MF == 32
+// ---- 32 x 32 x 16 shape ----------------------------------------------------------------------------------
+struct Acc {
+  float16v v[KB][RPW];
+};
+
 // Epilogue of one wave: acc[kb][j] holds, for output row y0 + wv*RPW + j and pixel
 // x0 + (lane & 31), the 16 channels kt*KT + kb*32 + (lane >> 5)*16 + i.
 __device__ DNX_INLINE void
-store_tile(const float16v (&acc)[KB][RPW], _Float16 *__restrict__ OUT, const _Float16 *__restrict__ BIAS,
+store_tile(const Acc &acc, _Float16 *__restrict__ OUT, const _Float16 *__restrict__ BIAS,
            int y0, int x0, int kt, int wv, int lane, const PushConstants &pc) {
   const unsigned W = pc.IN_W, H = pc.IN_H;
   const int l32 = lane & 31;
@@ -319,8 +337,8 @@ store_tile(const float16v (&acc)[KB][RPW], _Float16 *__restrict__ OUT, const _Fl
       half8 o[2];
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const _Float16 v0 = (_Float16)apply_act(acc[kb][j][i] + bias[i]);
-        const _Float16 v1 = (_Float16)apply_act(acc[kb][j + 1][i] + bias[i]);
+        const _Float16 v0 = (_Float16)apply_act(acc.v[kb][j][i] + bias[i]);
+        const _Float16 v1 = (_Float16)apply_act(acc.v[kb][j + 1][i] + bias[i]);
         const _Float16 n0 = __builtin_bit_cast(_Float16, dpp_xor1(__builtin_bit_cast(ushort_t, v0)));
         const _Float16 n1 = __builtin_bit_cast(_Float16, dpp_xor1(__builtin_bit_cast(ushort_t, v1)));
         // window order (0,0) (0,1) (1,0) (1,1); replace only on strictly greater
@@ -341,7 +359,7 @@ store_tile(const float16v (&acc)[KB][RPW], _Float16 *__restrict__ OUT, const _Fl
       half8 o[2];
 #pragma unroll
       for (int i = 0; i < 16; ++i)
-        o[i >> 3][i & 7] = (_Float16)apply_act(acc[kb][j][i] + bias[i]);
+        o[i >> 3][i & 7] = (_Float16)apply_act(acc.v[kb][j][i] + bias[i]);
 #if CROP
       const int oy = y - (int)pc.CROP_T, ox = x - (int)pc.CROP_L;
       if (y < (int)H && x < (int)W && oy >= 0 && oy < (int)pc.OUT_H && ox >= 0 && ox < (int)pc.OUT_W)
@@ -365,7 +383,7 @@ store_tile(const float16v (&acc)[KB][RPW], _Float16 *__restrict__ OUT, const _Fl
 // offset of this chunk inside a weight row.
 template <int L, int WPITCH>
 __device__ DNX_INLINE void
-mma_chunk(const _Float16 *sIn, const _Float16 *sW, int wofs, float16v (&acc)[KB][RPW], int wv, int lane) {
+mma_chunk(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, int wv, int lane) {
   const int l32 = lane & 31;
   const int kq = (lane >> 5) * 8;
 #pragma unroll
@@ -388,31 +406,180 @@ mma_chunk(const _Float16 *sIn, const _Float16 *sW, int wofs, float16v (&acc)[KB]
 #pragma unroll
           for (int j = 0; j < RPW; ++j)
 #ifndef DBG_SKIP_MMA
-            acc[kb][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[kb], px[j + r], acc[kb][j], 0, 0, 0);
+            acc.v[kb][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[kb], px[j + r], acc.v[kb][j], 0, 0, 0);
 #else
-            acc[kb][j][0] += (float)wf[kb][0] * (float)px[j + r][0]; // keeps the LDS reads alive without matrix work
+            acc.v[kb][j][0] += (float)wf[kb][0] * (float)px[j + r][0]; // keeps the LDS reads alive without matrix work
 #endif
       }
     }
   }
 }
 
-// mma_chunk for step `chunk` of a tile, whichever length that step has
-template <int WPITCH>
-__device__ DNX_INLINE void
-mma_step(const _Float16 *sIn, const _Float16 *sW, int wofs, float16v (&acc)[KB][RPW], int wv, int lane, int chunk) {
-  if (TAIL == CK || chunk < NCHUNK - 1)
-    mma_chunk<CK, WPITCH>(sIn, sW, wofs, acc, wv, lane);
-  else
-    mma_chunk<TAIL, WPITCH>(sIn, sW, wofs, acc, wv, lane);
-}
-
-__device__ DNX_INLINE void zero_acc(float16v (&acc)[KB][RPW]) {
+__device__ DNX_INLINE void zero_acc(Acc &acc) {
 #pragma unroll
   for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
     for (int j = 0; j < RPW; ++j)
 #pragma unroll
       for (int i = 0; i < 16; ++i)
-        acc[kb][j][i] = 0.0f;
+        acc.v[kb][j][i] = 0.0f;
 }
+
+#else
+// ---- 16 x 16 x 32 shape ----------------------------------------------------------------------------------
+// acc.v[kb][j][xb] holds, for output row y0 + wv*RPW + j and pixel x0 + xb*16 + (lane & 15), four channels of
+// 16-channel block kb.  Blocks are paired (kb = 2p, 2p+1) and their rows permuted on the host so that lane group
+// g = lane >> 4 owns the 8 consecutive channels 32p + 8g .. + 7 (one 16-byte store); an unpaired last block
+// gives 4 consecutive channels 16kb + 4g .. + 3.
+struct Acc {
+  float4v v[KB][RPW][XB];
+};
+
+__device__ DNX_INLINE void store_vec(_Float16 *dst, const _Float16 (&o)[8], int chb, int n) {
+  // n = 8 or 4 consecutive channels starting at chb
+  if (KOUT % 8 == 0 && n == 8) {
+    if (chb < KOUT) {
+      half8 h;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) h[i] = o[i];
+      *reinterpret_cast<half8 *>(dst) = h;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (i < n && chb + i < KOUT) dst[i] = o[i];
+  }
+}
+
+__device__ DNX_INLINE void
+store_tile(const Acc &acc, _Float16 *__restrict__ OUT, const _Float16 *__restrict__ BIAS,
+           int y0, int x0, int kt, int wv, int lane, const PushConstants &pc) {
+  const unsigned W = pc.IN_W, H = pc.IN_H;
+  const int l16 = lane & 15;
+  const int g = lane >> 4;
+#pragma unroll
+  for (int kp = 0; kp < (KB + 1) / 2; ++kp) {
+    const bool paired = 2 * kp + 1 < KB;
+    const int n = paired ? 8 : 4;
+    const int chb = kt * KT + (paired ? 32 * kp + 8 * g : 16 * (2 * kp) + 4 * g);
+    float bias[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+#if HAS_BIAS
+      bias[i] = i < n ? (float)BIAS[chb + i] : 0.0f; // the bias buffer is zero-padded to KOUTP
+#else
+      bias[i] = 0.0f;
+#endif
+    }
+#pragma unroll
+    for (int xb = 0; xb < XB; ++xb) {
+      const int x = x0 + xb * 16 + l16;
+#if POOL
+      const unsigned WP = W >> 1, HP = H >> 1;
+#pragma unroll
+      for (int j = 0; j < RPW; j += 2) {
+        const int y = y0 + wv * RPW + j;
+        _Float16 o[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int kb = 2 * kp + (i >> 2);
+          if (i < n) {
+            const _Float16 v0 = (_Float16)apply_act(acc.v[kb < KB ? kb : 0][j][xb][i & 3] + bias[i]);
+            const _Float16 v1 = (_Float16)apply_act(acc.v[kb < KB ? kb : 0][j + 1][xb][i & 3] + bias[i]);
+            const _Float16 n0 = __builtin_bit_cast(_Float16, dpp_xor1(__builtin_bit_cast(ushort_t, v0)));
+            const _Float16 n1 = __builtin_bit_cast(_Float16, dpp_xor1(__builtin_bit_cast(ushort_t, v1)));
+            _Float16 m = v0; // window order (0,0) (0,1) (1,0) (1,1); replace only on strictly greater
+            m = n0 > m ? n0 : m;
+            m = v1 > m ? v1 : m;
+            m = n1 > m ? n1 : m;
+            o[i] = m;
+          } else {
+            o[i] = (_Float16)0.0f;
+          }
+        }
+        const unsigned py = (unsigned)y >> 1, px = (unsigned)x >> 1;
+        if ((l16 & 1) == 0 && py < HP && px < WP)
+          store_vec(OUT + ((size_t)py * WP + px) * KOUT + chb, o, chb, n);
+      }
+#else
+#pragma unroll
+      for (int j = 0; j < RPW; ++j) {
+        const int y = y0 + wv * RPW + j;
+        _Float16 o[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int kb = 2 * kp + (i >> 2);
+          o[i] = i < n ? (_Float16)apply_act(acc.v[kb < KB ? kb : 0][j][xb][i & 3] + bias[i]) : (_Float16)0.0f;
+        }
+#if CROP
+        const int oy = y - (int)pc.CROP_T, ox = x - (int)pc.CROP_L;
+        if (y < (int)H && x < (int)W && oy >= 0 && oy < (int)pc.OUT_H && ox >= 0 && ox < (int)pc.OUT_W)
+          store_vec(OUT + ((size_t)oy * pc.OUT_W + ox) * KOUT + chb, o, chb, n);
+#else
+        if (y < (int)H && x < (int)W)
+          store_vec(OUT + ((size_t)y * W + x) * KOUT + chb, o, chb, n);
+#endif
+      }
+#endif
+    }
+  }
+}
+
+// 9 taps x (L/32) reduction steps; lane = (pixel or weight row) lane & 15, k group lane >> 4.
+template <int L, int WPITCH>
+__device__ DNX_INLINE void
+mma_chunk(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, int wv, int lane) {
+  const int l16 = lane & 15;
+  const int kq = (lane >> 4) * 8;
+#pragma unroll
+  for (int s = 0; s < 3; ++s) {
+#pragma unroll
+    for (int ks = 0; ks < L / 32; ++ks) {
+      const int kk = ks * 32 + kq;
+      half8 px[RPW + 2][XB];
+#pragma unroll
+      for (int hr = 0; hr < RPW + 2; ++hr)
+#pragma unroll
+        for (int xb = 0; xb < XB; ++xb)
+          px[hr][xb] = *reinterpret_cast<const half8 *>(sIn + ((wv * RPW + hr) * HALO_W + xb * 16 + l16 + s) * CKP + kk);
+#pragma unroll
+      for (int r = 0; r < 3; ++r) {
+        half8 wf[KB];
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+          wf[kb] = *reinterpret_cast<const half8 *>(sW + (((r * 3 + s) * KT) + kb * 16 + l16) * WPITCH + wofs + kk);
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+          for (int j = 0; j < RPW; ++j)
+#pragma unroll
+            for (int xb = 0; xb < XB; ++xb)
+              acc.v[kb][j][xb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[kb], px[j + r][xb], acc.v[kb][j][xb], 0, 0, 0);
+      }
+    }
+  }
+}
+
+__device__ DNX_INLINE void zero_acc(Acc &acc) {
+#pragma unroll
+  for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+    for (int j = 0; j < RPW; ++j)
+#pragma unroll
+      for (int xb = 0; xb < XB; ++xb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          acc.v[kb][j][xb][i] = 0.0f;
+}
+#endif // MF
+
+// mma_chunk for step `chunk` of a tile, whichever length that step has
+template <int WPITCH>
+__device__ DNX_INLINE void
+mma_step(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, int wv, int lane, int chunk) {
+  if (TAIL == CK || chunk < NCHUNK - 1)
+    mma_chunk<CK, WPITCH>(sIn, sW, wofs, acc, wv, lane);
+  else
+    mma_chunk<TAIL, WPITCH>(sIn, sW, wofs, acc, wv, lane);
+}
+

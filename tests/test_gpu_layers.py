@@ -47,7 +47,12 @@ def test_conv3x3(oracle, C, K, H, W, act):
 
 ALL_CONFIGS = ["w4r2k16", "w4r2k32", "w4r4k16", "w4r4k32", "w8r2k16", "w8r2k32", "w4r2k64", "w8r1k16", "w4r1k16", "w4r1k32",
                "w4r1k32n", "w4r2k32n", "w2r2k32n", "w2r2k32", "p8r1k16", "p8r1k32", "p16r1k16", "p16r1k32", "p8r2k16", "p8r2k32",
-               "p16r2k16", "p4r2k32", "p8r4k16", "p4r4k16", "p4r4k32", "p4r1k32", "p4r2k32n", "p4r1k32n", "s8r2k16", "s12r1k16"]
+               "p16r2k16", "p4r2k32", "p8r4k16", "p4r4k16", "p4r4k32", "p4r1k32", "p4r2k32n", "p4r1k32n", "s8r2k16", "s12r1k16",
+               "w4r1kfn", "w4r1khn", "w4r2kfn", "w2r2kfn", "w4r1kfm", "w4r2khn"]
+# the 16x16x32 matrix shape: output channels in blocks of 16, tiles 16 or 32 pixels wide
+M16_CONFIGS = ["m4r2k32x2", "m4r2k64x2", "m4r1k32x2", "m4r2k32x1", "m4r4k32x1", "m8r2k32x2", "m4r2kfx1", "m4r1kfx2", "m4r2k32x2n",
+               "m4r2kfx1n", "m4r1kfx1n", "m4r2k32x1n", "q8r2k32x2", "q8r1k32x2", "q4r2k32x2", "q8r2k32x1", "q8r2k64x2", "q4r2k32x1n"]
+ALL_CONFIGS += M16_CONFIGS
 
 
 @pytest.mark.parametrize("config", ALL_CONFIGS)
@@ -66,6 +71,35 @@ def test_conv_every_configuration(oracle, config, C, K, H, W):
         pytest.skip(str(e))
     assert config in dx.last_compile_report()
     want = oracle.run_graph(m.to_ops({"H": H, "W": W}), {"input": x}, "fp32")[t.name]
+    assert_conv_close(got, want, config)
+
+
+@pytest.mark.parametrize("config", M16_CONFIGS)
+@pytest.mark.parametrize("CA,CB,K,H,W", [(48, 0, 48, 34, 50), (64, 48, 80, 36, 40), (96, 9, 112, 20, 70), (32, 0, 3, 33, 47), (9, 0, 16, 40, 36)])
+def test_conv_16x16_shape_odd_channel_counts(oracle, config, CA, CB, K, H, W):
+    """Output-channel counts that are multiples of 16 but not of 32 (paired and unpaired 16-blocks), K = 3,
+    with the upsample + concat prologue and the pool epilogue."""
+    rng = np.random.default_rng(CA + K)
+    w, b = he_weights(rng, K, CA + CB), small_bias(rng, K)
+    m = dx.Model()
+    if CB:
+        lo = rng.standard_normal((H // 2, W // 2, CA)).astype(np.float16)
+        x = rng.standard_normal((H, W, CB)).astype(np.float16)
+        t = m.pool(m.relu(m.conv2d(m.concat(m.upsample(m.input("lo", m.sym("W") // 2, m.sym("H") // 2, CA)), m.input("x", "W", "H", CB)), w, b)))
+        feeds, args = {"lo": lo, "x": x}, (lo, x)
+    else:
+        x = rng.standard_normal((H, W, CA)).astype(np.float16)
+        t = m.relu(m.conv2d(m.input("x", "W", "H", CA), w, b))
+        feeds, args = {"x": x}, (x,)
+    m.output(t)
+    try:
+        mod = dx.Module.compile(m, conv_config=config)
+    except dx.DenoxHipError as e:
+        assert e.status == 5
+        pytest.skip(str(e))
+    assert config in dx.last_compile_report()
+    got = mod.instance(H=H, W=W).infer(*args)[0]
+    want = oracle.run_graph(m.to_ops({"H": H, "W": W}), feeds, "fp32")[t.name]
     assert_conv_close(got, want, config)
 
 
