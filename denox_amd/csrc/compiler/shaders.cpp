@@ -112,8 +112,9 @@ bool chooseKT(const ConvConfig &cfgIn, unsigned CA, unsigned CB, unsigned K, con
     if (cfg.maxKT && kb * blk > cfg.maxKT) continue;
     const unsigned accRegs = cfg.mf == 32 ? kb * cfg.rpw * 16 : kb * cfg.rpw * cfg.xb * 4;
     if (accRegs + 64 + (cfg.mf == 16 ? kb * 4 : 0) > regBudget) continue;
-    const size_t lds = cfg.resident ? static_cast<size_t>(9u * kb * blk) * (g.CPAD + 8) * 2u + 2u * static_cast<size_t>(haloPix) * ckp * 2u
-                                    : (static_cast<size_t>(haloPix) + 9u * kb * blk) * ckp * 2u;
+    const size_t lds = (cfg.resident ? static_cast<size_t>(9u * kb * blk) * (g.CPAD + 8) * 2u + 2u * static_cast<size_t>(haloPix) * ckp * 2u
+                                     : (static_cast<size_t>(haloPix) + 9u * kb * blk) * ckp * 2u) +
+                       static_cast<size_t>(kb * blk) * 2u; // + the staged bias
     if (lds > dev.maxComputeSharedMemory) continue;
     g.KT = kb * blk;
     g.ldsBytes = lds;

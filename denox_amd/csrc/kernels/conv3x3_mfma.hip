@@ -61,6 +61,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     PushConstants pc) {
   __shared__ __attribute__((aligned(16))) _Float16 sIn[HALO_PIX * CKP];
   __shared__ __attribute__((aligned(16))) _Float16 sW[9 * KT * CKP];
+  __shared__ __attribute__((aligned(16))) _Float16 sBias[KT];
 #if CB == 0
   const _Float16 *B = nullptr;
 #endif
@@ -68,6 +69,8 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   const _Float16 *BIAS = nullptr;
 #endif
   const int tid = DNX_TID;
+  const OutBuf out = out_buffer(OUT, pc);
+  const Sources srcs = make_sources(A, B, pc);
   const int wv = tid >> 6;
   const int lane = tid & 63;
   const bool rev = (pc.FLAGS & 1u) != 0;
@@ -78,6 +81,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
 
   Acc acc;
   zero_acc(acc);
+  stage_bias(sBias, BIAS, kt, tid);
 
   // packed filter: [kt][chunk][tap][KT][len(chunk)]
   const _Float16 *wbase = FILT + (size_t)kt * 9 * KT * CPAD;
@@ -88,7 +92,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   H::src_init(src, map, y0, x0, pc);
   H::Regs stIn;
   uint4v stW[NV_W];
-  H::fetch_step(A, B, stIn, map, src, 0);
+  H::fetch_step(srcs, stIn, map, src, 0);
   if (NCHUNK > 1 || TAIL == CK)
     weights_fetch<CK>(wbase, stW, tid);
   else
@@ -103,7 +107,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     DNX_SYNC();
     if (chunk + 1 < NCHUNK) { // loads for the next step fly during the MFMAs below
       const _Float16 *wnext = wbase + (size_t)9 * KT * (chunk + 1) * CK;
-      H::fetch_step(A, B, stIn, map, src, chunk + 1);
+      H::fetch_step(srcs, stIn, map, src, chunk + 1);
       if (TAIL == CK || chunk + 1 < NCHUNK - 1)
         weights_fetch<CK>(wnext, stW, tid);
       else
@@ -112,5 +116,5 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     mma_step<CKP>(sIn, sW, 0, acc, wv, lane, chunk);
     DNX_SYNC();
   }
-  store_tile(acc, OUT, BIAS, y0, x0, kt, wv, lane, pc);
+  store_tile(acc, out, sBias, y0, x0, kt, wv, lane, pc);
 }

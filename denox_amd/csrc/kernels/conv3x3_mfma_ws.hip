@@ -40,6 +40,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     PushConstants pc) {
   __shared__ __attribute__((aligned(16))) _Float16 sW[9 * KT * CPADP];
   __shared__ __attribute__((aligned(16))) _Float16 sIn[2][HALO_PIX * CKP];
+  __shared__ __attribute__((aligned(16))) _Float16 sBias[KT];
 #if CB == 0
   const _Float16 *B = nullptr;
 #endif
@@ -47,6 +48,8 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   const _Float16 *BIAS = nullptr;
 #endif
   const int tid = DNX_TID;
+  const OutBuf out = out_buffer(OUT, pc);
+  const Sources srcs = make_sources(A, B, pc);
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6); // wave-uniform: roles branch on it
   const int lane = tid & 63;
 
@@ -73,6 +76,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   auto tileY = [&](int t) { return ((rev ? numTiles - 1 - t : t) / tilesX) * TH; };
   auto tileX = [&](int t) { return ((rev ? numTiles - 1 - t : t) % tilesX) * TW; };
 
+  stage_bias(sBias, BIAS, kt, tid);
   // ---- resident weights: global [tap][KT][CPAD] (one chunk = whole reduction) -> LDS rows of CPADP ----
   {
     const _Float16 *wsrc = FILT + (size_t)kt * 9 * KT * CPAD;
@@ -90,10 +94,10 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   H::Map map;
   H::Src fsrc;
   int ftile = tile, fchunk = 0;
+  // Past its last tile the cursor stays where it is: the loads are issued all the same (and never used), so that
+  // the number of loads in flight is the same on every path through the loop.
   auto issue = [&](H::Regs &regs) {
-    if (ftile >= last)
-      return;
-    H::fetch_step(A, B, regs, map, fsrc, fchunk);
+    H::fetch_step(srcs, regs, map, fsrc, fchunk);
     if (++fchunk == NCHUNK) {
       fchunk = 0;
       ftile += SLOTS;
@@ -106,6 +110,20 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   H::map_init(map, tid);
   H::src_init(fsrc, map, tileY(ftile), tileX(ftile), pc);
   Acc acc;
+  // The finished tile, converted.  Its stores go out in NPARTS portions during the steps of the next tile: a
+  // burst of all stores of all waves at once would hold the waves up at the store queue while nothing multiplies.
+  constexpr int NPARTS = NCHUNK < NGROUPS ? NCHUNK : NGROUPS;
+  Packed done;
+  int dtile = 0, dpart = 0;
+  bool pend = false;
+  auto store_part = [&]() {
+#pragma unroll
+    for (int p = 0; p < NPARTS; ++p)
+      if (dpart == p)
+        store_packed(done, out, tileY(dtile), tileX(dtile), kt, wv, lane, pc, p, NPARTS);
+    if (++dpart == NPARTS)
+      pend = false;
+  };
   int cchunk = 0, buf = 0;
   auto step = [&](H::Regs &regs) {
     if (cchunk == 0)
@@ -114,26 +132,37 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     // One barrier per step: buffer `buf` was last read two steps ago, and every wave
     // has passed the barrier of the step in between since then.
     DNX_SYNC();
+    // A portion of the previous tile's stores, in front of this step's loads: when a later step waits for those
+    // loads, it counts back over at most these stores, which are old by then.
+    if (pend)
+      store_part();
     issue(regs); // refill this register set: the step after next
     mma_step<CPADP>(sIn[buf], sW, cchunk * CK, acc, wv, lane, cchunk);
     buf ^= 1;
     if (++cchunk == NCHUNK) {
-      store_tile(acc, OUT, BIAS, tileY(tile), tileX(tile), kt, wv, lane, pc);
+      pack_tile(acc, done, sBias, lane);
+      dtile = tile;
+      dpart = 0;
+      pend = tile < last; // false in the spare step below
       cchunk = 0;
       tile += SLOTS;
     }
   };
   H::Regs st0, st1;
   issue(st0);
+  __builtin_amdgcn_sched_barrier(0); // keep the two sets in issue order: the waits below count loads in flight
   issue(st1);
-  while (true) {
+  // The loop always runs both steps, so that it has one entry and one back edge with the same loads in flight on
+  // both: the compiler then waits for exactly the register set a step needs.  When the last tile ends after the
+  // first step, the second one is a spare: it stages and multiplies stale data and stores nothing.
+  do {
     step(st0);
-    if (tile >= last)
-      break;
     step(st1);
-    if (tile >= last)
-      break;
-  }
+  } while (tile < last);
+#pragma unroll
+  for (int p = 0; p < NPARTS; ++p)
+    if (pend)
+      store_part();
 #else
   // number of steps this workgroup runs: both roles execute exactly one barrier per step
   const int myTiles = (last - tile + SLOTS - 1) / SLOTS;
@@ -177,7 +206,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
       DNX_SYNC();
       mma_step<CPADP>(sIn[g & 1], sW, cchunk * CK, acc, wv, lane, cchunk);
       if (++cchunk == NCHUNK) {
-        store_tile(acc, OUT, BIAS, tileY(tile), tileX(tile), kt, wv, lane, pc);
+        store_tile(acc, out, sBias, tileY(tile), tileX(tile), kt, wv, lane, pc);
         cchunk = 0;
         tile += SLOTS;
       }

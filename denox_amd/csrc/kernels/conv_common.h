@@ -182,6 +182,70 @@ load_src8(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, size_t
   }
 }
 
+// When every 8-channel vector lies in one source and no source is narrower than 8 channels, a vector is one
+// 16-byte load whatever the lane: the address is selected (never branched on) and the fix-up of a partial last
+// vector and the zero fill happen when the value is written to LDS.  Every lane then issues the same number of
+// loads in every step, so the compiler can wait for exactly the loads a step needs and leave younger ones in flight.
+#define VEC_SRC ((CA % 8 == 0 || CB == 0) && CA >= 8 && (CB == 0 || CB >= 8))
+
+__device__ DNX_INLINE const _Float16 *
+src8_ptr(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, size_t pa, size_t pb, int cc) {
+  const int rel = cc - CA;
+  const _Float16 *qa = A + pa + ((CA % 8 == 0 || cc + 8 <= CA) ? cc : CA - 8);
+  const _Float16 *qb = B + pb + ((CB % 8 == 0 || rel + 8 <= CB) ? rel : CB - 8);
+  return (CB > 0 && cc >= CA) ? qb : qa;
+}
+
+__device__ DNX_INLINE uint4v src8_fix(uint4v v, int cc) {
+  if (CA % 8 != 0) { // single source: its last vector was loaded so that it ends at the last channel
+    const uint4v sh = shr_halves<(8 - CA % 8) % 8>(v);
+    const bool part = cc < CA && cc + 8 > CA;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = part ? sh[i] : v[i];
+  }
+  if (CB > 0 && CB % 8 != 0) {
+    const uint4v sh = shr_halves<(8 - CB % 8) % 8>(v);
+    const bool part = cc >= CA && cc - CA + 8 > CB;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = part ? sh[i] : v[i];
+  }
+  return v;
+}
+
+template <bool WIDE> struct MaskType { typedef unsigned int type; };
+template <> struct MaskType<true> { typedef unsigned long long type; };
+
+// When, in addition, every step of CK channels lies in one source, the step's loads go through that source's buffer
+// resource with 32-bit byte offsets: one add per load, and a lane with nothing to load (halo pixel outside the image,
+// padding channel) passes an offset past the end and gets zeros from the hardware.
+#define SRC_UNIFORM (VEC_SRC && (CB == 0 || CA % CK == 0))
+#define NO_LOAD 0xFFFFF000u // past the end of every tensor this code accepts; stays past it when a channel offset is added
+static_assert(2 * CPAD + 16 < 4096, "channel offsets must not wrap the no-access offset");
+
+struct Sources {
+  const _Float16 *A, *B;
+  unsigned bytesA, bytesB;
+};
+
+__device__ DNX_INLINE Sources make_sources(const _Float16 *A, const _Float16 *B, const PushConstants &pc) {
+  Sources s;
+  s.A = A;
+  s.B = B;
+#if PADA
+  const unsigned pixA = pc.SRC_W * pc.SRC_H;
+#else
+  const unsigned pixA = UPA ? (pc.IN_W >> 1) * (pc.IN_H >> 1) : pc.IN_W * pc.IN_H;
+#endif
+#if PADB
+  const unsigned pixB = pc.SRC_W * pc.SRC_H;
+#else
+  const unsigned pixB = pc.IN_W * pc.IN_H;
+#endif
+  s.bytesA = pixA * (unsigned)CA * 2u;
+  s.bytesB = pixB * (unsigned)CB * 2u;
+  return s;
+}
+
 // ---- halo staging ---------------------------------------------------------------------
 // The (TH+2) x 34 pixel halo of one reduction step is moved by NTH threads, 16 bytes
 // (8 channels) per access.  Vector i = t + it*NTH covers pixel i / (CK/8), channel group
@@ -198,9 +262,16 @@ struct Halo {
     int hy[NV], hx[NV], v8[NV];
   };
   struct Src {
-    int pa[NV], pb[NV]; // element offsets of the pixel in A and B, pa < 0: outside the image (reads as zero)
+    // offsets of the pixel in A and B.  SRC_UNIFORM: in bytes, NO_LOAD outside the image; else in elements,
+    // pa < 0 outside the image (reads as zero)
+    int pa[NV], pb[NV];
   };
-  typedef uint4v Regs[NV];
+  static_assert(NV <= 64, "halo share of one thread too large");
+  typedef typename MaskType<(NV > 32)>::type Mask;
+  struct Regs {
+    uint4v v[NV];
+    Mask ok; // bit it: vector it holds image data (clear: it reads as zero)
+  };
 
   static __device__ DNX_INLINE void map_init(Map &m, int t) {
 #pragma unroll
@@ -224,48 +295,100 @@ struct Halo {
       const bool inside = m.lds[it] >= 0 && gy >= 0 && gy < (int)pc.IN_H && gx >= 0 && gx < (int)pc.IN_W;
       if (inside)
         src_offsets(gy, gx, pc, pa, pb);
+#if SRC_UNIFORM
+      s.pa[it] = inside ? (int)((unsigned)pa * 2u) : (int)NO_LOAD;
+      s.pb[it] = inside ? (int)((unsigned)pb * 2u) : (int)NO_LOAD;
+#else
       s.pa[it] = inside ? (int)pa : -1;
       s.pb[it] = (int)pb;
+#endif
     }
   }
 
   // Issue the loads of the L channels starting at c0 into registers ...
   template <int L>
-  static __device__ DNX_INLINE void
-  fetch(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, Regs &st, const Map &m, const Src &s, int c0) {
+  static __device__ DNX_INLINE void fetch(const Sources &src, Regs &st, const Map &m, const Src &s, int c0) {
+#if SRC_UNIFORM
+    st.ok = 0;
+    // One stream of load instructions whichever the source (no branch: the waits for these loads are counted),
+    // with the source's base, size and channel count selected by scalar conditions.
+    const bool fromA = CB == 0 || c0 < CA; // the same for all lanes
+    const int cs = fromA ? CA : CB;        // channels of the step's source
+    const int cbase = fromA ? 0 : CA;
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<_Float16 *>(fromA ? src.A : src.B), 0, (int)(fromA ? src.bytesA : src.bytesB), 0x00020000);
 #pragma unroll
     for (int it = 0; it < NV; ++it) {
+      const int rel = c0 + m.v8[it] - cbase;
+      const int chan = ((CA % 8 == 0 && CB % 8 == 0) || rel + 8 <= cs) ? rel : cs - 8;
+      unsigned off = (unsigned)(fromA ? s.pa[it] : s.pb[it]) + 2u * (unsigned)chan;
+      off = (m.v8[it] < L && rel < cs) ? off : NO_LOAD;
+#ifdef DBG_SKIP_FETCH
+      off = NO_LOAD;
+#endif
+      st.v[it] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0);
+    }
+#else
+    const _Float16 *__restrict__ A = src.A;
+    const _Float16 *__restrict__ B = src.B;
+    Mask ok = 0;
+#pragma unroll
+    for (int it = 0; it < NV; ++it) {
+      const int cc = c0 + m.v8[it];
+#if VEC_SRC
+      const bool act = s.pa[it] >= 0 && m.v8[it] < L && cc < CIN;
+#ifndef DBG_SKIP_FETCH
+      const _Float16 *p = src8_ptr(A, B, (size_t)s.pa[it], (size_t)s.pb[it], cc);
+      st.v[it] = *reinterpret_cast<const uint4v_u *>(act ? p : A); // idle lanes re-read the first pixel
+#else
+      st.v[it] = uint4v{0u, 0u, 0u, 0u};
+#endif
+      ok |= act ? (Mask)1 << it : (Mask)0;
+#else
       uint4v val = {0u, 0u, 0u, 0u};
 #ifndef DBG_SKIP_FETCH
       if (s.pa[it] >= 0 && m.v8[it] < L)
-        val = load_src8(A, B, (size_t)s.pa[it], (size_t)s.pb[it], c0 + m.v8[it]);
+        val = load_src8(A, B, (size_t)s.pa[it], (size_t)s.pb[it], cc);
 #endif
-      st[it] = val;
+      st.v[it] = val;
+#endif
     }
+    st.ok = ok;
+#endif
   }
 
   // ... and write them to the staged halo.
   template <int L>
-  static __device__ DNX_INLINE void commit(const Regs &st, _Float16 *sIn, const Map &m) {
+  static __device__ DNX_INLINE void commit(const Regs &st, _Float16 *sIn, const Map &m, int c0) {
 #pragma unroll
     for (int it = 0; it < NV; ++it)
-      if (m.lds[it] >= 0 && m.v8[it] < L)
-        *reinterpret_cast<uint4v *>(sIn + m.lds[it]) = st[it];
+      if (m.lds[it] >= 0 && m.v8[it] < L) {
+        uint4v v = st.v[it];
+#if VEC_SRC
+        v = src8_fix(v, c0 + m.v8[it]);
+#if !SRC_UNIFORM // (with SRC_UNIFORM the hardware already returned zeros where nothing was to be read)
+        const bool keep = ((st.ok >> it) & 1) != 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = keep ? v[i] : 0u;
+#endif
+#endif
+        *reinterpret_cast<uint4v *>(sIn + m.lds[it]) = v;
+      }
   }
 
   // fetch / commit of step `chunk` of a tile, whichever length that step has
   static __device__ DNX_INLINE void
-  fetch_step(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, Regs &st, const Map &m, const Src &s, int chunk) {
+  fetch_step(const Sources &src, Regs &st, const Map &m, const Src &s, int chunk) {
     if (TAIL == CK || chunk < NCHUNK - 1)
-      fetch<CK>(A, B, st, m, s, chunk * CK);
+      fetch<CK>(src, st, m, s, chunk * CK);
     else
-      fetch<TAIL>(A, B, st, m, s, chunk * CK);
+      fetch<TAIL>(src, st, m, s, chunk * CK);
   }
   static __device__ DNX_INLINE void commit_step(const Regs &st, _Float16 *sIn, const Map &m, int chunk) {
     if (TAIL == CK || chunk < NCHUNK - 1)
-      commit<CK>(st, sIn, m);
+      commit<CK>(st, sIn, m, chunk * CK);
     else
-      commit<TAIL>(st, sIn, m);
+      commit<TAIL>(st, sIn, m, chunk * CK);
   }
 };
 
@@ -285,21 +408,53 @@ __device__ DNX_INLINE ushort_t dpp_xor1(ushort_t v) {
   return (ushort_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xF, 0xF, true);
 }
 
-__device__ DNX_INLINE void store16(_Float16 *dst, const half8 (&o)[2], int chb) {
-#ifdef DBG_SKIP_STORE
-  if (o[0][0] != (_Float16)12345.0f) return; // practically never true: keeps the epilogue arithmetic, drops the stores
+// ---- output stores ---------------------------------------------------------------------
+// The output is written through a buffer resource: a lane that has nothing to store (pixel outside the image or the
+// crop window, odd lane of a pooled pair, channel past KOUT) passes an offset past the end and the hardware drops
+// its part of the store.  No branch surrounds a store, so every wave issues the same number of them per tile.
+typedef __amdgpu_buffer_rsrc_t OutBuf;
+#define NO_STORE 0xFFFFF000u // beyond every output this code accepts (byte sizes are limited to below this value)
+
+__device__ DNX_INLINE OutBuf out_buffer(_Float16 *OUT, const PushConstants &pc) {
+#if POOL
+  const unsigned w = pc.IN_W >> 1, h = pc.IN_H >> 1;
+#elif CROP
+  const unsigned w = pc.OUT_W, h = pc.OUT_H;
+#else
+  const unsigned w = pc.IN_W, h = pc.IN_H;
 #endif
+  return __builtin_amdgcn_make_buffer_rsrc(OUT, 0, (int)(w * h * (unsigned)KOUT * 2u), 0x00020000);
+}
+
+// 16 consecutive channels starting at chb of the pixel with linear index `pix`
+__device__ DNX_INLINE void store16(OutBuf out, bool ok, unsigned pix, const half8 (&o)[2], int chb) {
+#ifdef DBG_SKIP_STORE
+  ok = ok && o[0][0] == (_Float16)12345.0f; // practically never true: keeps the epilogue, drops the memory traffic
+#endif
+  const unsigned off = (pix * (unsigned)KOUT + (unsigned)chb) * 2u;
   if (KOUT % 16 == 0) {
-    if (chb < KOUT) {
-      *reinterpret_cast<half8 *>(dst) = o[0];
-      *reinterpret_cast<half8 *>(dst + 8) = o[1];
-    }
+    const unsigned o0 = (ok && chb < KOUT) ? off : NO_STORE;
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, o[0]), out, o0, 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, o[1]), out, o0 + 16u, 0, 0);
+  } else if (KOUT % 8 == 0) {
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, o[0]), out, (ok && chb < KOUT) ? off : NO_STORE, 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, o[1]), out, (ok && chb + 8 < KOUT) ? off + 16u : NO_STORE, 0, 0);
   } else {
 #pragma unroll
-    for (int i = 0; i < 16; ++i)
-      if (chb + i < KOUT)
-        dst[i] = o[i >> 3][i & 7];
+    for (int i = 0; i < (KOUT < 16 ? KOUT : 16); ++i) {
+      const _Float16 h = o[i >> 3][i & 7]; // a vector element is no object: copy it before reinterpreting its bits
+      __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(ushort_t, h), out, (ok && chb + i < KOUT) ? off + 2u * i : NO_STORE, 0, 0);
+    }
   }
+}
+
+// The KT bias values of a workgroup's output channels are staged in LDS once (the global buffer is zero-padded to
+// KOUTP), so that the epilogue waits for no global load.  Visible after the first barrier.
+__device__ DNX_INLINE void stage_bias(_Float16 *sBias, const _Float16 *__restrict__ BIAS, int kt, int tid) {
+#if HAS_BIAS
+  for (int i = tid; i < KT; i += NT)
+    sBias[i] = BIAS[kt * KT + i];
+#endif
 }
 
 #if MF == 32
@@ -308,33 +463,31 @@ struct Acc {
   float16v v[KB][RPW];
 };
 
-// Epilogue of one wave: acc[kb][j] holds, for output row y0 + wv*RPW + j and pixel
+// Epilogue of one wave in two parts, so that a persistent kernel can convert a finished tile at once and issue
+// its stores later, after the next loads.  acc[kb][j] holds, for output row y0 + wv*RPW + j and pixel
 // x0 + (lane & 31), the 16 channels kt*KT + kb*32 + (lane >> 5)*16 + i.
-__device__ DNX_INLINE void
-store_tile(const Acc &acc, _Float16 *__restrict__ OUT, const _Float16 *__restrict__ BIAS,
-           int y0, int x0, int kt, int wv, int lane, const PushConstants &pc) {
-  const unsigned W = pc.IN_W, H = pc.IN_H;
-  const int l32 = lane & 31;
+#define OROWS (POOL ? RPW / 2 : RPW) // output rows a wave stores per tile
+struct Packed {
+  half8 o[KB][OROWS][2];
+};
+
+// bias, activation, rounding to fp16 and (POOL) the 2x2 maximum
+__device__ DNX_INLINE void pack_tile(const Acc &acc, Packed &pk, const _Float16 *sBias, int lane) {
   const int hsel = lane >> 5;
-  const int x = x0 + l32;
 #pragma unroll
   for (int kb = 0; kb < KB; ++kb) {
-    const int chb = kt * KT + kb * 32 + hsel * 16; // first of this lane's 16 channels
     float bias[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
 #if HAS_BIAS
-      bias[i] = (float)BIAS[chb + i]; // the bias buffer is zero-padded to KOUTP
+      bias[i] = (float)sBias[kb * 32 + hsel * 16 + i];
 #else
       bias[i] = 0.0f;
 #endif
     }
 #if POOL
-    const unsigned WP = W >> 1, HP = H >> 1;
 #pragma unroll
     for (int j = 0; j < RPW; j += 2) {
-      const int y = y0 + wv * RPW + j;
-      half8 o[2];
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const _Float16 v0 = (_Float16)apply_act(acc.v[kb][j][i] + bias[i]);
@@ -346,35 +499,49 @@ store_tile(const Acc &acc, _Float16 *__restrict__ OUT, const _Float16 *__restric
         m = n0 > m ? n0 : m;
         m = v1 > m ? v1 : m;
         m = n1 > m ? n1 : m;
-        o[i >> 3][i & 7] = m;
+        pk.o[kb][j >> 1][i >> 3][i & 7] = m;
       }
-      const unsigned py = (unsigned)y >> 1, px = (unsigned)x >> 1;
-      if ((l32 & 1) == 0 && py < HP && px < WP)
-        store16(OUT + ((size_t)py * WP + px) * KOUT + chb, o, chb);
     }
 #else
 #pragma unroll
-    for (int j = 0; j < RPW; ++j) {
-      const int y = y0 + wv * RPW + j;
-      half8 o[2];
+    for (int j = 0; j < RPW; ++j)
 #pragma unroll
       for (int i = 0; i < 16; ++i)
-        o[i >> 3][i & 7] = (_Float16)apply_act(acc.v[kb][j][i] + bias[i]);
+        pk.o[kb][j][i >> 3][i & 7] = (_Float16)apply_act(acc.v[kb][j][i] + bias[i]);
+#endif
+  }
+}
+
+#define NGROUPS (KB * OROWS) // store groups of a tile: one output row of one 32-channel block each
+
+// Stores the groups g with g % nparts == part (all of them with nparts = 1).
+__device__ DNX_INLINE void
+store_packed(const Packed &pk, OutBuf out, int y0, int x0, int kt, int wv, int lane, const PushConstants &pc, int part = 0, int nparts = 1) {
+  const unsigned W = pc.IN_W, H = pc.IN_H;
+  const int l32 = lane & 31;
+  const int x = x0 + l32;
+#pragma unroll
+  for (int kb = 0; kb < KB; ++kb) {
+    const int chb = kt * KT + kb * 32 + (lane >> 5) * 16; // first of this lane's 16 channels
+#pragma unroll
+    for (int r = 0; r < OROWS; ++r) {
+      if ((kb * OROWS + r) % nparts != part)
+        continue;
+#if POOL
+      const unsigned WP = W >> 1, HP = H >> 1;
+      const unsigned py = (unsigned)(y0 + wv * RPW + 2 * r) >> 1, px = (unsigned)x >> 1;
+      store16(out, (l32 & 1) == 0 && py < HP && px < WP, py * WP + px, pk.o[kb][r], chb);
+#else
+      const int y = y0 + wv * RPW + r;
 #if CROP
       const int oy = y - (int)pc.CROP_T, ox = x - (int)pc.CROP_L;
-      if (y < (int)H && x < (int)W && oy >= 0 && oy < (int)pc.OUT_H && ox >= 0 && ox < (int)pc.OUT_W)
-        store16(OUT + ((size_t)oy * pc.OUT_W + ox) * KOUT + chb, o, chb);
+      store16(out, y < (int)H && x < (int)W && oy >= 0 && oy < (int)pc.OUT_H && ox >= 0 && ox < (int)pc.OUT_W,
+              (unsigned)oy * pc.OUT_W + (unsigned)ox, pk.o[kb][r], chb);
 #else
-#ifdef DBG_STORE_SMALL // timing experiment: same instructions, all stores land in a 4096-pixel window
-      if (y < (int)H && x < (int)W)
-        store16(OUT + ((((size_t)y * W + x) & 4095) * KOUT) + chb, o, chb);
-#else
-      if (y < (int)H && x < (int)W)
-        store16(OUT + ((size_t)y * W + x) * KOUT + chb, o, chb);
+      store16(out, y < (int)H && x < (int)W, (unsigned)y * W + (unsigned)x, pk.o[kb][r], chb);
 #endif
 #endif
     }
-#endif
   }
 }
 
@@ -435,92 +602,112 @@ struct Acc {
   float4v v[KB][RPW][XB];
 };
 
-__device__ DNX_INLINE void store_vec(_Float16 *dst, const _Float16 (&o)[8], int chb, int n) {
-  // n = 8 or 4 consecutive channels starting at chb
+// n = 8 or 4 consecutive channels starting at chb of the pixel with linear index `pix`
+__device__ DNX_INLINE void store_vec(OutBuf out, bool ok, unsigned pix, const _Float16 (&o)[8], int chb, int n) {
+#ifdef DBG_SKIP_STORE
+  ok = ok && o[0] == (_Float16)12345.0f;
+#endif
+  const unsigned off = (pix * (unsigned)KOUT + (unsigned)chb) * 2u;
   if (KOUT % 8 == 0 && n == 8) {
-    if (chb < KOUT) {
-      half8 h;
+    half8 h;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) h[i] = o[i];
-      *reinterpret_cast<half8 *>(dst) = h;
-    }
+    for (int i = 0; i < 8; ++i) h[i] = o[i];
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, h), out, (ok && chb < KOUT) ? off : NO_STORE, 0, 0);
   } else {
 #pragma unroll
     for (int i = 0; i < 8; ++i)
-      if (i < n && chb + i < KOUT) dst[i] = o[i];
+      if (i < n)
+        __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(ushort_t, o[i]), out, (ok && chb + i < KOUT) ? off + 2u * i : NO_STORE, 0, 0);
   }
 }
 
-__device__ DNX_INLINE void
-store_tile(const Acc &acc, _Float16 *__restrict__ OUT, const _Float16 *__restrict__ BIAS,
-           int y0, int x0, int kt, int wv, int lane, const PushConstants &pc) {
-  const unsigned W = pc.IN_W, H = pc.IN_H;
-  const int l16 = lane & 15;
+#define OROWS (POOL ? RPW / 2 : RPW) // output rows a wave stores per tile
+#define KPAIRS ((KB + 1) / 2)
+struct Packed {
+  _Float16 o[KPAIRS][XB][OROWS][8];
+};
+
+// bias, activation, rounding to fp16 and (POOL) the 2x2 maximum
+__device__ DNX_INLINE void pack_tile(const Acc &acc, Packed &pk, const _Float16 *sBias, int lane) {
   const int g = lane >> 4;
 #pragma unroll
-  for (int kp = 0; kp < (KB + 1) / 2; ++kp) {
+  for (int kp = 0; kp < KPAIRS; ++kp) {
     const bool paired = 2 * kp + 1 < KB;
     const int n = paired ? 8 : 4;
-    const int chb = kt * KT + (paired ? 32 * kp + 8 * g : 16 * (2 * kp) + 4 * g);
+    const int chl = paired ? 32 * kp + 8 * g : 16 * (2 * kp) + 4 * g; // first channel, relative to the workgroup's KT
     float bias[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
 #if HAS_BIAS
-      bias[i] = i < n ? (float)BIAS[chb + i] : 0.0f; // the bias buffer is zero-padded to KOUTP
+      bias[i] = i < n ? (float)sBias[chl + i] : 0.0f;
 #else
       bias[i] = 0.0f;
 #endif
     }
 #pragma unroll
     for (int xb = 0; xb < XB; ++xb) {
-      const int x = x0 + xb * 16 + l16;
-#if POOL
-      const unsigned WP = W >> 1, HP = H >> 1;
 #pragma unroll
-      for (int j = 0; j < RPW; j += 2) {
-        const int y = y0 + wv * RPW + j;
-        _Float16 o[8];
+      for (int r = 0; r < OROWS; ++r) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-          const int kb = 2 * kp + (i >> 2);
+          const int kb = 2 * kp + (i >> 2) < KB ? 2 * kp + (i >> 2) : 0;
+          _Float16 m = (_Float16)0.0f;
           if (i < n) {
-            const _Float16 v0 = (_Float16)apply_act(acc.v[kb < KB ? kb : 0][j][xb][i & 3] + bias[i]);
-            const _Float16 v1 = (_Float16)apply_act(acc.v[kb < KB ? kb : 0][j + 1][xb][i & 3] + bias[i]);
+#if POOL
+            const _Float16 v0 = (_Float16)apply_act(acc.v[kb][2 * r][xb][i & 3] + bias[i]);
+            const _Float16 v1 = (_Float16)apply_act(acc.v[kb][2 * r + 1][xb][i & 3] + bias[i]);
             const _Float16 n0 = __builtin_bit_cast(_Float16, dpp_xor1(__builtin_bit_cast(ushort_t, v0)));
             const _Float16 n1 = __builtin_bit_cast(_Float16, dpp_xor1(__builtin_bit_cast(ushort_t, v1)));
-            _Float16 m = v0; // window order (0,0) (0,1) (1,0) (1,1); replace only on strictly greater
+            m = v0; // window order (0,0) (0,1) (1,0) (1,1); replace only on strictly greater
             m = n0 > m ? n0 : m;
             m = v1 > m ? v1 : m;
             m = n1 > m ? n1 : m;
-            o[i] = m;
-          } else {
-            o[i] = (_Float16)0.0f;
-          }
-        }
-        const unsigned py = (unsigned)y >> 1, px = (unsigned)x >> 1;
-        if ((l16 & 1) == 0 && py < HP && px < WP)
-          store_vec(OUT + ((size_t)py * WP + px) * KOUT + chb, o, chb, n);
-      }
 #else
-#pragma unroll
-      for (int j = 0; j < RPW; ++j) {
-        const int y = y0 + wv * RPW + j;
-        _Float16 o[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const int kb = 2 * kp + (i >> 2);
-          o[i] = i < n ? (_Float16)apply_act(acc.v[kb < KB ? kb : 0][j][xb][i & 3] + bias[i]) : (_Float16)0.0f;
+            m = (_Float16)apply_act(acc.v[kb][r][xb][i & 3] + bias[i]);
+#endif
+          }
+          pk.o[kp][xb][r][i] = m;
         }
+      }
+    }
+  }
+}
+
+#define NGROUPS (KPAIRS * XB * OROWS) // store groups of a tile
+
+// Stores the groups g with g % nparts == part (all of them with nparts = 1).
+__device__ DNX_INLINE void
+store_packed(const Packed &pk, OutBuf out, int y0, int x0, int kt, int wv, int lane, const PushConstants &pc, int part = 0, int nparts = 1) {
+  const unsigned W = pc.IN_W, H = pc.IN_H;
+  const int l16 = lane & 15;
+  const int g = lane >> 4;
+#pragma unroll
+  for (int kp = 0; kp < KPAIRS; ++kp) {
+    const bool paired = 2 * kp + 1 < KB;
+    const int n = paired ? 8 : 4;
+    const int chb = kt * KT + (paired ? 32 * kp + 8 * g : 16 * (2 * kp) + 4 * g);
+#pragma unroll
+    for (int xb = 0; xb < XB; ++xb) {
+      const int x = x0 + xb * 16 + l16;
+#pragma unroll
+      for (int r = 0; r < OROWS; ++r) {
+        if (((kp * XB + xb) * OROWS + r) % nparts != part)
+          continue;
+#if POOL
+        const unsigned WP = W >> 1, HP = H >> 1;
+        const unsigned py = (unsigned)(y0 + wv * RPW + 2 * r) >> 1, px = (unsigned)x >> 1;
+        store_vec(out, (l16 & 1) == 0 && py < HP && px < WP, py * WP + px, pk.o[kp][xb][r], chb, n);
+#else
+        const int y = y0 + wv * RPW + r;
 #if CROP
         const int oy = y - (int)pc.CROP_T, ox = x - (int)pc.CROP_L;
-        if (y < (int)H && x < (int)W && oy >= 0 && oy < (int)pc.OUT_H && ox >= 0 && ox < (int)pc.OUT_W)
-          store_vec(OUT + ((size_t)oy * pc.OUT_W + ox) * KOUT + chb, o, chb, n);
+        store_vec(out, y < (int)H && x < (int)W && oy >= 0 && oy < (int)pc.OUT_H && ox >= 0 && ox < (int)pc.OUT_W,
+                  (unsigned)oy * pc.OUT_W + (unsigned)ox, pk.o[kp][xb][r], chb, n);
 #else
-        if (y < (int)H && x < (int)W)
-          store_vec(OUT + ((size_t)y * W + x) * KOUT + chb, o, chb, n);
+        store_vec(out, y < (int)H && x < (int)W, (unsigned)y * W + (unsigned)x, pk.o[kp][xb][r], chb, n);
+#endif
 #endif
       }
-#endif
     }
   }
 }
@@ -572,6 +759,13 @@ __device__ DNX_INLINE void zero_acc(Acc &acc) {
           acc.v[kb][j][xb][i] = 0.0f;
 }
 #endif // MF
+
+__device__ DNX_INLINE void
+store_tile(const Acc &acc, OutBuf out, const _Float16 *sBias, int y0, int x0, int kt, int wv, int lane, const PushConstants &pc) {
+  Packed pk;
+  pack_tile(acc, pk, sBias, lane);
+  store_packed(pk, out, y0, x0, kt, wv, lane, pc);
+}
 
 // mma_chunk for step `chunk` of a tile, whichever length that step has
 template <int WPITCH>

@@ -111,6 +111,9 @@ Instance::Instance(ModelHandle model, const std::vector<ValueSpec> &specs) : m_m
     const int64_t off = t.offset.eval(m_sym), sz = t.size.eval(m_sym);
     if (off < 0 || sz < 0 || static_cast<uint64_t>(off) + static_cast<uint64_t>(sz) > m_bufferSizes[t.buffer])
       fail(Status::InvalidModel, "tensor '" + t.info.name + "' does not fit its buffer");
+    // the kernels address a tensor with 32-bit byte offsets (buffer resources); offsets from 0xFFFFF000 up mean "no access"
+    if (static_cast<uint64_t>(sz) >= 0xFFFFF000ull)
+      fail(Status::Unsupported, "tensor '" + t.info.name + "' is " + std::to_string(sz) + " bytes at these extents; tensors of 4 GiB and more are not supported");
   }
   try {
     m_buffers.assign(m.buffers.size(), nullptr);

@@ -3,6 +3,14 @@ import sys
 
 import pytest
 
+# PyTorch ships its own copy of the HIP/HSA runtime.  A test that hands torch device pointers to the library needs
+# both to share one runtime in the process, which is the case when torch is loaded first, whatever subset of the
+# test files is collected.
+try:
+    import torch  # noqa: F401
+except ImportError:
+    pass
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)

@@ -103,6 +103,17 @@ def test_conv_16x16_shape_odd_channel_counts(oracle, config, CA, CB, K, H, W):
     assert_conv_close(got, want, config)
 
 
+def test_tensor_size_limit_is_reported():
+    """Tensors are addressed with 32-bit byte offsets: extents that make one reach 4 GiB are refused when the
+    instance is created, before anything is allocated."""
+    m = dx.Model()
+    m.output(m.relu(m.conv2d(m.input("x", "W", "H", 64), np.zeros((64, 64, 3, 3), np.float16))))
+    mod = dx.Module.compile(m)
+    with pytest.raises(dx.DenoxHipError) as e:
+        mod.instance(H=6000, W=6000)
+    assert e.value.status == 5 and "4 GiB" in str(e.value)
+
+
 def test_conv_closed_forms():
     # centre-tap identity: out == in, bit for bit; all-ones: C * (#taps inside the image)
     C = 16
