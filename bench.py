@@ -109,8 +109,9 @@ def main() -> int:
         db.bench(min_samples=10, max_relative_error=0.03, max_samples=50, save_progress=bool(args.db))
         tune_s = time.perf_counter() - t0
     blob = dx.compile_model(model, assume={"H": H, "W": W}, conv_config=args.conv_config, db=db, input_layout=lay, output_layout=lay)
+    report = dx.last_compile_report()
     if args.per_dispatch:
-        print(dx.last_compile_report(), file=sys.stderr)
+        print(report, file=sys.stderr)
     mod = dx.Module.load(blob)
     inst = mod.instance(H=H, W=W)
 
@@ -176,14 +177,17 @@ def main() -> int:
                 "non_conv_frac_of_hbm": other_bytes / other_ms * 1e-6 / PEAK_HBM_GBPS if other_ms else None,
                 "sum_dispatch_ms": sum(a["latency_ms"] for a in acc)}
 
-    # HBM traffic of the dominant kernel from the committed rocprofv3 --pmc summary, when it covers this kernel
+    # HBM traffic of the dominant kernel from the committed rocprofv3 --pmc summary, when it covers this kernel:
+    # the summary lists every configuration of that layer; the compile report says which one this schedule uses
     try:
         with open(os.path.join(ROOT, "profiles", "dominant_conv_traffic.json")) as f:
             tr = json.load(f)
         if tr["dispatch_name"] == dom["name"] and (H, W) == (tr["height"], tr["width"]):
-            roofline["traffic"] = tr["fetch_bytes"] + tr["write_bytes"]
+            cfg = next(l.split()[1] for l in report.splitlines() if l.startswith("conv3x3_mfma ") and l.split()[2] == dom["name"])
+            roofline["kernel_config"] = cfg
+            roofline["traffic"] = tr["configs"][cfg]["fetch_bytes"] + tr["configs"][cfg]["write_bytes"]
             roofline["traffic_unit"] = "bytes per launch (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel)"
-    except (OSError, KeyError, ValueError):
+    except (OSError, KeyError, ValueError, StopIteration):
         pass
 
     line = {

@@ -112,7 +112,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   Acc acc;
   // The finished tile, converted.  Its stores go out in NPARTS portions during the steps of the next tile: a
   // burst of all stores of all waves at once would hold the waves up at the store queue while nothing multiplies.
-  constexpr int NPARTS = NCHUNK < NGROUPS ? NCHUNK : NGROUPS;
+  constexpr int NPARTS = NCHUNK < OROWS ? NCHUNK : OROWS; // whole output rows per portion
   Packed done;
   int dtile = 0, dpart = 0;
   bool pend = false;

@@ -512,9 +512,8 @@ __device__ DNX_INLINE void pack_tile(const Acc &acc, Packed &pk, const _Float16 
   }
 }
 
-#define NGROUPS (KB * OROWS) // store groups of a tile: one output row of one 32-channel block each
-
-// Stores the groups g with g % nparts == part (all of them with nparts = 1).
+// Stores the output rows r with r % nparts == part (all of them with nparts = 1).  All channels of a pixel go out
+// together: a 128-byte line that is filled in two portions far apart in time is written to memory twice.
 __device__ DNX_INLINE void
 store_packed(const Packed &pk, OutBuf out, int y0, int x0, int kt, int wv, int lane, const PushConstants &pc, int part = 0, int nparts = 1) {
   const unsigned W = pc.IN_W, H = pc.IN_H;
@@ -525,7 +524,7 @@ store_packed(const Packed &pk, OutBuf out, int y0, int x0, int kt, int wv, int l
     const int chb = kt * KT + kb * 32 + (lane >> 5) * 16; // first of this lane's 16 channels
 #pragma unroll
     for (int r = 0; r < OROWS; ++r) {
-      if ((kb * OROWS + r) % nparts != part)
+      if (r % nparts != part)
         continue;
 #if POOL
       const unsigned WP = W >> 1, HP = H >> 1;
@@ -673,9 +672,8 @@ __device__ DNX_INLINE void pack_tile(const Acc &acc, Packed &pk, const _Float16 
   }
 }
 
-#define NGROUPS (KPAIRS * XB * OROWS) // store groups of a tile
-
-// Stores the groups g with g % nparts == part (all of them with nparts = 1).
+// Stores the output rows r with r % nparts == part (all of them with nparts = 1).  All channels of a pixel go out
+// together: a 128-byte line that is filled in two portions far apart in time is written to memory twice.
 __device__ DNX_INLINE void
 store_packed(const Packed &pk, OutBuf out, int y0, int x0, int kt, int wv, int lane, const PushConstants &pc, int part = 0, int nparts = 1) {
   const unsigned W = pc.IN_W, H = pc.IN_H;
@@ -691,7 +689,7 @@ store_packed(const Packed &pk, OutBuf out, int y0, int x0, int kt, int wv, int l
       const int x = x0 + xb * 16 + l16;
 #pragma unroll
       for (int r = 0; r < OROWS; ++r) {
-        if (((kp * XB + xb) * OROWS + r) % nparts != part)
+        if (r % nparts != part)
           continue;
 #if POOL
         const unsigned WP = W >> 1, HP = H >> 1;
