@@ -83,6 +83,11 @@ SIGNATURES = {
     "denox_hip_builder_pad": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, POINTER(c_int)]),
     "denox_hip_builder_slice": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, POINTER(c_int)]),
     "denox_hip_builder_output": (c_int, [c_void_p, c_int, c_char_p]),
+    "denox_hip_builder_import_onnx": (c_int, [c_void_p, c_char_p, c_size_t]),
+    "denox_hip_builder_input_count": (c_int, [c_void_p, POINTER(c_uint32)]),
+    "denox_hip_builder_output_count": (c_int, [c_void_p, POINTER(c_uint32)]),
+    "denox_hip_builder_input_info": (c_int, [c_void_p, c_uint32, c_char_p, c_size_t, POINTER(c_uint32)]),
+    "denox_hip_builder_output_info": (c_int, [c_void_p, c_uint32, c_char_p, c_size_t, POINTER(c_uint32)]),
     "denox_hip_compile_options_default": (None, [POINTER(CompileOptions)]),
     "denox_hip_compile": (c_int, [c_void_p, POINTER(CompileOptions), c_void_p, POINTER(c_void_p), POINTER(c_size_t)]),
     "denox_hip_last_compile_report": (c_char_p, []),

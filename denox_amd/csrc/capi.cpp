@@ -5,6 +5,7 @@
 #include "compiler/compile.hpp"
 #include "database/db.hpp"
 #include "device_info/device_info.hpp"
+#include "frontend/onnx_import.hpp"
 #include "hip/hip_compiler.hpp"
 #include "runtime/db_bench.hpp"
 #include "runtime/runtime.hpp"
@@ -196,6 +197,34 @@ int denox_hip_builder_slice(denox_hip_builder *b, int src, int64_t l, int64_t r,
 }
 int denox_hip_builder_output(denox_hip_builder *b, int src, const char *name) {
   return guarded([&] { need(b, "builder"); need(name, "name"); b->model.output(src, name); });
+}
+
+int denox_hip_builder_import_onnx(denox_hip_builder *b, const void *onnx_bytes, size_t size) {
+  return guarded([&] { need(b, "builder"); need(onnx_bytes, "onnx_bytes"); onnx::importModel(b->model, static_cast<const uint8_t *>(onnx_bytes), size); });
+}
+int denox_hip_builder_input_count(const denox_hip_builder *b, uint32_t *out) {
+  return guarded([&] { need(b, "builder"); need(out, "out"); *out = static_cast<uint32_t>(b->model.inputs().size()); });
+}
+int denox_hip_builder_output_count(const denox_hip_builder *b, uint32_t *out) {
+  return guarded([&] { need(b, "builder"); need(out, "out"); *out = static_cast<uint32_t>(b->model.outputs().size()); });
+}
+namespace {
+void tensorInfo(const compiler::Model &m, const std::vector<compiler::TensorHandle> &list, uint32_t i, char *name, size_t capacity, uint32_t *channels) {
+  if (i >= list.size()) fail(Status::InvalidArgument, "index out of range");
+  const auto &t = m.tensors()[static_cast<size_t>(list[i])];
+  if (name && capacity) {
+    const size_t n = std::min(capacity - 1, t.name.size());
+    std::memcpy(name, t.name.data(), n);
+    name[n] = 0;
+  }
+  if (channels) *channels = t.channels;
+}
+} // namespace
+int denox_hip_builder_input_info(const denox_hip_builder *b, uint32_t i, char *name, size_t capacity, uint32_t *out_channels) {
+  return guarded([&] { need(b, "builder"); tensorInfo(b->model, b->model.inputs(), i, name, capacity, out_channels); });
+}
+int denox_hip_builder_output_info(const denox_hip_builder *b, uint32_t i, char *name, size_t capacity, uint32_t *out_channels) {
+  return guarded([&] { need(b, "builder"); tensorInfo(b->model, b->model.outputs(), i, name, capacity, out_channels); });
 }
 
 // ---------------------------------------------------------------- compile

@@ -51,6 +51,8 @@ class Tensor:
         self.width, self.height, self.channels = width, height, channels
 
     def __repr__(self):
+        if self.width is None:
+            return f"Tensor({self.name}: C={self.channels})"
         return f"Tensor({self.name}: H={self.height.text} W={self.width.text} C={self.channels})"
 
 
@@ -75,6 +77,30 @@ class Model:
         h, self._h = getattr(self, "_h", None), None
         if h:
             _capi.lib().denox_hip_builder_destroy(h)
+
+    @classmethod
+    def from_onnx(cls, source) -> "Model":
+        """Build the graph from an ONNX file (path) or its bytes, as the reference's
+        ``denox.compile(onnx, ...)`` does (compiler/src/denox/compiler/compile.cpp:21-61).
+        Image tensors are NCHW with N = 1; dynamic height / width dimensions keep their
+        ``dim_param`` names as extents (give them to ``assume=`` / ``instance(...)``)."""
+        if isinstance(source, (bytes, bytearray, memoryview)):
+            data = bytes(source)
+        else:
+            with open(source, "rb") as f:
+                data = f.read()
+        m = cls()
+        m._imported = True
+        _capi.check(_capi.lib().denox_hip_builder_import_onnx(m._h, data, len(data)))
+        from ctypes import c_uint32, create_string_buffer
+        for which, dst in (("input", m.inputs), ("output", m.outputs)):
+            n = c_uint32()
+            _capi.check(getattr(_capi.lib(), f"denox_hip_builder_{which}_count")(m._h, byref(n)))
+            for i in range(n.value):
+                name, ch = create_string_buffer(256), c_uint32()
+                _capi.check(getattr(_capi.lib(), f"denox_hip_builder_{which}_info")(m._h, i, name, 256, byref(ch)))
+                dst.append(Tensor(m, -1, name.value.decode(), None, None, ch.value))
+        return m
 
     # ------------------------------------------------------------- symbols
     def sym(self, v: Union[int, str, Sym]) -> Sym:
@@ -185,6 +211,9 @@ class Model:
     # ------------------------------------------------------------- export for checkers
     def to_ops(self, extents: Dict[str, int]) -> List[dict]:
         """Layer records with symbolic pad / slice amounts evaluated at `extents`."""
+        if getattr(self, "_imported", False):
+            raise ValueError("a model imported from ONNX keeps no Python-side layer record")
+
         def ev(s):
             if not isinstance(s, Sym):
                 return s

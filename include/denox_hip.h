@@ -114,6 +114,20 @@ int denox_hip_builder_pad(denox_hip_builder *b, int src, int64_t left_sym, int64
 int denox_hip_builder_slice(denox_hip_builder *b, int src, int64_t left_sym, int64_t right_sym, int64_t top_sym, int64_t bottom_sym, int *out_tensor);
 int denox_hip_builder_output(denox_hip_builder *b, int src, const char *name);
 
+/* Fills an empty builder from an ONNX ModelProto held in memory: inputs (NCHW, N = 1; dynamic height / width become
+ * named extents after their dim_param), layers and outputs.  Stands for denox::onnx::read
+ * (compiler/src/denox/compiler/frontend/onnx/onnx.cpp:70-158), the first step of denox::compile
+ * (compiler/src/denox/compiler/compile.cpp:21-61).  Operators: Conv, Relu, LeakyRelu, MaxPool, Resize / Upsample
+ * (nearest, integer factor), Concat, Pad (edge), Slice, and the shape arithmetic exporters emit around them;
+ * anything else reports DENOX_HIP_UNSUPPORTED with the operator's name. */
+int denox_hip_builder_import_onnx(denox_hip_builder *b, const void *onnx_bytes, size_t size);
+/* graph inputs / outputs of a builder, in declaration order */
+int denox_hip_builder_input_count(const denox_hip_builder *b, uint32_t *out);
+int denox_hip_builder_output_count(const denox_hip_builder *b, uint32_t *out);
+/* name (written to `name`, at most `capacity` bytes with the terminator) and channel count of input / output i */
+int denox_hip_builder_input_info(const denox_hip_builder *b, uint32_t i, char *name, size_t capacity, uint32_t *out_channels);
+int denox_hip_builder_output_info(const denox_hip_builder *b, uint32_t i, char *name, size_t capacity, uint32_t *out_channels);
+
 /* ------------------------------------------------------------------ compile
  * denox::compile(onnx, db, options) -> bytes (compiler/src/denox/compiler/compile.cpp:21-61)
  * with CompileOptions (compiler/src/denox/compiler/Options.hpp:13-72). */
