@@ -326,7 +326,17 @@ int denox_hip_dnx_describe(const void *dnxbuf, size_t size, const char *const *n
       o << (i ? "," : "") << "{\"buffer\":" << t.buffer << ",\"offset\":" << t.offset.eval(dp) << ",\"size\":" << t.size.eval(dp) << ",\"format\":" << static_cast<int>(t.info.format)
         << ",\"param\":" << (isParam[i] ? "true" : "false") << ",\"name\":";
       jsonEscape(o, t.info.name);
-      if (t.info.has_extent) o << ",\"width\":" << t.info.width.eval(dp) << ",\"height\":" << t.info.height.eval(dp) << ",\"channels\":" << t.info.channels.eval(dp);
+      if (t.info.has_extent) {
+        o << ",\"width\":" << t.info.width.eval(dp) << ",\"height\":" << t.info.height.eval(dp) << ",\"channels\":" << t.info.channels.eval(dp);
+        // the named extent an input's width / height is, when it is one (what `infer` sets from the image it is given)
+        auto nameOf = [&](const dnx::ScalarSource &src) -> const std::string * {
+          if (!src.symbolic) return nullptr;
+          for (const auto &vn : m.value_names) if (vn.value.symbolic && vn.value.value == src.value) return &vn.name;
+          return nullptr;
+        };
+        if (const std::string *nm = nameOf(t.info.width)) { o << ",\"width_name\":"; jsonEscape(o, *nm); }
+        if (const std::string *nm = nameOf(t.info.height)) { o << ",\"height_name\":"; jsonEscape(o, *nm); }
+      }
       o << "}";
     }
     o << "],\"binaries\":" << m.shader_binaries.size() << ",\"dispatches\":[";
