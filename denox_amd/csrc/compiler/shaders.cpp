@@ -45,7 +45,8 @@ std::string fmtFloat(float v) {
 // waves: computing waves; rpw: image rows per wave; ck: input channels per LDS step (0 = all, 1 = half);
 // resident: weights stay in LDS (persistent launch); pw: extra staging-only waves; maxKT: cap on output channels
 // per workgroup (0 = none); mf: matrix shape 32 (32x32x16) or 16 (16x16x32); xb: 16-pixel blocks per row (mf 16).
-struct ConvConfig { unsigned waves, rpw, ck; bool resident; unsigned pw; unsigned maxKT; unsigned mf, xb; const char *name; };
+// pp: two-phase schedule of the persistent kernel (two wave groups alternate matrix work and everything else).
+struct ConvConfig { unsigned waves, rpw, ck; bool resident; unsigned pw; unsigned maxKT; unsigned mf, xb; const char *name; bool pp = false; };
 const ConvConfig kConvConfigs[] = {
     // weights streamed per step
     {4, 2, 16, false, 0, 0, 32, 1, "w4r2k16"}, {4, 2, 32, false, 0, 0, 32, 1, "w4r2k32"}, {4, 4, 16, false, 0, 0, 32, 1, "w4r4k16"}, {4, 4, 32, false, 0, 0, 32, 1, "w4r4k32"},
@@ -70,6 +71,10 @@ const ConvConfig kConvConfigs[] = {
     {4, 2, 32, false, 0, 32, 16, 2, "m4r2k32x2n"}, {4, 2, 0, false, 0, 32, 16, 1, "m4r2kfx1n"}, {4, 1, 0, false, 0, 48, 16, 1, "m4r1kfx1n"}, {4, 2, 32, false, 0, 48, 16, 1, "m4r2k32x1n"},
     {8, 2, 32, true, 0, 0, 16, 2, "q8r2k32x2"}, {8, 1, 32, true, 0, 0, 16, 2, "q8r1k32x2"}, {4, 2, 32, true, 0, 0, 16, 2, "q4r2k32x2"}, {8, 2, 32, true, 0, 0, 16, 1, "q8r2k32x1"},
     {8, 2, 64, true, 0, 0, 16, 2, "q8r2k64x2"}, {4, 2, 32, true, 0, 48, 16, 1, "q4r2k32x1n"},
+    // resident, two-phase schedule
+    {16, 1, 16, true, 0, 0, 32, 1, "t16r1k16", true}, {16, 1, 32, true, 0, 0, 32, 1, "t16r1k32", true}, {16, 2, 16, true, 0, 0, 32, 1, "t16r2k16", true},
+    {8, 2, 16, true, 0, 0, 32, 1, "t8r2k16", true},   {8, 2, 32, true, 0, 0, 32, 1, "t8r2k32", true},   {8, 4, 16, true, 0, 0, 32, 1, "t8r4k16", true},
+    {8, 1, 16, true, 0, 0, 32, 1, "t8r1k16", true},   {8, 2, 32, true, 0, 0, 16, 2, "u8r2k32x2", true}, {16, 1, 32, true, 0, 0, 16, 2, "u16r1k32x2", true},
 };
 constexpr unsigned kNumConvConfigs = sizeof(kConvConfigs) / sizeof(kConvConfigs[0]);
 
@@ -304,6 +309,7 @@ public:
     k.define("WAVES", cfg.waves); k.define("RPW", cfg.rpw); k.define("CK", stepChannels(cfg, g.CPAD));
     if (cfg.resident) k.define("SLOTS", g.slots);
     if (cfg.pw) k.define("PW", cfg.pw);
+    if (cfg.pp) k.define("PP", 1);
     if (cfg.mf != 32) { k.define("MF", cfg.mf); k.define("XB", cfg.xb); }
     std::string entry = "conv3x3_c" + std::to_string(CA) + (up ? "u" : "") + (padA ? "e" : "") + (CB ? "p" + std::to_string(CB) + (padB ? "e" : "") : "") + "_k" +
                         std::to_string(conv.K) + (act == 1 ? "_relu" : act == 2 ? "_lrelu" : "") + (pool ? "_pool" : "") + (crop ? "_crop" : "") + "_" + cfg.name;

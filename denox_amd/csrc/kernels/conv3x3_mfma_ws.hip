@@ -124,6 +124,55 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     if (++dpart == NPARTS)
       pend = false;
   };
+#if PP
+  // Two-phase schedule.  The waves form two groups that every SIMD holds in equal parts ((wave / 4) % 2).  A step has
+  // two phases with a barrier after each: in the first, group A multiplies step k while group B does everything
+  // else (converting and storing finished tiles, writing its share of halo k+1 to LDS, issuing loads); in the second
+  // the roles swap.  The matrix pipe then always has one group feeding it, instead of idling while all waves stage,
+  // convert or wait at the same time.  Halo k+1 goes to the buffer that held halo k-1, which both groups finished
+  // reading before the phase in which the first share is written.
+  static_assert(WAVES % 8 == 0, "two wave groups on four SIMDs");
+  const bool groupB = ((wv >> 2) & 1) != 0;
+  int cchunk = 0, commitChunk = 0;
+  auto mma = [&](int buf) { mma_step<CPADP>(sIn[buf], sW, cchunk * CK, acc, wv, lane, cchunk); };
+  auto post = [&]() { // after this wave's matrix work of a step
+    if (++cchunk == NCHUNK) {
+      pack_tile(acc, done, sBias, lane);
+      zero_acc(acc);
+      dtile = tile;
+      dpart = 0;
+      pend = tile < last; // false in the spare step
+      cchunk = 0;
+      tile += SLOTS;
+    }
+  };
+  auto stage = [&](H::Regs &regs, int buf) { // this wave's share of the next halo, and the refill of the register set
+    if (pend)
+      store_part();
+    H::commit_step(regs, sIn[buf], map, commitChunk);
+    if (++commitChunk == NCHUNK)
+      commitChunk = 0;
+    issue(regs);
+  };
+  H::Regs st0, st1;
+  issue(st0);
+  __builtin_amdgcn_sched_barrier(0); // keep the two sets in issue order: the waits count loads in flight
+  issue(st1);
+  zero_acc(acc);
+  stage(st0, 0); // halo 0, by all waves
+  DNX_SYNC();
+  if (!groupB) {
+    do {
+      mma(0); DNX_SYNC(); post(); stage(st1, 1); DNX_SYNC();
+      mma(1); DNX_SYNC(); post(); stage(st0, 0); DNX_SYNC();
+    } while (tile < last);
+  } else {
+    do {
+      stage(st1, 1); DNX_SYNC(); mma(0); DNX_SYNC(); post();
+      stage(st0, 0); DNX_SYNC(); mma(1); DNX_SYNC(); post();
+    } while (tile < last);
+  }
+#else
   int cchunk = 0, buf = 0;
   auto step = [&](H::Regs &regs) {
     if (cchunk == 0)
@@ -159,6 +208,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     step(st0);
     step(st1);
   } while (tile < last);
+#endif
 #pragma unroll
   for (int p = 0; p < NPARTS; ++p)
     if (pend)

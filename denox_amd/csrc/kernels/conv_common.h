@@ -64,6 +64,9 @@ typedef unsigned short ushort_t;
 #define HALO_PIX (HALO_W * HALO_H)
 #define CKP (CK + 8)
 #define KB (KT / MF)
+#ifndef PP
+#define PP 0 // 1: two-phase schedule of the weight-stationary kernel (wave groups alternate matrix work and everything else)
+#endif
 #ifndef PW
 #define PW 0 // extra waves that only stage halos (weight-stationary kernel)
 #endif

@@ -53,6 +53,8 @@ ALL_CONFIGS = ["w4r2k16", "w4r2k32", "w4r4k16", "w4r4k32", "w8r2k16", "w8r2k32",
 M16_CONFIGS = ["m4r2k32x2", "m4r2k64x2", "m4r1k32x2", "m4r2k32x1", "m4r4k32x1", "m8r2k32x2", "m4r2kfx1", "m4r1kfx2", "m4r2k32x2n",
                "m4r2kfx1n", "m4r1kfx1n", "m4r2k32x1n", "q8r2k32x2", "q8r1k32x2", "q4r2k32x2", "q8r2k32x1", "q8r2k64x2", "q4r2k32x1n"]
 ALL_CONFIGS += M16_CONFIGS
+# two-phase schedule of the persistent kernel
+ALL_CONFIGS += ["t16r1k16", "t16r1k32", "t16r2k16", "t8r2k16", "t8r2k32", "t8r4k16", "t8r1k16", "u8r2k32x2", "u16r1k32x2"]
 
 
 @pytest.mark.parametrize("config", ALL_CONFIGS)
@@ -169,7 +171,7 @@ FUSION_FLAGS = [
 ]
 
 
-@pytest.mark.parametrize("config", ["w4r2k16", "p8r1k16", "p16r1k16", "w8r2k16", "s8r2k16", "s12r1k16"])
+@pytest.mark.parametrize("config", ["w4r2k16", "p8r1k16", "p16r1k16", "w8r2k16", "s8r2k16", "s12r1k16", "t16r1k16", "t8r2k16"])
 @pytest.mark.parametrize("features", [{}, {"pad_fusion": False}, {"slice_fusion": False}, {"pad_fusion": False, "slice_fusion": False}])
 def test_pad_and_slice_fold_into_the_conv(oracle, features, config):
     """pad -> (upsample, pad) concat -> conv -> relu -> slice, with offsets on every side."""
