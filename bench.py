@@ -58,9 +58,54 @@ def cpu_baseline(net: str, kw: dict, seed: int, budget_h: int, budget_w: int) ->
     t0 = time.perf_counter()
     oracle.run_graph(ops, {"input": x}, "f16")
     dt = time.perf_counter() - t0
-    return {"value": budget_h * budget_w / dt * 1e-6, "unit": "Mpix/s", "cores": oracle.num_threads(), "kind": "port",
-            "sample": f"one {budget_w}x{budget_h} frame of the same network, fp32 accumulation, {dt:.1f} s wall",
-            "lavapipe_baseline": lavapipe_probe()}
+    out = {"value": budget_h * budget_w / dt * 1e-6, "unit": "Mpix/s", "cores": oracle.num_threads(), "kind": "port",
+           "sample": f"one {budget_w}x{budget_h} frame of the same network, fp32 accumulation, {dt:.1f} s wall",
+           "lavapipe_baseline": lavapipe_probe()}
+    try:
+        out.update(torch_cpu_baseline(ops, x, budget_h, budget_w))
+    except Exception as e:  # context only: never fail the benchmark over it
+        out["torch_fp32_Mpix_s"] = None
+        out["torch_error"] = str(e)[:200]
+    return out
+
+
+def torch_cpu_baseline(ops, x, h, w) -> dict:
+    """The same frame through torch.nn.functional in fp32 on the host cores: a library evaluation for context beside
+    the oracle's time (the reference's own tests compare against torch, test/system)."""
+    import numpy as np
+    import torch
+    import torch.nn.functional as F
+    env = {"input": torch.from_numpy(np.ascontiguousarray(x.astype(np.float32).transpose(2, 0, 1)))[None]}
+    prepared = []
+    for op in ops:
+        o = dict(op)
+        if o["op"] == "conv2d":
+            o["weight"] = torch.from_numpy(o["weight"].astype(np.float32))
+            o["bias"] = None if o.get("bias") is None else torch.from_numpy(o["bias"].astype(np.float32))
+        prepared.append(o)
+    t0 = time.perf_counter()
+    with torch.no_grad():
+        for o in prepared:
+            k, src = o["op"], o["src"]
+            if k == "conv2d":
+                y = F.conv2d(env[src], o["weight"], o["bias"], stride=o.get("stride", (1, 1)), padding=o.get("padding", (1, 1)))
+            elif k == "activation":
+                y = F.relu(env[src]) if o["func"] == "relu" else F.leaky_relu(env[src], o.get("alpha", 0.0))
+            elif k == "pool":
+                y = F.max_pool2d(env[src], o.get("kernel", (2, 2)))
+            elif k == "upsample":
+                y = F.interpolate(env[src], scale_factor=o.get("factor", 2), mode="nearest")
+            elif k == "concat":
+                y = torch.cat([env[src[0]], env[src[1]]], 1)
+            elif k == "pad":
+                y = F.pad(env[src], (o["left"], o["right"], o["top"], o["bottom"]), mode="replicate")
+            elif k == "slice":
+                y = env[src][:, :, o["top"]:o["top"] + o["out_h"], o["left"]:o["left"] + o["out_w"]]
+            else:
+                raise ValueError(k)
+            env[o["dst"]] = y
+    dt = time.perf_counter() - t0
+    return {"torch_fp32_Mpix_s": h * w / dt * 1e-6, "torch_threads": torch.get_num_threads(), "torch_seconds": round(dt, 2)}
 
 
 def main() -> int:
@@ -134,6 +179,16 @@ def main() -> int:
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ms = dt / args.steps * 1e3
+    # single replays, each synchronised and timed on the host (launch latency included): the spread of the frame time, for
+    # context; `value` is the bulk timing above
+    singles = []
+    for _ in range(min(100, max(20, args.steps))):
+        inst.synchronize()
+        t1 = time.perf_counter()
+        inst.infer_device(ins, outs)
+        inst.synchronize()
+        singles.append((time.perf_counter() - t1) * 1e3)
+    singles.sort()
     out_host = d_out.cpu().numpy()
     if not np.isfinite(out_host).all():
         print("bench.py: non-finite output", file=sys.stderr)
@@ -196,7 +251,8 @@ def main() -> int:
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": f"{description}; {mod.runtime_model.dispatch_count} dispatches in one hipGraph", "device_bytes": inst.device_bytes,
                    "schedule": "min-cost over measured dispatch latencies" if db is not None else "min-cost over roofline estimates",
-                   "tuning_seconds": round(tune_s, 2), "host_pointer_path_ms_per_frame": round(host_ms, 3)},
+                   "tuning_seconds": round(tune_s, 2), "host_pointer_path_ms_per_frame": round(host_ms, 3),
+                   "single_replay_ms_median": round(singles[len(singles) // 2], 4), "single_replay_ms_p95": round(singles[int(len(singles) * 0.95)], 4)},
         "roofline": roofline,
     }
     if not args.no_cpu_baseline:
