@@ -1,0 +1,75 @@
+"""Seeded random layer graphs on the GPU against the CPU oracle: channel counts, extents, pad / crop offsets, fusion
+switches and kernel configurations drawn at random, so that combinations nobody listed by hand get exercised
+(odd extents down to 1 x 1, channel counts around the 8 / 16 / 32 vector and block boundaries, every prologue and
+epilogue of the conv kernels in one dispatch).  Each case prints its parameters before it runs."""
+import numpy as np
+import pytest
+
+import denox_amd as dx
+from util import assert_conv_close, he_weights, small_bias
+
+pytestmark = pytest.mark.gpu
+
+CONFIGS = [None, None, None, "w4r2k16", "w4r1k32", "w8r2k32", "w2r2kfn", "w4r1kfm", "p8r1k16", "p16r1k16", "p8r2k32", "p4r4k16", "p4r2k32n",
+           "s8r2k16", "m4r2k32x2", "m4r1kfx2", "m4r2kfx1n", "q8r2k32x2", "q4r2k32x1n", "t16r1k16", "t8r2k16", "u8r2k32x2"]
+CHANNELS = [1, 2, 3, 7, 8, 9, 15, 16, 17, 24, 31, 32, 33, 40, 48, 64, 73, 80]
+
+
+def one_case(oracle, seed):
+    rng = np.random.default_rng(seed)
+    H, W = int(rng.integers(1, 48)), int(rng.integers(1, 72))
+    up, cat = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+    pool, crop, pad = bool(rng.integers(0, 2)), bool(rng.integers(0, 3) == 0), bool(rng.integers(0, 3) == 0)
+    act = ["none", "relu", "leaky"][int(rng.integers(0, 3))]
+    CA, CB, K = (int(rng.choice(CHANNELS)) for _ in range(3))
+    config = CONFIGS[int(rng.integers(0, len(CONFIGS)))]
+    feats = {k: bool(rng.integers(0, 4)) for k in ("conv_relu_fusion", "concat_conv_fusion", "upsample_fusion", "pool_fusion", "pad_fusion", "slice_fusion")}
+    if up:
+        H, W = 2 * max(1, H // 2), 2 * max(1, W // 2)
+    pl, pr, pt, pb = (int(v) for v in rng.integers(0, 5, 4)) if pad else (0, 0, 0, 0)
+    print(f"fuzz seed={seed} H={H} W={W} CA={CA} CB={CB if cat else 0} K={K} up={up} pool={pool} pad={(pl, pr, pt, pb)} crop={crop} act={act} config={config} feats={feats}", flush=True)
+
+    m = dx.Model()
+    feeds = {}
+    Hs, Ws = H - pt - pb, W - pl - pr  # extents of the stored (un-padded) full-resolution source
+    if pad and (Hs < 1 or Ws < 1):
+        pad, (pl, pr, pt, pb), Hs, Ws = False, (0, 0, 0, 0), H, W
+    if up:
+        a = m.input("a", m.sym("W") // 2, m.sym("H") // 2, CA)
+        feeds["a"] = rng.standard_normal((H // 2, W // 2, CA)).astype(np.float16)
+        t = m.upsample(a)
+    else:
+        a = m.input("a", m.sym("W") - (pl + pr), m.sym("H") - (pt + pb), CA)
+        feeds["a"] = rng.standard_normal((Hs, Ws, CA)).astype(np.float16)
+        t = m.pad(a, pl, pr, pt, pb) if pad else a
+    C = CA
+    if cat:
+        b = m.input("b", m.sym("W") - (pl + pr), m.sym("H") - (pt + pb), CB)
+        feeds["b"] = rng.standard_normal((Hs, Ws, CB)).astype(np.float16)
+        t = m.concat(t, m.pad(b, pl, pr, pt, pb) if pad else b)
+        C += CB
+    t = m.conv2d(t, he_weights(rng, K, C), small_bias(rng, K) if rng.integers(0, 4) else None)
+    if act == "relu":
+        t = m.relu(t)
+    elif act == "leaky":
+        t = m.activation(t, "leaky_relu", 0.125)
+    if pool and H >= 2 and W >= 2:
+        t = m.pool(t)
+    elif crop and H >= 3 and W >= 3:
+        l, tp = int(rng.integers(0, W // 2)), int(rng.integers(0, H // 2))
+        t = m.slice(t, l, int(rng.integers(l + 1, W + 1)), tp, int(rng.integers(tp + 1, H + 1)))
+    m.output(t)
+    try:
+        mod = dx.Module.compile(m, features=feats, conv_config=config)
+    except dx.DenoxHipError as e:
+        assert e.status == 5, str(e)  # this configuration does not exist for this layer
+        mod = dx.Module.compile(m, features=feats)
+    got = mod.instance(H=H, W=W).infer(*[feeds[k] for k in ("a", "b") if k in feeds])[0]
+    want = oracle.run_graph(m.to_ops({"H": H, "W": W}), feeds, "fp32")[t.name]
+    assert_conv_close(got, want, f"fuzz seed {seed}")
+
+
+@pytest.mark.parametrize("block", range(8))
+def test_random_fused_conv_graphs(oracle, block):
+    for seed in range(block * 25, block * 25 + 25):
+        one_case(oracle, seed)
