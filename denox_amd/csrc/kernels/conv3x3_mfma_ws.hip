@@ -68,9 +68,6 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   int tile = first + slot;
   if (tile >= last)
     return; // uniform for the workgroup: nothing was staged yet
-#ifdef DBG_STAGGER // timing experiment: de-synchronise the workgroups at the start
-  for (int i = 0; i < ((b / NXCD) % 8); ++i) __builtin_amdgcn_s_sleep(DBG_STAGGER);
-#endif
   const bool rev = (pc.FLAGS & 1u) != 0;
   // position of the t-th tile of the walk
   auto tileY = [&](int t) { return ((rev ? numTiles - 1 - t : t) / tilesX) * TH; };

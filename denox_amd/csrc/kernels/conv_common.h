@@ -64,6 +64,9 @@ typedef unsigned short ushort_t;
 #define HALO_PIX (HALO_W * HALO_H)
 #define CKP (CK + 8)
 #define KB (KT / MF)
+#ifndef STORE_AUX
+#define STORE_AUX 0 // cache policy bits of the output stores (bit 1: non-temporal)
+#endif
 #ifndef PP
 #define PP 0 // 1: two-phase schedule of the weight-stationary kernel (wave groups alternate matrix work and everything else)
 #endif
@@ -437,16 +440,16 @@ __device__ DNX_INLINE void store16(OutBuf out, bool ok, unsigned pix, const half
   const unsigned off = (pix * (unsigned)KOUT + (unsigned)chb) * 2u;
   if (KOUT % 16 == 0) {
     const unsigned o0 = (ok && chb < KOUT) ? off : NO_STORE;
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, o[0]), out, o0, 0, 0);
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, o[1]), out, o0 + 16u, 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, o[0]), out, o0, 0, STORE_AUX);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, o[1]), out, o0 + 16u, 0, STORE_AUX);
   } else if (KOUT % 8 == 0) {
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, o[0]), out, (ok && chb < KOUT) ? off : NO_STORE, 0, 0);
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, o[1]), out, (ok && chb + 8 < KOUT) ? off + 16u : NO_STORE, 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, o[0]), out, (ok && chb < KOUT) ? off : NO_STORE, 0, STORE_AUX);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, o[1]), out, (ok && chb + 8 < KOUT) ? off + 16u : NO_STORE, 0, STORE_AUX);
   } else {
 #pragma unroll
     for (int i = 0; i < (KOUT < 16 ? KOUT : 16); ++i) {
       const _Float16 h = o[i >> 3][i & 7]; // a vector element is no object: copy it before reinterpreting its bits
-      __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(ushort_t, h), out, (ok && chb + i < KOUT) ? off + 2u * i : NO_STORE, 0, 0);
+      __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(ushort_t, h), out, (ok && chb + i < KOUT) ? off + 2u * i : NO_STORE, 0, STORE_AUX);
     }
   }
 }
@@ -614,12 +617,12 @@ __device__ DNX_INLINE void store_vec(OutBuf out, bool ok, unsigned pix, const _F
     half8 h;
 #pragma unroll
     for (int i = 0; i < 8; ++i) h[i] = o[i];
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, h), out, (ok && chb < KOUT) ? off : NO_STORE, 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, h), out, (ok && chb < KOUT) ? off : NO_STORE, 0, STORE_AUX);
   } else {
 #pragma unroll
     for (int i = 0; i < 8; ++i)
       if (i < n)
-        __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(ushort_t, o[i]), out, (ok && chb + i < KOUT) ? off + 2u * i : NO_STORE, 0, 0);
+        __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(ushort_t, o[i]), out, (ok && chb + i < KOUT) ? off + 2u * i : NO_STORE, 0, STORE_AUX);
   }
 }
 
