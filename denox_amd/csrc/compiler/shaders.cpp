@@ -82,6 +82,7 @@ enum ConvPatternBits : unsigned { PAT_CONCAT = 1, PAT_UPSAMPLE = 2, PAT_ACT = 4,
 
 struct ConvGeometry {
   unsigned CA, CB, C, CPAD, K, KOUTP, KT, slots;
+  unsigned R = 3, S = 3; // filter rows / columns (set before chooseKT)
   size_t ldsBytes;
 };
 
@@ -106,7 +107,7 @@ bool chooseKT(const ConvConfig &cfgIn, unsigned CA, unsigned CB, unsigned K, con
   if (cfg.ck > 192 || cfg.ck % kstep) return false; // staging registers; whole matrix steps only
   const unsigned th = cfg.waves * cfg.rpw;
   const unsigned tw = cfg.mf == 32 ? 32 : 16 * cfg.xb;
-  const unsigned haloPix = (th + 2) * (tw + 2);
+  const unsigned haloPix = (th + g.R - 1) * (tw + g.S - 1), taps = g.R * g.S;
   const unsigned ckp = cfg.ck + 8;
   const unsigned blocks = g.KOUTP / blk;
   // registers per lane: 512 shared by the waves of one SIMD; a workgroup of `waves` waves puts waves/4 on each
@@ -117,10 +118,16 @@ bool chooseKT(const ConvConfig &cfgIn, unsigned CA, unsigned CB, unsigned K, con
     if (cfg.maxKT && kb * blk > cfg.maxKT) continue;
     const unsigned accRegs = cfg.mf == 32 ? kb * cfg.rpw * 16 : kb * cfg.rpw * cfg.xb * 4;
     if (accRegs + 64 + (cfg.mf == 16 ? kb * 4 : 0) > regBudget) continue;
-    const size_t lds = (cfg.resident ? static_cast<size_t>(9u * kb * blk) * (g.CPAD + 8) * 2u + 2u * static_cast<size_t>(haloPix) * ckp * 2u
-                                     : (static_cast<size_t>(haloPix) + 9u * kb * blk) * ckp * 2u) +
+    const size_t lds = (cfg.resident ? static_cast<size_t>(taps * kb * blk) * (g.CPAD + 8) * 2u + 2u * static_cast<size_t>(haloPix) * ckp * 2u
+                                     : (static_cast<size_t>(haloPix) + taps * kb * blk) * ckp * 2u) +
                        static_cast<size_t>(kb * blk) * 2u; // + the staged bias
     if (lds > dev.maxComputeSharedMemory) continue;
+    if (taps > 9) { // larger filters: the registers that stage one step's weights and halo share count as well
+      const unsigned vppk = cfg.ck / 8, threads = cfg.waves * 64, stagers = (cfg.pw ? cfg.pw : cfg.waves) * 64;
+      const unsigned stage = cfg.resident ? 2 * 4 * ((haloPix * vppk + stagers - 1) / stagers)
+                                          : 4 * ((taps * kb * blk * vppk + threads - 1) / threads + (haloPix * vppk + threads - 1) / threads);
+      if (accRegs + stage + 48 > regBudget) continue;
+    }
     g.KT = kb * blk;
     g.ldsBytes = lds;
     const unsigned nkt = blocks / kb;
@@ -142,23 +149,24 @@ unsigned rowChannel(unsigned mf, unsigned KT, unsigned row) {
   return paired ? 32 * (kb / 2) + 8 * grp + 4 * (kb % 2) + jj : 16 * kb + 4 * grp + jj;
 }
 
-// Weight layout the kernels read: [kt][chunk][tap r*3+s][KT rows][len(chunk)], rows
+// Weight layout the kernels read: [kt][chunk][tap r*S+s][KT rows][len(chunk)], rows
 // permuted by rowChannel(); zero for c >= C or k >= K.
 // (The resident kernel uses one chunk spanning the whole reduction.)
 std::vector<uint8_t> packConvWeights(const Op &conv, const ConvGeometry &g, unsigned ck, unsigned mf) {
-  std::vector<uint16_t> out(static_cast<size_t>(g.KOUTP) * 9 * g.CPAD, 0);
+  const unsigned R = conv.R, S = conv.S;
+  std::vector<uint16_t> out(static_cast<size_t>(g.KOUTP) * R * S * g.CPAD, 0);
   const unsigned nkt = g.KOUTP / g.KT;
   size_t pos = 0;
   for (unsigned kt = 0; kt < nkt; ++kt)
     for (unsigned c0 = 0; c0 < g.CPAD; c0 += ck) {
       const unsigned len = std::min(ck, g.CPAD - c0);
-      for (unsigned tap = 0; tap < 9; ++tap) {
-        const unsigned r = tap / 3, s = tap % 3;
+      for (unsigned tap = 0; tap < R * S; ++tap) {
+        const unsigned r = tap / S, s = tap % S;
         for (unsigned row = 0; row < g.KT; ++row) {
           const unsigned k = kt * g.KT + rowChannel(mf, g.KT, row);
           for (unsigned e = 0; e < len; ++e, ++pos) {
             const unsigned c = c0 + e;
-            if (k < g.K && c < g.C) out[pos] = conv.weights[((static_cast<size_t>(k) * g.C + c) * 3 + r) * 3 + s];
+            if (k < g.K && c < g.C) out[pos] = conv.weights[((static_cast<size_t>(k) * g.C + c) * R + r) * S + s];
           }
         }
       }
@@ -193,7 +201,9 @@ public:
     for (size_t i = 0; i < ops.size(); ++i) {
       const Op &conv = ops[i];
       if (conv.kind != OpKind::Conv) continue;
-      if (conv.R != 3 || conv.S != 3 || conv.strideX != 1 || conv.strideY != 1 || conv.padX != 1 || conv.padY != 1 || conv.dilX != 1 || conv.dilY != 1) continue;
+      // odd filter extents up to 7 with "same" zero padding, stride 1, no dilation
+      if (conv.R % 2 == 0 || conv.S % 2 == 0 || conv.R > 7 || conv.S > 7 || conv.strideX != 1 || conv.strideY != 1 || conv.padX != (conv.S - 1) / 2 ||
+          conv.padY != (conv.R - 1) / 2 || conv.dilX != 1 || conv.dilY != 1) continue;
       // A fused-away tensor may have other consumers: whoever needs it materialised gets it
       // from another edge, and the selection weighs both.
       struct Pro { unsigned bits; std::vector<int> ops; std::vector<int> inputs; };
@@ -265,6 +275,7 @@ public:
       if ((m.pattern & PAT_POOL) && (cfg.rpw % 2)) continue;
       if ((cfg.waves + cfg.pw) * 64 > opt.deviceInfo.maxComputeWorkGroupInvocations) continue;
       ConvGeometry g;
+      g.R = conv.R; g.S = conv.S;
       if (!chooseKT(cfg, CA, CB, conv.K, opt.deviceInfo, g)) continue;
       out.push_back(c);
     }
@@ -275,7 +286,7 @@ public:
   size_t parameterMemorySize(const Model &model, const Match &m) const override {
     const Op &conv = opOf(model, m, OpKind::Conv);
     const unsigned C = conv.C, cpad = (C + 31) / 32 * 32, kp = (conv.K + 31) / 32 * 32; // upper bound over configurations
-    return static_cast<size_t>(kp) * 9 * cpad * 2 + static_cast<size_t>(kp) * 2;
+    return static_cast<size_t>(kp) * conv.R * conv.S * cpad * 2 + static_cast<size_t>(kp) * 2;
   }
 
   void implement(OpImpl &impl, const Model &model, const Match &m, unsigned config, SymGraph &sym, const CompileOptions &opt) const override {
@@ -286,6 +297,7 @@ public:
     const unsigned CA = tA.channels;
     const unsigned CB = m.inputs.size() > 1 ? model.tensors()[m.inputs[1]].channels : 0;
     ConvGeometry g;
+    g.R = conv.R; g.S = conv.S;
     if (!chooseKT(cfg, CA, CB, conv.K, opt.deviceInfo, g)) fail(Status::Internal, "conv config rejected at implement time");
     int act = 0;
     float alpha = 0.0f;
@@ -310,8 +322,9 @@ public:
     if (cfg.resident) k.define("SLOTS", g.slots);
     if (cfg.pw) k.define("PW", cfg.pw);
     if (cfg.pp) k.define("PP", 1);
+    if (conv.R != 3 || conv.S != 3) { k.define("KR", conv.R); k.define("KS", conv.S); }
     if (cfg.mf != 32) { k.define("MF", cfg.mf); k.define("XB", cfg.xb); }
-    std::string entry = "conv3x3_c" + std::to_string(CA) + (up ? "u" : "") + (padA ? "e" : "") + (CB ? "p" + std::to_string(CB) + (padB ? "e" : "") : "") + "_k" +
+    std::string entry = "conv" + std::to_string(conv.R) + "x" + std::to_string(conv.S) + "_c" + std::to_string(CA) + (up ? "u" : "") + (padA ? "e" : "") + (CB ? "p" + std::to_string(CB) + (padB ? "e" : "") : "") + "_k" +
                         std::to_string(conv.K) + (act == 1 ? "_relu" : act == 2 ? "_lrelu" : "") + (pool ? "_pool" : "") + (crop ? "_crop" : "") + "_" + cfg.name;
     k.define("KERNEL_NAME", entry);
     const Sym W = convIn.width, H = convIn.height;
@@ -324,7 +337,7 @@ public:
     d.addBinding(dnx::Access::WriteOnly, m.output);
     const Op convCopy = conv; // the lazy packers outlive the model reference
     const unsigned ck = cfg.resident ? g.CPAD : stepChannels(cfg, g.CPAD);
-    TensorId wt = impl.createParameter(static_cast<size_t>(g.KOUTP) * 9 * g.CPAD * 2, dnx::ScalarType::F16,
+    TensorId wt = impl.createParameter(static_cast<size_t>(g.KOUTP) * conv.R * conv.S * g.CPAD * 2, dnx::ScalarType::F16,
                                        [convCopy, g, ck, mf = cfg.mf]() { return packConvWeights(convCopy, g, ck, mf); });
     d.addParamBinding(wt);
     if (conv.hasBias) {
@@ -350,7 +363,8 @@ public:
     }
     d.addTraversalFlag();
 
-    std::string nm = "conv3x3";
+    const std::string base = "conv" + std::to_string(conv.R) + "x" + std::to_string(conv.S);
+    std::string nm = base;
     if (up) nm = "upsample+" + nm;
     if (padA || padB) nm = "pad+" + nm;
     if (m.pattern & PAT_CONCAT) nm = "concat+" + nm;
@@ -364,10 +378,10 @@ public:
     // bytes that cross HBM: sources at their stored resolution, weights, bias; the (pooled / cropped) output
     Sym reads = bytesOf(sym, tA);
     if (CB) reads = sym.add(reads, bytesOf(sym, model.tensors()[m.inputs[1]]));
-    reads = sym.add(reads, static_cast<int64_t>(conv.K) * conv.C * 9 * 2 + (conv.hasBias ? conv.K * 2 : 0));
+    reads = sym.add(reads, static_cast<int64_t>(conv.K) * conv.C * conv.R * conv.S * 2 + (conv.hasBias ? conv.K * 2 : 0));
     d.setMemoryReads(reads);
     d.setMemoryWrites(bytesOf(sym, model.tensors()[m.output]));
-    d.setFlops(sym.mul(sym.mul(W, H), static_cast<int64_t>(2) * 9 * conv.C * conv.K));
+    d.setFlops(sym.mul(sym.mul(W, H), static_cast<int64_t>(2) * conv.R * conv.S * conv.C * conv.K));
   }
 
 private:

@@ -21,7 +21,7 @@
 #define KERNEL_NAME conv3x3_mfma
 #endif
 
-#define NV_W ((9 * KT * VPPK + NT - 1) / NT)
+#define NV_W ((NTAPS * KT * VPPK + NT - 1) / NT)
 
 // weight slice of one step: global [tap][KT rows][L] -> registers -> LDS rows of CKP
 template <int L>
@@ -30,7 +30,7 @@ __device__ DNX_INLINE void weights_fetch(const _Float16 *__restrict__ wchunk, ui
 #pragma unroll
   for (int it = 0; it < NV_W; ++it) {
     const int i = tid + it * NT;
-    if (i < 9 * KT * VPP)
+    if (i < NTAPS * KT * VPP)
       st[it] = ld16(wchunk + (size_t)i * 8);
   }
 }
@@ -41,7 +41,7 @@ __device__ DNX_INLINE void weights_commit(const uint4v (&st)[NV_W], _Float16 *sW
 #pragma unroll
   for (int it = 0; it < NV_W; ++it) {
     const int i = tid + it * NT;
-    if (i < 9 * KT * VPP) {
+    if (i < NTAPS * KT * VPP) {
       const int row = i / VPP;
       const int v = i - row * VPP;
       *reinterpret_cast<uint4v *>(sW + row * CKP + v * 8) = st[it];
@@ -60,7 +60,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
 #endif
     PushConstants pc) {
   __shared__ __attribute__((aligned(16))) _Float16 sIn[HALO_PIX * CKP];
-  __shared__ __attribute__((aligned(16))) _Float16 sW[9 * KT * CKP];
+  __shared__ __attribute__((aligned(16))) _Float16 sW[NTAPS * KT * CKP];
   __shared__ __attribute__((aligned(16))) _Float16 sBias[KT];
 #if CB == 0
   const _Float16 *B = nullptr;
@@ -84,7 +84,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   stage_bias(sBias, BIAS, kt, tid);
 
   // packed filter: [kt][chunk][tap][KT][len(chunk)]
-  const _Float16 *wbase = FILT + (size_t)kt * 9 * KT * CPAD;
+  const _Float16 *wbase = FILT + (size_t)kt * NTAPS * KT * CPAD;
   typedef Halo<NT> H;
   H::Map map;
   H::Src src;
@@ -106,7 +106,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
       weights_commit<TAIL>(stW, sW, tid);
     DNX_SYNC();
     if (chunk + 1 < NCHUNK) { // loads for the next step fly during the MFMAs below
-      const _Float16 *wnext = wbase + (size_t)9 * KT * (chunk + 1) * CK;
+      const _Float16 *wnext = wbase + (size_t)NTAPS * KT * (chunk + 1) * CK;
       H::fetch_step(srcs, stIn, map, src, chunk + 1);
       if (TAIL == CK || chunk + 1 < NCHUNK - 1)
         weights_fetch<CK>(wnext, stW, tid);

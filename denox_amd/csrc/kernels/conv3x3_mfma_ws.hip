@@ -38,7 +38,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     const _Float16 *__restrict__ BIAS,
 #endif
     PushConstants pc) {
-  __shared__ __attribute__((aligned(16))) _Float16 sW[9 * KT * CPADP];
+  __shared__ __attribute__((aligned(16))) _Float16 sW[NTAPS * KT * CPADP];
   __shared__ __attribute__((aligned(16))) _Float16 sIn[2][HALO_PIX * CKP];
   __shared__ __attribute__((aligned(16))) _Float16 sBias[KT];
 #if CB == 0
@@ -76,9 +76,9 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   stage_bias(sBias, BIAS, kt, tid);
   // ---- resident weights: global [tap][KT][CPAD] (one chunk = whole reduction) -> LDS rows of CPADP ----
   {
-    const _Float16 *wsrc = FILT + (size_t)kt * 9 * KT * CPAD;
+    const _Float16 *wsrc = FILT + (size_t)kt * NTAPS * KT * CPAD;
     constexpr int VPR = CPAD / 8;
-    for (int i = tid; i < 9 * KT * VPR; i += NT) {
+    for (int i = tid; i < NTAPS * KT * VPR; i += NT) {
       const int row = i / VPR;
       const int v = i - row * VPR;
       *reinterpret_cast<uint4v *>(sW + row * CPADP + v * 8) = ld16(wsrc + (size_t)i * 8);

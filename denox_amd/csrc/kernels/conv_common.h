@@ -2,7 +2,7 @@
 // source loader (concat / upsample / replicate-pad folded into the addressing)
 // and the epilogue (bias, activation, rounding, 2x2 max pool or crop, store).
 //
-//   out[y,x,k] = act(bias[k] + sum_{r,s,c} src[y+r-1, x+s-1, c] * W[k,c,r,s])       (zero outside the image)
+//   out[y,x,k] = act(bias[k] + sum_{r,s,c} src[y+r-PADY, x+s-PADX, c] * W[k,c,r,s])   (zero outside the image; KR x KS taps)
 //   src[y,x,c] = c < CA ? A'[y,x,c] : B'[y,x,c-CA]
 //   A' = UPA ? A[y/2, x/2] : (PADA ? A[clamp(y-PAD_T), clamp(x-PAD_L)] : A[y,x]),   B' likewise with PADB
 //
@@ -46,6 +46,16 @@ typedef unsigned short ushort_t;
 // channels per step), MF = 16 -> v_mfma_f32_16x16x32_f16 (16 x 16 per block, 32 input channels per step; XB blocks
 // side by side in x).  The 16-wide shape wastes less on output-channel counts like 48, 80, 112 or 3 and makes
 // smaller tiles for low-resolution layers; the 32-wide shape pads input channels less (73 -> 80 instead of 96).
+// Filter extent KR x KS (odd; the convolution keeps the image extent: zero padding (KR-1)/2, (KS-1)/2, stride 1).
+#ifndef KR
+#define KR 3
+#endif
+#ifndef KS
+#define KS 3
+#endif
+#define NTAPS (KR * KS)
+#define PADY ((KR - 1) / 2)
+#define PADX ((KS - 1) / 2)
 #ifndef MF
 #define MF 32
 #endif
@@ -59,8 +69,8 @@ typedef unsigned short ushort_t;
 #define TAIL (CPAD - (NCHUNK - 1) * CK)
 #define TW (MF == 32 ? 32 : 16 * XB)
 #define TH (WAVES * RPW)
-#define HALO_W (TW + 2)
-#define HALO_H (TH + 2)
+#define HALO_W (TW + KS - 1)
+#define HALO_H (TH + KR - 1)
 #define HALO_PIX (HALO_W * HALO_H)
 #define CKP (CK + 8)
 #define KB (KT / MF)
@@ -295,8 +305,8 @@ struct Halo {
   static __device__ DNX_INLINE void src_init(Src &s, const Map &m, int y0, int x0, const PushConstants &pc) {
 #pragma unroll
     for (int it = 0; it < NV; ++it) {
-      const int gy = y0 + m.hy[it] - 1;
-      const int gx = x0 + m.hx[it] - 1;
+      const int gy = y0 + m.hy[it] - PADY;
+      const int gx = x0 + m.hx[it] - PADX;
       size_t pa = 0, pb = 0;
       const bool inside = m.lds[it] >= 0 && gy >= 0 && gy < (int)pc.IN_H && gx >= 0 && gx < (int)pc.IN_W;
       if (inside)
@@ -559,20 +569,20 @@ mma_chunk(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, int wv, i
   const int l32 = lane & 31;
   const int kq = (lane >> 5) * 8;
 #pragma unroll
-  for (int s = 0; s < 3; ++s) {
+  for (int s = 0; s < KS; ++s) {
 #pragma unroll
     for (int ks = 0; ks < L / 16; ++ks) {
       const int kk = ks * 16 + kq;
-      half8 px[RPW + 2];
+      half8 px[RPW + KR - 1];
 #pragma unroll
-      for (int hr = 0; hr < RPW + 2; ++hr)
+      for (int hr = 0; hr < RPW + KR - 1; ++hr)
         px[hr] = *reinterpret_cast<const half8 *>(sIn + ((wv * RPW + hr) * HALO_W + l32 + s) * CKP + kk);
 #pragma unroll
-      for (int r = 0; r < 3; ++r) {
+      for (int r = 0; r < KR; ++r) {
         half8 wf[KB];
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
-          wf[kb] = *reinterpret_cast<const half8 *>(sW + (((r * 3 + s) * KT) + kb * 32 + l32) * WPITCH + wofs + kk);
+          wf[kb] = *reinterpret_cast<const half8 *>(sW + (((r * KS + s) * KT) + kb * 32 + l32) * WPITCH + wofs + kk);
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -723,22 +733,22 @@ mma_chunk(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, int wv, i
   const int l16 = lane & 15;
   const int kq = (lane >> 4) * 8;
 #pragma unroll
-  for (int s = 0; s < 3; ++s) {
+  for (int s = 0; s < KS; ++s) {
 #pragma unroll
     for (int ks = 0; ks < L / 32; ++ks) {
       const int kk = ks * 32 + kq;
-      half8 px[RPW + 2][XB];
+      half8 px[RPW + KR - 1][XB];
 #pragma unroll
-      for (int hr = 0; hr < RPW + 2; ++hr)
+      for (int hr = 0; hr < RPW + KR - 1; ++hr)
 #pragma unroll
         for (int xb = 0; xb < XB; ++xb)
           px[hr][xb] = *reinterpret_cast<const half8 *>(sIn + ((wv * RPW + hr) * HALO_W + xb * 16 + l16 + s) * CKP + kk);
 #pragma unroll
-      for (int r = 0; r < 3; ++r) {
+      for (int r = 0; r < KR; ++r) {
         half8 wf[KB];
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
-          wf[kb] = *reinterpret_cast<const half8 *>(sW + (((r * 3 + s) * KT) + kb * 16 + l16) * WPITCH + wofs + kk);
+          wf[kb] = *reinterpret_cast<const half8 *>(sW + (((r * KS + s) * KT) + kb * 16 + l16) * WPITCH + wofs + kk);
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
 #pragma unroll

@@ -105,6 +105,37 @@ def test_conv_16x16_shape_odd_channel_counts(oracle, config, CA, CB, K, H, W):
     assert_conv_close(got, want, config)
 
 
+@pytest.mark.parametrize("config", [None, "w4r2k16", "p8r1k16", "m4r2k32x2", "t8r2k16", "s8r2k16"])
+@pytest.mark.parametrize("R,S", [(1, 1), (5, 5), (1, 3), (3, 1), (7, 7), (5, 3)])
+def test_odd_filter_extents(oracle, R, S, config):
+    """R x S filters with "same" zero padding (the reference's direct_conv.comp takes any extent), bare and with the
+    upsample + concat prologue and the pool epilogue."""
+    rng = np.random.default_rng(R * 10 + S)
+    H, W, CA, CB, K = 26, 44, 24, 9, 40
+    pad = ((R - 1) // 2, (S - 1) // 2)
+    lo = rng.standard_normal((H // 2, W // 2, CA)).astype(np.float16)
+    x = rng.standard_normal((H, W, CB)).astype(np.float16)
+    w1 = (rng.standard_normal((K, CA + CB, R, S)) * np.sqrt(2.0 / (R * S * (CA + CB)))).astype(np.float16)
+    w2 = (rng.standard_normal((16, CB, R, S)) * np.sqrt(2.0 / (R * S * CB))).astype(np.float16)
+    m = dx.Model()
+    a = m.input("lo", m.sym("W") // 2, m.sym("H") // 2, CA)
+    b = m.input("x", "W", "H", CB)
+    o1 = m.pool(m.relu(m.conv2d(m.concat(m.upsample(a), b), w1, small_bias(rng, K), padding=pad)))
+    o2 = m.conv2d(b, w2, None, padding=pad)
+    m.output(o1, "o1")
+    m.output(o2, "o2")
+    try:
+        mod = dx.Module.compile(m, conv_config=config)
+    except dx.DenoxHipError as e:
+        assert e.status == 5
+        pytest.skip(str(e))
+    assert f"conv{R}x{S}" in dx.last_compile_report() and mod.runtime_model.dispatch_count == 2
+    got1, got2 = mod.instance(H=H, W=W).infer(lo, x)
+    env = oracle.run_graph(m.to_ops({"H": H, "W": W}), {"lo": lo, "x": x}, "fp32")
+    assert_conv_close(got1, env[o1.name], f"{R}x{S} fused {config}")
+    assert_conv_close(got2, env[o2.name], f"{R}x{S} bare {config}")
+
+
 def test_tensor_size_limit_is_reported():
     """Tensors are addressed with 32-bit byte offsets: extents that make one reach 4 GiB are refused when the
     instance is created, before anything is allocated."""

@@ -162,6 +162,20 @@ def test_resize_scales_input_position_follows_the_opset(opset, scales_at):
     assert (out["height"], out["width"]) == (18, 24)
 
 
+def test_one_by_one_and_five_by_five_convs_import():
+    w1, w5 = np.zeros((4, 8, 1, 1), np.float32), np.zeros((8, 4, 5, 5), np.float32)
+    nodes = [node("Conv", ["x", "w1"], ["a"], attr_ints("kernel_shape", [1, 1])),
+             node("Conv", ["a", "w5"], ["y"], attr_ints("kernel_shape", [5, 5]), attr_ints("pads", [2, 2, 2, 2]))]
+    onnx = model(nodes, [value_info("x", (1, 8, "H", "W"))], [value_info("y", (1, 8, "H", "W"))], [tensor("w1", w1), tensor("w5", w5)])
+    assert dispatch_names(dx.compile_model(dx.Model.from_onnx(onnx)), H=9, W=9) == ["conv1x1", "conv5x5"]
+    # a 5x5 filter without padding changes the extent: no kernel for that
+    nodes[1] = node("Conv", ["a", "w5"], ["y"], attr_ints("kernel_shape", [5, 5]))
+    onnx = model(nodes, [value_info("x", (1, 8, "H", "W"))], [value_info("y", (1, 8, "h", "w"))], [tensor("w1", w1), tensor("w5", w5)])
+    with pytest.raises(dx.DenoxHipError) as e:
+        dx.compile_model(dx.Model.from_onnx(onnx))
+    assert e.value.status == 5
+
+
 def test_unsupported_and_malformed_models_are_reported():
     with pytest.raises(dx.DenoxHipError) as e:
         dx.Model.from_onnx(conv_model([node("Softmax", ["c"], ["y"], name="sm0")], "y", (1, 8, "h", "w")))
