@@ -17,6 +17,7 @@ struct Features {
   bool enablePoolFusion = true;       // conv stores the 2x2 max only
   bool enablePadFusion = true;        // conv reads an un-padded source through the replicate clamp
   bool enableSliceFusion = true;      // conv stores only the cropped window
+  bool enableUpsampleFold = true;     // candidates that fold a fused 2x upsample into the conv weights (2x2 taps per output parity)
   bool enableAlternatingTraversal = true; // consecutive conv dispatches walk their tiles in opposite directions
   bool enableImplicitConcat = true;   // memory-aliasing concat where layouts allow it
 };

@@ -46,7 +46,8 @@ std::string fmtFloat(float v) {
 // resident: weights stay in LDS (persistent launch); pw: extra staging-only waves; maxKT: cap on output channels
 // per workgroup (0 = none); mf: matrix shape 32 (32x32x16) or 16 (16x16x32); xb: 16-pixel blocks per row (mf 16).
 // pp: two-phase schedule of the persistent kernel (two wave groups alternate matrix work and everything else).
-struct ConvConfig { unsigned waves, rpw, ck; bool resident; unsigned pw; unsigned maxKT; unsigned mf, xb; const char *name; bool pp = false; };
+// fold: the 2x upsample of source A folded into the weights (conv3x3_upfold.hip; rpw counts low-resolution rows).
+struct ConvConfig { unsigned waves, rpw, ck; bool resident; unsigned pw; unsigned maxKT; unsigned mf, xb; const char *name; bool pp = false; bool fold = false; };
 const ConvConfig kConvConfigs[] = {
     // weights streamed per step
     {4, 2, 16, false, 0, 0, 32, 1, "w4r2k16"}, {4, 2, 32, false, 0, 0, 32, 1, "w4r2k32"}, {4, 4, 16, false, 0, 0, 32, 1, "w4r4k16"}, {4, 4, 32, false, 0, 0, 32, 1, "w4r4k32"},
@@ -75,6 +76,8 @@ const ConvConfig kConvConfigs[] = {
     {16, 1, 16, true, 0, 0, 32, 1, "t16r1k16", true}, {16, 1, 32, true, 0, 0, 32, 1, "t16r1k32", true}, {16, 2, 16, true, 0, 0, 32, 1, "t16r2k16", true},
     {8, 2, 16, true, 0, 0, 32, 1, "t8r2k16", true},   {8, 2, 32, true, 0, 0, 32, 1, "t8r2k32", true},   {8, 4, 16, true, 0, 0, 32, 1, "t8r4k16", true},
     {8, 1, 16, true, 0, 0, 32, 1, "t8r1k16", true},   {8, 2, 32, true, 0, 0, 16, 2, "u8r2k32x2", true}, {16, 1, 32, true, 0, 0, 16, 2, "u16r1k32x2", true},
+    // upsample folded into the weights (layers whose source A is upsampled; one parity class of output pixels per workgroup)
+    {8, 1, 16, true, 0, 0, 32, 1, "f8r1", false, true},  {4, 2, 16, true, 0, 0, 32, 1, "f4r2", false, true}, {4, 1, 16, true, 0, 0, 32, 1, "f4r1", false, true},
 };
 constexpr unsigned kNumConvConfigs = sizeof(kConvConfigs) / sizeof(kConvConfigs[0]);
 
@@ -176,6 +179,73 @@ std::vector<uint8_t> packConvWeights(const Op &conv, const ConvGeometry &g, unsi
   return bytes;
 }
 
+// ---- upsample folded into the weights ------------------------------------------------------------------------
+struct FoldGeometry {
+  unsigned CA, CB, CAP, CBP, K, KOUTP, KT, slots, bpitch;
+  size_t ldsBytes;
+};
+
+bool chooseFold(const ConvConfig &cfg, unsigned CA, unsigned CB, unsigned K, const DeviceInfo &dev, FoldGeometry &g) {
+  if (CA % 8 || (CB > 0 && CB < 8)) return false; // whole vectors of A; B's partial last vector is read ending at its last channel
+  g.CA = CA; g.CB = CB; g.CAP = (CA + 15) / 16 * 16; g.CBP = CB ? (CB + 15) / 16 * 16 : 0; g.K = K; g.KOUTP = (K + 31) / 32 * 32;
+  const unsigned tlh = cfg.waves * cfg.rpw, threads = cfg.waves * 64;
+  const unsigned aPix = (tlh + 1) * 33, bPix = (2 * tlh + 1) * 65, blocks = g.KOUTP / 32;
+  const unsigned regBudget = std::min(256u, 512u / ((cfg.waves + 3) / 4));
+  const unsigned nva = (aPix * (g.CAP / 8) + threads - 1) / threads, nvb = CB ? (bPix * (g.CBP / 8) + threads - 1) / threads : 0;
+  for (unsigned kb = blocks; kb >= 1; --kb) {
+    if (blocks % kb) continue;
+    if (cfg.maxKT && kb * 32 > cfg.maxKT) continue;
+    const unsigned kt = kb * 32;
+    if (kb * cfg.rpw * 24 + (nva + nvb) * 4 + 64 > regBudget) continue; // accumulators, converted tile, halo registers
+    for (unsigned pitchPad : {8u, 0u}) { // the B halo gives up its bank-conflict padding where LDS is short
+      const size_t lds = (static_cast<size_t>(4 * kt) * (g.CAP + 8) + (CB ? static_cast<size_t>(9 * kt) * (g.CBP + 8) : 8) + static_cast<size_t>(aPix) * (g.CAP + 8) +
+                          (CB ? static_cast<size_t>(bPix) * (g.CBP + pitchPad) : 8) + kt) * 2u;
+      if (lds > dev.maxComputeSharedMemory) continue;
+      g.KT = kt; g.bpitch = g.CBP + pitchPad; g.ldsBytes = lds;
+      g.slots = std::max(1u, dev.computeUnits / (dev.xcdCount * 4 * (blocks / kb)));
+      return true;
+    }
+  }
+  return false;
+}
+
+// Folded weights: [class a*2+b][kt][A tap ty*2+tx][KT rows][CAP] [B tap r*3+s][KT rows][CBP].  Tap r of output row
+// parity a reads low-resolution row y + a - 1 + ty with ty = (r + 1) / 2 for a = 0 and r / 2 for a = 1 (columns alike);
+// coinciding taps are summed in fp32 and rounded to binary16 once.
+std::vector<uint8_t> packFoldWeights(const Op &conv, const FoldGeometry &g) {
+  const unsigned nkt = g.KOUTP / g.KT, C = g.CA + g.CB;
+  std::vector<uint16_t> out(static_cast<size_t>(4) * g.KOUTP * (4 * g.CAP + 9 * g.CBP), 0);
+  auto tmap = [](unsigned parity, unsigned tap) { return parity == 0 ? (tap + 1) / 2 : tap / 2; };
+  size_t pos = 0;
+  for (unsigned cls = 0; cls < 4; ++cls) {
+    const unsigned a = cls >> 1, b = cls & 1;
+    for (unsigned kt = 0; kt < nkt; ++kt) {
+      for (unsigned ty = 0; ty < 2; ++ty)
+        for (unsigned tx = 0; tx < 2; ++tx)
+          for (unsigned row = 0; row < g.KT; ++row) {
+            const unsigned k = kt * g.KT + rowChannel(32, g.KT, row);
+            for (unsigned c = 0; c < g.CAP; ++c, ++pos) {
+              if (k >= g.K || c >= g.CA) continue;
+              float sum = 0.0f;
+              for (unsigned r = 0; r < 3; ++r)
+                for (unsigned s2 = 0; s2 < 3; ++s2)
+                  if (tmap(a, r) == ty && tmap(b, s2) == tx) sum += f16_to_f32(conv.weights[((static_cast<size_t>(k) * C + c) * 3 + r) * 3 + s2]);
+              out[pos] = f32_to_f16(sum);
+            }
+          }
+      for (unsigned tap = 0; tap < 9; ++tap)
+        for (unsigned row = 0; row < g.KT; ++row) {
+          const unsigned k = kt * g.KT + rowChannel(32, g.KT, row);
+          for (unsigned c = 0; c < g.CBP; ++c, ++pos)
+            if (k < g.K && c < g.CB) out[pos] = conv.weights[((static_cast<size_t>(k) * C + g.CA + c) * 3 + tap / 3) * 3 + tap % 3];
+        }
+    }
+  }
+  std::vector<uint8_t> bytes(out.size() * 2);
+  std::memcpy(bytes.data(), out.data(), bytes.size());
+  return bytes;
+}
+
 class ConvMfmaShader final : public IShader {
 public:
   explicit ConvMfmaShader(const hip::HipCompiler *c) : m_compiler(c) {}
@@ -270,6 +340,13 @@ public:
       const unsigned kstep = cfg.mf == 32 ? 16 : 32;
       const unsigned cpad = (CA + CB + kstep - 1) / kstep * kstep;
       if (!opt.forceConvConfig.empty() && opt.forceConvConfig != cfg.name) continue;
+      if (cfg.fold) {
+        const unsigned others = PAT_POOL | PAT_CROP | PAT_PADA;
+        FoldGeometry fg;
+        if ((m.pattern & PAT_UPSAMPLE) && !(m.pattern & others) && conv.R == 3 && conv.S == 3 && opt.features.enableUpsampleFold && chooseFold(cfg, CA, CB, conv.K, opt.deviceInfo, fg))
+          out.push_back(c);
+        continue;
+      }
       if (cfg.ck > cpad && cfg.ck != kstep) continue; // a larger stage than the whole reduction adds nothing
       if (cfg.ck <= 1 && cpad <= 32) continue;     // "whole / half reduction" duplicates a fixed-size stage for narrow layers
       if ((m.pattern & PAT_POOL) && (cfg.rpw % 2)) continue;
@@ -279,7 +356,10 @@ public:
       if (!chooseKT(cfg, CA, CB, conv.K, opt.deviceInfo, g)) continue;
       out.push_back(c);
     }
-    if (out.empty() && !opt.forceConvConfig.empty()) fail(Status::Unsupported, "conv configuration '" + opt.forceConvConfig + "' is not valid for this layer");
+    bool forcedFold = false; // a forced upsample-folding configuration leaves matches without an upsample to nobody: not an error
+    for (unsigned c = 0; c < kNumConvConfigs; ++c) forcedFold |= kConvConfigs[c].fold && opt.forceConvConfig == kConvConfigs[c].name;
+    if (out.empty() && !opt.forceConvConfig.empty() && !(forcedFold && !(m.pattern & PAT_UPSAMPLE)))
+      fail(Status::Unsupported, "conv configuration '" + opt.forceConvConfig + "' is not valid for this layer");
     return out;
   }
 
@@ -298,7 +378,11 @@ public:
     const unsigned CB = m.inputs.size() > 1 ? model.tensors()[m.inputs[1]].channels : 0;
     ConvGeometry g;
     g.R = conv.R; g.S = conv.S;
-    if (!chooseKT(cfg, CA, CB, conv.K, opt.deviceInfo, g)) fail(Status::Internal, "conv config rejected at implement time");
+    FoldGeometry fg{};
+    if (cfg.fold) {
+      if (!chooseFold(cfg, CA, CB, conv.K, opt.deviceInfo, fg)) fail(Status::Internal, "conv config rejected at implement time");
+      g.CA = CA; g.CB = CB; g.C = CA + CB; g.K = conv.K; g.KOUTP = fg.KOUTP; g.KT = fg.KT; g.slots = fg.slots; g.CPAD = fg.CAP + fg.CBP;
+    } else if (!chooseKT(cfg, CA, CB, conv.K, opt.deviceInfo, g)) fail(Status::Internal, "conv config rejected at implement time");
     int act = 0;
     float alpha = 0.0f;
     if (m.pattern & PAT_ACT) {
@@ -309,7 +393,8 @@ public:
     const bool pool = (m.pattern & PAT_POOL) != 0, up = (m.pattern & PAT_UPSAMPLE) != 0, crop = (m.pattern & PAT_CROP) != 0;
     const bool padA = (m.pattern & PAT_PADA) != 0, padB = (m.pattern & PAT_PADB) != 0;
 
-    hip::HipCompilerInstance k = m_compiler->read(cfg.resident ? "conv3x3_mfma_ws.hip" : "conv3x3_mfma.hip");
+    hip::HipCompilerInstance k = m_compiler->read(cfg.fold ? "conv3x3_upfold.hip" : cfg.resident ? "conv3x3_mfma_ws.hip" : "conv3x3_mfma.hip");
+    if (cfg.fold) k.define("BPITCH", fg.bpitch ? fg.bpitch : 8);
     k.define("CA", CA); k.define("CB", CB); k.define("UPA", up ? 1 : 0);
     k.define("KOUT", conv.K); k.define("KT", g.KT);
     k.define("ACT", act);
@@ -318,7 +403,7 @@ public:
     if (padA) k.define("PADA", 1);
     if (padB) k.define("PADB", 1);
     if (crop) k.define("CROP", 1);
-    k.define("WAVES", cfg.waves); k.define("RPW", cfg.rpw); k.define("CK", stepChannels(cfg, g.CPAD));
+    k.define("WAVES", cfg.waves); k.define("RPW", cfg.rpw); k.define("CK", cfg.fold ? 16u : stepChannels(cfg, g.CPAD));
     if (cfg.resident) k.define("SLOTS", g.slots);
     if (cfg.pw) k.define("PW", cfg.pw);
     if (cfg.pp) k.define("PP", 1);
@@ -330,15 +415,18 @@ public:
     const Sym W = convIn.width, H = convIn.height;
     const unsigned th = cfg.waves * cfg.rpw;
     const unsigned nkt = g.KOUTP / g.KT;
-    auto d = cfg.resident ? impl.registerDispatch(k, entry, Sym::Const(opt.deviceInfo.xcdCount * nkt * g.slots), Sym::Const(1), Sym::Const(1), (cfg.waves + cfg.pw) * 64)
+    auto d = cfg.fold ? impl.registerDispatch(k, entry, Sym::Const(opt.deviceInfo.xcdCount * 4 * nkt * g.slots), Sym::Const(1), Sym::Const(1), cfg.waves * 64)
+           : cfg.resident ? impl.registerDispatch(k, entry, Sym::Const(opt.deviceInfo.xcdCount * nkt * g.slots), Sym::Const(1), Sym::Const(1), (cfg.waves + cfg.pw) * 64)
                           : impl.registerDispatch(k, entry, sym.cdiv(W, cfg.mf == 32 ? 32 : 16 * cfg.xb), sym.cdiv(H, th), Sym::Const(nkt), cfg.waves * 64);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     if (CB) d.addBinding(dnx::Access::ReadOnly, m.inputs[1]);
     d.addBinding(dnx::Access::WriteOnly, m.output);
     const Op convCopy = conv; // the lazy packers outlive the model reference
     const unsigned ck = cfg.resident ? g.CPAD : stepChannels(cfg, g.CPAD);
-    TensorId wt = impl.createParameter(static_cast<size_t>(g.KOUTP) * conv.R * conv.S * g.CPAD * 2, dnx::ScalarType::F16,
-                                       [convCopy, g, ck, mf = cfg.mf]() { return packConvWeights(convCopy, g, ck, mf); });
+    TensorId wt = cfg.fold ? impl.createParameter(static_cast<size_t>(4) * fg.KOUTP * (4 * fg.CAP + 9 * fg.CBP) * 2, dnx::ScalarType::F16,
+                                                  [convCopy, fg]() { return packFoldWeights(convCopy, fg); })
+                           : impl.createParameter(static_cast<size_t>(g.KOUTP) * conv.R * conv.S * g.CPAD * 2, dnx::ScalarType::F16,
+                                                  [convCopy, g, ck, mf = cfg.mf]() { return packConvWeights(convCopy, g, ck, mf); });
     d.addParamBinding(wt);
     if (conv.hasBias) {
       const unsigned koutp = g.KOUTP;

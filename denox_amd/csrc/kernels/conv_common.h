@@ -531,10 +531,11 @@ __device__ DNX_INLINE void pack_tile(const Acc &acc, Packed &pk, const _Float16 
 // Stores the output rows r with r % nparts == part (all of them with nparts = 1).  All channels of a pixel go out
 // together: a 128-byte line that is filled in two portions far apart in time is written to memory twice.
 __device__ DNX_INLINE void
-store_packed(const Packed &pk, OutBuf out, int y0, int x0, int kt, int wv, int lane, const PushConstants &pc, int part = 0, int nparts = 1) {
+store_packed(const Packed &pk, OutBuf out, int y0, int x0, int kt, int wv, int lane, const PushConstants &pc, int part = 0, int nparts = 1,
+             int ystep = 1, int xstep = 1) { // (steps of 2: a kernel that computes every other row / column of the output)
   const unsigned W = pc.IN_W, H = pc.IN_H;
   const int l32 = lane & 31;
-  const int x = x0 + l32;
+  const int x = x0 + l32 * xstep;
 #pragma unroll
   for (int kb = 0; kb < KB; ++kb) {
     const int chb = kt * KT + kb * 32 + (lane >> 5) * 16; // first of this lane's 16 channels
@@ -547,7 +548,7 @@ store_packed(const Packed &pk, OutBuf out, int y0, int x0, int kt, int wv, int l
       const unsigned py = (unsigned)(y0 + wv * RPW + 2 * r) >> 1, px = (unsigned)x >> 1;
       store16(out, (l32 & 1) == 0 && py < HP && px < WP, py * WP + px, pk.o[kb][r], chb);
 #else
-      const int y = y0 + wv * RPW + r;
+      const int y = y0 + (wv * RPW + r) * ystep;
 #if CROP
       const int oy = y - (int)pc.CROP_T, ox = x - (int)pc.CROP_L;
       store16(out, y < (int)H && x < (int)W && oy >= 0 && oy < (int)pc.OUT_H && ox >= 0 && ox < (int)pc.OUT_W,

@@ -11,7 +11,7 @@ from util import assert_conv_close, he_weights, small_bias
 pytestmark = pytest.mark.gpu
 
 CONFIGS = [None, None, None, "w4r2k16", "w4r1k32", "w8r2k32", "w2r2kfn", "w4r1kfm", "p8r1k16", "p16r1k16", "p8r2k32", "p4r4k16", "p4r2k32n",
-           "s8r2k16", "m4r2k32x2", "m4r1kfx2", "m4r2kfx1n", "q8r2k32x2", "q4r2k32x1n", "t16r1k16", "t8r2k16", "u8r2k32x2"]
+           "s8r2k16", "m4r2k32x2", "m4r1kfx2", "m4r2kfx1n", "q8r2k32x2", "q4r2k32x1n", "t16r1k16", "t8r2k16", "u8r2k32x2", "f8r1", "f4r2", "f4r1"]
 CHANNELS = [1, 2, 3, 7, 8, 9, 15, 16, 17, 24, 31, 32, 33, 40, 48, 64, 73, 80]
 
 

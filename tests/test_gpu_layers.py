@@ -136,6 +136,39 @@ def test_odd_filter_extents(oracle, R, S, config):
     assert_conv_close(got2, env[o2.name], f"{R}x{S} bare {config}")
 
 
+@pytest.mark.parametrize("config", ["f8r1", "f4r2", "f4r1"])
+@pytest.mark.parametrize("CA,CB,K,H,W,padb", [(64, 9, 64, 36, 70, False), (16, 0, 32, 18, 34, False), (32, 24, 40, 62, 130, False),
+                                              (8, 3, 3, 2, 2, False), (24, 9, 16, 40, 52, True), (96, 32, 64, 34, 66, False)])
+def test_upsample_folded_into_weights(oracle, config, CA, CB, K, H, W, padb):
+    """conv(concat(upsample(A), B)) with the upsample folded into 2x2-tap weights per output parity: the same tensor
+    as the layer-by-layer evaluation, within the conv tolerance (the summed weights are rounded to binary16 once)."""
+    rng = np.random.default_rng(CA + CB + K)
+    w, b = he_weights(rng, K, CA + CB), small_bias(rng, K)
+    m = dx.Model()
+    lo = rng.standard_normal((H // 2, W // 2, CA)).astype(np.float16)
+    feeds = {"lo": lo}
+    t = m.upsample(m.input("lo", m.sym("W") // 2, m.sym("H") // 2, CA))
+    if CB:
+        if padb:  # the skip source is stored 3 rows / 5 columns short and replicate-padded
+            x = rng.standard_normal((H - 3, W - 5, CB)).astype(np.float16)
+            t = m.concat(t, m.pad(m.input("x", m.sym("W") - 5, m.sym("H") - 3, CB), 2, 3, 1, 2))
+        else:
+            x = rng.standard_normal((H, W, CB)).astype(np.float16)
+            t = m.concat(t, m.input("x", "W", "H", CB))
+        feeds["x"] = x
+    t = m.activation(m.conv2d(t, w, b), "leaky_relu", 0.25)
+    m.output(t)
+    try:
+        mod = dx.Module.compile(m, conv_config=config)
+    except dx.DenoxHipError as e:
+        assert e.status == 5
+        pytest.skip(str(e))
+    assert config in dx.last_compile_report() and mod.runtime_model.dispatch_count == 1
+    got = mod.instance(H=H, W=W).infer(*[feeds[k] for k in ("lo", "x") if k in feeds])[0]
+    want = oracle.run_graph(m.to_ops({"H": H, "W": W}), feeds, "fp32")[t.name]
+    assert_conv_close(got, want, f"fold {config}")
+
+
 def test_tensor_size_limit_is_reported():
     """Tensors are addressed with 32-bit byte offsets: extents that make one reach 4 GiB are refused when the
     instance is created, before anything is allocated."""
