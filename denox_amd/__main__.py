@@ -99,8 +99,8 @@ def cmd_populate(args):
 
 def cmd_bench(args):
     with open(args.target, "rb") as f:
-        head = f.read(4)
-    if head == b"DNXH":  # a compiled model: per-dispatch report (Instance::bench().report() of the reference)
+        head = f.read(8)
+    if head[4:8] == b"dnxx":  # a compiled model (file identifier of dnx.fbs): per-dispatch report (Instance::bench().report() of the reference)
         with open(args.target, "rb") as f:
             mod = Module.load(f.read())
         spec = {k: int(v) for k, v in _pairs(args.spec, "--spec").items()}

@@ -293,7 +293,10 @@ static void jsonEscape(std::ostringstream &o, const std::string &s) {
   for (char c : s) {
     if (c == '"' || c == '\\') o << '\\' << c;
     else if (static_cast<unsigned char>(c) < 0x20) o << ' ';
-    else o << c;
+    else if (static_cast<unsigned char>(c) >= 0x80) { // names are ASCII; a damaged file must still yield valid JSON
+      static const char *hex = "0123456789abcdef";
+      o << "\\u00" << hex[(static_cast<unsigned char>(c) >> 4) & 15] << hex[c & 15];
+    } else o << c;
   }
   o << '"';
 }

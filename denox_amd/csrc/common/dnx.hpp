@@ -1,16 +1,15 @@
 // In-memory form and byte serialisation of a compiled model ("dnx").
 //
-// Mirrors the reference schema dnx.fbs:1-195 table by table -- Model{tensors,
-// initializers, inputs, outputs, buffers, dispatches, shader_binaries, sym_ir,
-// value_names}, ComputeDispatch{binary_id, workgroup_count_{x,y,z}, entry_point,
-// bindings, push_constant, info} -- with the two changes a HIP backend needs:
-//   * ShaderBinary carries a gfx950 code object (bytes) instead of SPIR-V words
+// The bytes are a FlatBuffer of the reference's schema dnx.fbs:1-195 (file identifier "dnxx", root table Model), written
+// and read by hand over common/flatbuf.hpp: field ids are the declaration order of each table, a union takes two ids
+// (member index, then the member).  A HIP backend needs two things the schema does not hold, and both are added the way
+// FlatBuffers schemas evolve -- new fields at the end of a table, which a reader generated from the original schema skips:
+//   * ShaderBinary.code_object:[ubyte] (id 1, after spirv): a gfx950 code object instead of SPIR-V words
 //     (dnx.fbs:169-171);
-//   * ComputeDispatch gains the workgroup size, which SPIR-V bakes into the
-//     module as local_size but a HIP launch takes as an argument.
-// FlatBuffers (flatc and its headers) are not available, so the bytes on the
-// wire are a plain little-endian tagged stream with a bounds-checked reader;
-// the field set, not the byte layout, is what matches the reference.
+//   * ComputeDispatch.workgroup_size_{x,y,z}:uint (ids 11-13, after info): SPIR-V bakes the workgroup size into the
+//     module as local_size, a HIP launch takes it as an argument;
+//   * RuntimeFeature gains HipCodeObject = 1 (dnx.fbs:160-162), listed in required_features of every model written here.
+// A model written by the reference (SPIR-V only) parses and can be described; running it reports UNSUPPORTED.
 #pragma once
 #include "error.hpp"
 #include "sym.hpp"
@@ -77,11 +76,12 @@ struct TensorInfo {
 struct Tensor { uint32_t buffer = 0; ScalarSource offset, size; TensorInfo info; };
 struct TensorInitializer { uint32_t tensor; std::vector<uint8_t> data; };
 struct ValueName { std::string name; ScalarSource value; };
-struct ShaderBinary { std::vector<uint8_t> code_object; };
+struct ShaderBinary { std::vector<uint8_t> code_object; uint32_t spirv_words = 0; };
 struct ModelInfo { std::string producer, producer_version, model_version; };
 
 struct Model {
   uint16_t version = 0;
+  std::vector<uint32_t> required_features; // RuntimeFeature: 0 CooperativeMatrix (reference), 1 HipCodeObject
   ModelInfo info;
   std::vector<Tensor> tensors;
   std::vector<TensorInitializer> initializers;
@@ -94,10 +94,13 @@ struct Model {
 };
 
 std::vector<uint8_t> serialize(const Model &m);
-// Throws Error(InvalidModel) on a truncated, corrupt or inconsistent stream
+// Throws Error(InvalidModel) on a truncated, corrupt or inconsistent buffer
 // (the role of the FlatBuffers verifier in runtime/src/denox/runtime/model.cpp:639-644).
 Model deserialize(const void *data, size_t size);
 // Index / reference consistency checks shared by the reader and the compiler.
 void validate(const Model &m);
+// What a model needs on top of `validate` before it can be launched: a code object behind every binary a dispatch names
+// and a workgroup size of 1..1024 threads.  Error(Unsupported) for a model that holds SPIR-V only.
+void requireExecutable(const Model &m);
 
 } // namespace denox::dnx

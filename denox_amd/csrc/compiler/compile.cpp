@@ -341,7 +341,9 @@ std::vector<uint8_t> compile(const Model &modelIn, const hip::HipCompiler &hipc,
 
   out.sym_ir = sym.compile();
   for (const auto &nv : model.valueNames()) out.value_names.push_back(dnx::ValueName{nv.name, src(nv.value)});
+  out.required_features = {1u}; // HipCodeObject: the binaries are gfx950 code objects, not SPIR-V
   dnx::validate(out);
+  dnx::requireExecutable(out);
   if (report) {
     report->superGraphEdges = g.edges.size();
     report->selectedEdges = chosen.size();

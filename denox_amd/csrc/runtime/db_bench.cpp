@@ -1,5 +1,6 @@
 #include "db_bench.hpp"
 #include <algorithm>
+#include <chrono>
 #include <cstring>
 #include <sstream>
 #include <vector>
@@ -20,6 +21,7 @@ DbBenchResult db_bench(Db &db, const ContextHandle &ctx, const hip::HipCompiler 
   void *scratch = nullptr;
   uint64_t scratchBytes = 0;
   size_t sinceWriteback = 0;
+  bool envRecorded = false;
   auto cleanup = [&]() {
     if (scratch) (void)hipFree(scratch);
     (void)hipEventDestroy(e0);
@@ -30,6 +32,22 @@ DbBenchResult db_bench(Db &db, const ContextHandle &ctx, const hip::HipCompiler 
       DbDispatch &row = db.rows()[r];
       if (!opt.filter.empty() && row.shader.find(opt.filter) == std::string::npos && row.operation.find(opt.filter) == std::string::npos) { ++res.skipped; continue; }
       if (converged(row, opt)) { ++res.skipped; continue; }
+      if (!envRecorded) { // one BenchEnv per session that measures anything (runtime/src/denox/runtime/db.cpp:694-698 of the reference)
+        hipDeviceProp_t prop;
+        hipCheck(hipGetDeviceProperties(&prop, ctx->device()), "hipGetDeviceProperties");
+        int driver = 0;
+        (void)hipDriverGetVersion(&driver);
+        DbEnv env;
+        env.device = std::string(prop.name) + " (" + prop.gcnArchName + ")";
+        env.os = "Linux";
+        env.driverVersion = "HIP " + std::to_string(driver);
+        env.version = "denox-hip 0.1";
+        env.startTimestamp = static_cast<uint64_t>(std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::system_clock::now().time_since_epoch()).count());
+        env.jitWarmupIterations = static_cast<uint16_t>(std::min<uint32_t>(opt.warmup, 0xFFFF));
+        env.measurementIterations = static_cast<uint16_t>(std::min<uint32_t>(opt.batch, 0xFFFF));
+        db.create_bench_environment(std::move(env));
+        envRecorded = true;
+      }
       // rebuild the kernel variant from its source path and definitions
       hip::HipCompilerInstance k = hipc.read(row.srcPath);
       std::stringstream ss(row.defines);

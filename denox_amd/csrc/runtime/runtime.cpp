@@ -28,11 +28,12 @@ void Context::makeCurrent() const { hipCheck(hipSetDevice(m_device), "hipSetDevi
 
 // ---------------------------------------------------------------- Model
 Model::Model(ContextHandle ctx, const void *dnxbuf, size_t size) : m_ctx(std::move(ctx)), m_dnx(dnx::deserialize(dnxbuf, size)) {
+  dnx::requireExecutable(m_dnx);
   m_ctx->makeCurrent();
   m_modules.resize(m_dnx.shader_binaries.size(), nullptr);
   try {
     for (size_t i = 0; i < m_modules.size(); ++i) {
-      if (m_dnx.shader_binaries[i].code_object.empty()) fail(Status::InvalidModel, "empty shader binary");
+      if (m_dnx.shader_binaries[i].code_object.empty()) continue; // a binary no dispatch names
       hipCheck(hipModuleLoadData(&m_modules[i], m_dnx.shader_binaries[i].code_object.data()), "hipModuleLoadData");
     }
     m_dispatches.reserve(m_dnx.dispatches.size());

@@ -176,3 +176,21 @@ def test_full_size_oidn_unet_centre_of_crop(oracle):
         ys = slice(0 if y0 == 0 else Mg, h if y0 + h >= FULL_H else h - Mg)
         xs = slice(0 if x0 == 0 else Mg, S if x0 + S >= FULL_W else S - Mg)
         assert_conv_close(got[y0:y0 + h, x0:x0 + S][ys, xs], want[ys, xs], f"crop at {(y0, x0)}")
+
+
+def test_model_file_round_trip_and_a_model_compiled_for_vulkan(tmp_path):
+    # the bytes on disk are the whole model: save, load in a fresh Module, same bits out
+    m, _ = networks.build("tiny_unet", seed=5)
+    x = networks.synthetic_input("tiny_unet", 32, 48, seed=5)
+    mod = dx.Module.compile(m)
+    want = mod.instance(H=32, W=48).infer(x)[0]
+    path = tmp_path / "tiny.dnx"
+    mod.save(str(path))
+    blob = path.read_bytes()
+    assert blob[4:8] == b"dnxx"
+    assert_bits_equal(dx.Module.load(blob).instance(H=32, W=48).infer(x)[0], want, "reloaded model")
+    # the same model with its binaries stored the way the reference stores SPIR-V: described, but refused by the runtime
+    from test_flatbuf import as_written_for_vulkan
+    with pytest.raises(dx.DenoxHipError) as e:
+        dx.Module.load(as_written_for_vulkan(blob)).instance(H=32, W=48)
+    assert e.value.status == 5 and "SPIR-V" in str(e.value)
