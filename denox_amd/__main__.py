@@ -59,7 +59,7 @@ def _layouts(args, model):
 
 def _features(args):
     if getattr(args, "no_fusion", False):
-        return {k: False for k in ("conv_relu_fusion", "concat_conv_fusion", "upsample_fusion", "pool_fusion", "pad_fusion", "slice_fusion")}
+        return {k: False for k in ("conv_relu_fusion", "concat_conv_fusion", "upsample_fusion", "pool_fusion", "pad_fusion", "slice_fusion", "implicit_concat")}
     return {}
 
 

@@ -143,12 +143,21 @@ std::vector<size_t> minimum_cost_subgraph(const std::vector<bool> &isInput, cons
 }
 
 std::vector<size_t> select_schedule(const Model &model, const SuperGraph &g, const std::vector<double> &edgeCost) {
-  std::vector<bool> isInput(model.tensors().size());
-  for (size_t i = 0; i < isInput.size(); ++i) isInput[i] = model.tensors()[i].isInput;
+  // node 2 t: tensor t in a buffer of its own; node 2 t + 1: tensor t as a channel range of its concat's output
+  // (SuperGraphEdge::outputVariant).  Tensor handles are topologically ordered, and so are these.
+  std::vector<bool> isInput(2 * model.tensors().size(), false);
+  for (size_t i = 0; i < model.tensors().size(); ++i) isInput[2 * i] = model.tensors()[i].isInput;
   std::vector<HyperEdge> edges;
-  for (const auto &e : g.edges) edges.push_back(HyperEdge{e.inputs, e.output});
+  for (const auto &e : g.edges) {
+    HyperEdge h;
+    for (size_t i = 0; i < e.inputs.size(); ++i) h.inputs.push_back(2 * e.inputs[i] + (e.inputVariants.empty() ? 0 : e.inputVariants[i]));
+    h.output = 2 * e.output + e.outputVariant;
+    edges.push_back(std::move(h));
+  }
+  std::vector<int> outputs;
+  for (TensorHandle o : model.outputs()) outputs.push_back(2 * o);
   double total = 0.0;
-  std::vector<size_t> chosen = minimum_cost_subgraph(isInput, edges, edgeCost, model.outputs(), &total);
+  std::vector<size_t> chosen = minimum_cost_subgraph(isInput, edges, edgeCost, outputs, &total);
   if (total >= kInfiniteCost) fail(Status::Unsupported, "no kernel implements part of this graph (a layer has no matching shader)");
   return chosen;
 }
@@ -282,8 +291,8 @@ std::vector<uint8_t> compile(const Model &modelIn, const hip::HipCompiler &hipc,
     d.workgroupCountX = sym.cdiv(sym.mul(sym.mul(n.width, n.height), blocky ? static_cast<int64_t>(n.channels / 8) : 1), 256);
     d.workgroupCountY = d.workgroupCountZ = Sym::Const(1);
     d.workgroupSize[0] = 256;
-    TensorBinding in{0, 0, dnx::Access::ReadOnly, TensorId{external_is_source ? extId : static_cast<uint32_t>(t)}, BindingType::Input};
-    TensorBinding ob{0, 1, dnx::Access::WriteOnly, TensorId{external_is_source ? static_cast<uint32_t>(t) : extId}, BindingType::Output};
+    TensorBinding in{0, 0, dnx::Access::ReadOnly, TensorId{external_is_source ? extId : static_cast<uint32_t>(t)}, BindingType::Input, false, Sym::Const(0)};
+    TensorBinding ob{0, 1, dnx::Access::WriteOnly, TensorId{external_is_source ? static_cast<uint32_t>(t) : extId}, BindingType::Output, false, Sym::Const(0)};
     d.bindings = {in, ob};
     d.pushConstants = {PushConstantDesc{n.width, dnx::ScalarType::U32}, PushConstantDesc{n.height, dnx::ScalarType::U32}};
     d.info.name = "relayout"; d.info.operation = "relayout"; d.info.srcPath = "relayout.hip";
@@ -325,6 +334,14 @@ std::vector<uint8_t> compile(const Model &modelIn, const hip::HipCompiler &hipc,
       out.tensors[a].offset = src(Sym::Const(0));
       out.tensors[b].offset = out.tensors[a].size;
     }
+    // pixel-major concat without a copy: the source is a channel range of the destination, from its first channel
+    // to the end of the destination
+    for (const auto &vc : edge.viewConstrains) {
+      const uint32_t a = place(vc.src.index), dd = place(vc.dst.index);
+      out.tensors[a].buffer = out.tensors[dd].buffer;
+      out.tensors[a].offset = src(Sym::Const(static_cast<int64_t>(vc.byteOffset)));
+      out.tensors[a].size = src(sym.sub(g.tensors[vc.dst.index].byteSize, static_cast<int64_t>(vc.byteOffset)));
+    }
     total += cost[e];
     if (report) {
       report->schedule.push_back(ScheduleEntry{edge.shader, edge.config, edge.dispatches.empty() ? "" : edge.dispatches[0].info.name, cost[e], measured[e]});
@@ -337,6 +354,16 @@ std::vector<uint8_t> compile(const Model &modelIn, const hip::HipCompiler &hipc,
     const dnx::TensorFormat f = formatOf(opt.outputDescriptors, model.tensors()[t].name, i);
     if (f == dnx::TensorFormat::SSBO_HWC) out.outputs.push_back(place(static_cast<uint32_t>(t)));
     else out.outputs.push_back(relayout(t, dnx::TensorFormat::SSBO_HWC, f, false));
+  }
+
+  { // buffers whose tensor moved into another buffer are dropped
+    std::vector<int> newIndex(out.buffers.size(), -1);
+    std::vector<dnx::Buffer> kept;
+    for (auto &t : out.tensors) {
+      if (newIndex[t.buffer] < 0) { newIndex[t.buffer] = static_cast<int>(kept.size()); kept.push_back(out.buffers[t.buffer]); }
+      t.buffer = static_cast<uint32_t>(newIndex[t.buffer]);
+    }
+    out.buffers = std::move(kept);
   }
 
   out.sym_ir = sym.compile();
@@ -376,7 +403,7 @@ size_t populate(Db &db, const Model &modelIn, const hip::HipCompiler &hipc, cons
       for (int i = 0; i < 3; ++i) row.block[i] = d.workgroupSize[i];
       for (const auto &b : d.bindings) {
         const SuperTensor &t = g.tensors[b.tensor.index];
-        row.bindings.push_back(DbBinding{static_cast<uint64_t>(symValue(dp, t.byteSize)), t.alignment, t.isParam, static_cast<uint8_t>(b.access)});
+        row.bindings.push_back(DbBinding{static_cast<uint64_t>(symValue(dp, b.hasSpan ? b.span : t.byteSize)), t.alignment, t.isParam, static_cast<uint8_t>(b.access)});
       }
       row.operation = d.info.operation; row.shader = edge.shader; row.config = d.info.config;
       row.memoryReads = d.info.hasReads ? static_cast<uint64_t>(symValue(dp, d.info.memoryReads)) : 0;

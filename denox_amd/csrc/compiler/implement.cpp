@@ -18,6 +18,12 @@ void ComputeDispatchBuilder::addBinding(dnx::Access access, TensorHandle t) {
   self().bindings.push_back(b);
 }
 
+void ComputeDispatchBuilder::addBinding(dnx::Access access, TensorHandle t, Sym span) {
+  addBinding(access, t);
+  self().bindings.back().hasSpan = true;
+  self().bindings.back().span = span;
+}
+
 void ComputeDispatchBuilder::addParamBinding(TensorId tensor) {
   TensorBinding b;
   b.access = dnx::Access::ReadOnly;
@@ -75,6 +81,26 @@ void OpImpl::createImplicitConcatConstrain(TensorHandle src0, TensorHandle src1,
   m_edge.memoryConstrains.push_back(MemoryConstrain{TensorId{static_cast<uint32_t>(src0)}, TensorId{static_cast<uint32_t>(src1)}, TensorId{static_cast<uint32_t>(dst)}});
 }
 
+void OpImpl::createViewConstrain(TensorHandle src, TensorHandle dst, uint64_t byteOffset) {
+  const size_t n = m_model->tensors().size();
+  if (src < 0 || dst < 0 || static_cast<size_t>(src) >= n || static_cast<size_t>(dst) >= n) fail(Status::Internal, "Failed to create memory constrain, invalid node ids.");
+  m_edge.viewConstrains.push_back(ViewConstrain{TensorId{static_cast<uint32_t>(src)}, TensorId{static_cast<uint32_t>(dst)}, byteOffset});
+}
+
+ConcatView concatViewOf(const Model &model, TensorHandle t) {
+  ConcatView v;
+  const TensorNode &n = model.tensors()[static_cast<size_t>(t)];
+  if (n.isInput || n.isOutput || n.consumers.size() != 1) return v;
+  const Op &cat = model.ops()[static_cast<size_t>(n.consumers[0])];
+  if (cat.kind != OpKind::Concat || cat.inputs.size() != 2 || cat.inputs[0] == cat.inputs[1]) return v;
+  v.valid = true;
+  v.concatOp = n.consumers[0];
+  v.parent = cat.output;
+  v.pitch = model.tensors()[static_cast<size_t>(cat.output)].channels;
+  v.channelOffset = cat.inputs[0] == t ? 0 : model.tensors()[static_cast<size_t>(cat.inputs[0])].channels;
+  return v;
+}
+
 void OpImpl::finish() { m_graph->edges.push_back(std::move(m_edge)); }
 
 SuperGraph implement(const Model &model, SymGraph &sym, const std::vector<std::unique_ptr<IShader>> &shaders, const CompileOptions &opt) {
@@ -95,6 +121,8 @@ SuperGraph implement(const Model &model, SymGraph &sym, const std::vector<std::u
         OpImpl impl(&g, &model, m.inputs, m.output, m.ops);
         impl.edge().shader = shader->name();
         impl.edge().speedup = shader->speedup(config);
+        impl.edge().outputVariant = m.outputVariant;
+        impl.edge().inputVariants = m.inputVariants;
         shader->implement(impl, model, m, config, sym, opt);
         impl.finish();
       }

@@ -35,6 +35,10 @@ struct TensorBinding {
   dnx::Access access;
   TensorId tensor;
   BindingType type;
+  // bytes the kernel may touch from the bound address, when that is not the tensor's own size (a channel range
+  // written with the pixel pitch of a wider tensor); the timing table sizes its scratch buffers with it
+  bool hasSpan = false;
+  Sym span;
 };
 
 struct ComputeDispatchInfo {
@@ -69,6 +73,19 @@ struct SuperTensor {
 
 struct Parameter { TensorId tensor; std::function<std::vector<uint8_t>()> lazyValue; };
 struct MemoryConstrain { TensorId src0, src1, dst; };
+// `src` lives inside `dst`, `byteOffset` from its start, with dst's pixel pitch (pixel-major concat without a copy)
+struct ViewConstrain { TensorId src, dst; uint64_t byteOffset; };
+
+// A tensor that may be produced directly as a channel range of a concat's output: its only consumer is that concat,
+// it is neither a model input nor output, and the concat's result is an ordinary tensor.  The reference restricts its
+// implicit concat the same way (each source feeds exactly one concat, CopyTransformShader.cpp:198-237).
+struct ConcatView {
+  bool valid = false;
+  int concatOp = -1;
+  TensorHandle parent = -1;
+  unsigned pitch = 0, channelOffset = 0;
+};
+ConcatView concatViewOf(const Model &model, TensorHandle t);
 
 struct SuperGraphEdge {
   std::vector<int> inputs; // model tensor handles
@@ -77,6 +94,11 @@ struct SuperGraphEdge {
   std::vector<ComputeDispatch> dispatches;
   std::vector<Parameter> parameters;
   std::vector<MemoryConstrain> memoryConstrains;
+  std::vector<ViewConstrain> viewConstrains;
+  // 0: the tensor as a buffer of its own; 1: the tensor as a channel range of its concat's output (ConcatView).
+  // The two are different nodes of the hyper-graph the schedule is selected from.
+  int outputVariant = 0;
+  std::vector<int> inputVariants; // one per input, empty = all 0
   std::string shader, config;
   float speedup = 1.0f;
 };
@@ -91,6 +113,7 @@ class OpImpl;
 class ComputeDispatchBuilder {
 public:
   void addBinding(dnx::Access access, TensorHandle modelTensor);
+  void addBinding(dnx::Access access, TensorHandle modelTensor, Sym span); // see TensorBinding::span
   void addParamBinding(TensorId tensor);
   void addPushConstant(Sym value, dnx::ScalarType dtype = dnx::ScalarType::U32);
   void addTraversalFlag(); // a U32 push constant, 0 here, set per position in the schedule
@@ -123,6 +146,7 @@ public:
                                           Sym wgX, Sym wgY, Sym wgZ, uint32_t blockX, uint32_t blockY = 1, uint32_t blockZ = 1);
   TensorId createParameter(size_t byteSize, dnx::ScalarType dtype, std::function<std::vector<uint8_t>()> value, uint16_t alignment = 256);
   void createImplicitConcatConstrain(TensorHandle src0, TensorHandle src1, TensorHandle dst);
+  void createViewConstrain(TensorHandle src, TensorHandle dst, uint64_t byteOffset);
   SuperGraphEdge &edge() { return m_edge; }
   void finish();
 
@@ -138,6 +162,8 @@ struct Match {
   std::vector<int> ops;      // covered op indices, in execution order
   std::vector<int> inputs;   // tensor handles read
   int output = -1;           // tensor handle written
+  int outputVariant = 0;     // as SuperGraphEdge::outputVariant
+  std::vector<int> inputVariants;
 };
 
 class IShader {

@@ -319,6 +319,12 @@ public:
           m.ops.insert(m.ops.end(), e.ops.begin(), e.ops.end());
           m.inputs = p.inputs;
           m.output = e.output;
+          // the same dispatch writing straight into the channel range of the concat that consumes its output
+          if (opt.features.enableImplicitConcat && concatViewOf(model, m.output).valid) {
+            Match v = m;
+            v.outputVariant = 1;
+            out.push_back(std::move(v));
+          }
           out.push_back(std::move(m));
         }
     }
@@ -409,8 +415,13 @@ public:
     if (cfg.pp) k.define("PP", 1);
     if (conv.R != 3 || conv.S != 3) { k.define("KR", conv.R); k.define("KS", conv.S); }
     if (cfg.mf != 32) { k.define("MF", cfg.mf); k.define("XB", cfg.xb); }
+    const ConcatView view = m.outputVariant ? concatViewOf(model, m.output) : ConcatView{};
+    if (m.outputVariant && !view.valid) fail(Status::Internal, "conv match writes into a concat that does not exist");
+    const bool ovec = view.valid && view.pitch % 8 == 0 && view.channelOffset % 8 == 0;
+    if (view.valid) { k.define("OPITCH", view.pitch); k.define("OVEC", ovec ? 1 : 0); }
     std::string entry = "conv" + std::to_string(conv.R) + "x" + std::to_string(conv.S) + "_c" + std::to_string(CA) + (up ? "u" : "") + (padA ? "e" : "") + (CB ? "p" + std::to_string(CB) + (padB ? "e" : "") : "") + "_k" +
-                        std::to_string(conv.K) + (act == 1 ? "_relu" : act == 2 ? "_lrelu" : "") + (pool ? "_pool" : "") + (crop ? "_crop" : "") + "_" + cfg.name;
+                        std::to_string(conv.K) + (act == 1 ? "_relu" : act == 2 ? "_lrelu" : "") + (pool ? "_pool" : "") + (crop ? "_crop" : "") +
+                        (view.valid ? "_into" + std::to_string(view.pitch) + (ovec ? "" : "e") : "") + "_" + cfg.name;
     k.define("KERNEL_NAME", entry);
     const Sym W = convIn.width, H = convIn.height;
     const unsigned th = cfg.waves * cfg.rpw;
@@ -420,7 +431,12 @@ public:
                           : impl.registerDispatch(k, entry, sym.cdiv(W, cfg.mf == 32 ? 32 : 16 * cfg.xb), sym.cdiv(H, th), Sym::Const(nkt), cfg.waves * 64);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     if (CB) d.addBinding(dnx::Access::ReadOnly, m.inputs[1]);
-    d.addBinding(dnx::Access::WriteOnly, m.output);
+    if (view.valid) {
+      // from the range's first channel to the end of its last pixel: (pixels - 1) * pitch + K channels
+      const TensorNode &o = model.tensors()[m.output];
+      const Sym pixels = sym.mul(o.width, o.height);
+      d.addBinding(dnx::Access::WriteOnly, m.output, sym.sub(sym.mul(pixels, static_cast<int64_t>(view.pitch) * 2), static_cast<int64_t>(view.pitch - conv.K) * 2));
+    } else d.addBinding(dnx::Access::WriteOnly, m.output);
     const Op convCopy = conv; // the lazy packers outlive the model reference
     const unsigned ck = cfg.resident ? g.CPAD : stepChannels(cfg, g.CPAD);
     TensorId wt = cfg.fold ? impl.createParameter(static_cast<size_t>(4) * fg.KOUTP * (4 * fg.CAP + 9 * fg.CBP) * 2, dnx::ScalarType::F16,
@@ -459,6 +475,7 @@ public:
     if (act == 1) nm += "+relu"; else if (act == 2) nm += "+leaky_relu";
     if (pool) nm += "+maxpool";
     if (crop) nm += "+slice";
+    if (view.valid) nm += "+concat";
     d.setName(nm);
     d.setOperation(nm);
     d.setConfig(std::string(cfg.name) + "/kt" + std::to_string(g.KT));
@@ -555,14 +572,38 @@ public:
   explicit CopyTransformShader(const hip::HipCompiler *c) : SingleOpShader(c, OpKind::Concat) {}
   std::string name() const override { return "copy_transform"; }
   // Explicit concat: one strided channel copy per source (CopyTransformShader.cpp:437-537).
-  // The reference's zero-dispatch implicit concat needs channel-block-major
-  // tensors (CHWC8, CopyTransformShader.cpp:198-237); activations here are
-  // pixel-major HWC, where the sources interleave per pixel and cannot alias.
+  // Implicit concat: the reference aliases two channel-block-major (CHWC8) sources behind one another and needs no
+  // dispatch (CopyTransformShader.cpp:198-237, OpImpl.cpp:43-65).  Activations here are pixel-major, where the
+  // sources interleave per pixel; the same saving comes from the producer side instead: a source whose only
+  // consumer is this concat may be written by its producer straight into its channel range of the output (variant 1
+  // of the tensor, ConcatView), and the concat then copies only the sources that were not -- none, in the best case.
+  std::vector<Match> matchAll(const Model &model, const CompileOptions &opt) const override {
+    std::vector<Match> out;
+    for (const Match &m : SingleOpShader::matchAll(model, opt)) {
+      out.push_back(m);
+      if (!opt.features.enableImplicitConcat) continue;
+      const bool v0 = concatViewOf(model, m.inputs[0]).valid, v1 = concatViewOf(model, m.inputs[1]).valid;
+      for (int a = 0; a <= (v0 ? 1 : 0); ++a)
+        for (int b = 0; b <= (v1 ? 1 : 0); ++b) {
+          if (!a && !b) continue;
+          Match v = m;
+          v.inputVariants = {a, b};
+          out.push_back(std::move(v));
+        }
+    }
+    return out;
+  }
   void implement(OpImpl &impl, const Model &model, const Match &m, unsigned, SymGraph &sym, const CompileOptions &) const override {
     const TensorNode &out = model.tensors()[m.output];
     unsigned off = 0;
+    impl.edge().config = m.inputVariants.empty() ? "copy" : std::string(m.inputVariants[0] ? "in-place" : "copy") + "/" + (m.inputVariants[1] ? "in-place" : "copy");
     for (int s = 0; s < 2; ++s) {
       const TensorNode &in = model.tensors()[m.inputs[s]];
+      if (!m.inputVariants.empty() && m.inputVariants[static_cast<size_t>(s)]) { // already where it belongs
+        impl.createViewConstrain(m.inputs[s], m.output, static_cast<uint64_t>(off) * 2);
+        off += in.channels;
+        continue;
+      }
       const unsigned vec = (in.channels % 8 == 0 && off % 8 == 0 && out.channels % 8 == 0) ? 8 : 1;
       auto k = m_compiler->read("copy_transform.hip");
       k.define("IN_CH", in.channels); k.define("IN_CH_OFFSET", 0); k.define("OUT_CH", out.channels); k.define("OUT_CH_OFFSET", off);

@@ -15,6 +15,9 @@
 //   ACT         0 none, 1 ReLU, 2 LeakyReLU(ALPHA);   HAS_BIAS 0/1
 //   POOL        1: store max over 2x2 output windows at (y/2, x/2) only
 //   CROP        1: store only rows/cols inside [CROP_T, CROP_T+OUT_H) x [CROP_L, CROP_L+OUT_W)
+//   OPITCH      channels between consecutive output pixels (default KOUT).  Larger when the output is the channel
+//               range of a wider tensor -- a concat whose sources are written in place; OUT then points at the
+//               first channel of the range.  OVEC 0: that range is not 16-byte aligned, store element by element
 //   WAVES, RPW  computing waves per workgroup, output rows per wave -> tile = (WAVES*RPW) x 32 pixels
 //   CK          input channels staged in LDS per step (multiple of 16)
 //
@@ -40,6 +43,12 @@ typedef unsigned short ushort_t;
 #endif
 #ifndef CROP
 #define CROP 0
+#endif
+#ifndef OPITCH
+#define OPITCH KOUT
+#endif
+#ifndef OVEC
+#define OVEC 1
 #endif
 
 // Matrix-core shape: MF = 32 -> v_mfma_f32_32x32x16_f16 (32 output channels x 32 pixels per block, 16 input
@@ -439,7 +448,9 @@ __device__ DNX_INLINE OutBuf out_buffer(_Float16 *OUT, const PushConstants &pc) 
 #else
   const unsigned w = pc.IN_W, h = pc.IN_H;
 #endif
-  return __builtin_amdgcn_make_buffer_rsrc(OUT, 0, (int)(w * h * (unsigned)KOUT * 2u), 0x00020000);
+  // the last pixel ends after its KOUT channels, not after a whole pitch: the rest belongs to another tensor's range
+  const unsigned pixels = w * h;
+  return __builtin_amdgcn_make_buffer_rsrc(OUT, 0, (int)(pixels ? ((pixels - 1u) * (unsigned)OPITCH + (unsigned)KOUT) * 2u : 0u), 0x00020000);
 }
 
 // 16 consecutive channels starting at chb of the pixel with linear index `pix`
@@ -447,12 +458,12 @@ __device__ DNX_INLINE void store16(OutBuf out, bool ok, unsigned pix, const half
 #ifdef DBG_SKIP_STORE
   ok = ok && o[0][0] == (_Float16)12345.0f; // practically never true: keeps the epilogue, drops the memory traffic
 #endif
-  const unsigned off = (pix * (unsigned)KOUT + (unsigned)chb) * 2u;
-  if (KOUT % 16 == 0) {
+  const unsigned off = (pix * (unsigned)OPITCH + (unsigned)chb) * 2u;
+  if (KOUT % 16 == 0 && OPITCH % 8 == 0 && OVEC) {
     const unsigned o0 = (ok && chb < KOUT) ? off : NO_STORE;
     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, o[0]), out, o0, 0, STORE_AUX);
     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, o[1]), out, o0 + 16u, 0, STORE_AUX);
-  } else if (KOUT % 8 == 0) {
+  } else if (KOUT % 8 == 0 && OPITCH % 8 == 0 && OVEC) {
     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, o[0]), out, (ok && chb < KOUT) ? off : NO_STORE, 0, STORE_AUX);
     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, o[1]), out, (ok && chb + 8 < KOUT) ? off + 16u : NO_STORE, 0, STORE_AUX);
   } else {
@@ -623,8 +634,8 @@ __device__ DNX_INLINE void store_vec(OutBuf out, bool ok, unsigned pix, const _F
 #ifdef DBG_SKIP_STORE
   ok = ok && o[0] == (_Float16)12345.0f;
 #endif
-  const unsigned off = (pix * (unsigned)KOUT + (unsigned)chb) * 2u;
-  if (KOUT % 8 == 0 && n == 8) {
+  const unsigned off = (pix * (unsigned)OPITCH + (unsigned)chb) * 2u;
+  if (KOUT % 8 == 0 && OPITCH % 8 == 0 && OVEC && n == 8) {
     half8 h;
 #pragma unroll
     for (int i = 0; i < 8; ++i) h[i] = o[i];

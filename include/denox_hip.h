@@ -141,6 +141,8 @@ typedef struct denox_hip_compile_options {
   int32_t enable_alternating_traversal; /* consecutive conv dispatches walk their tiles in opposite directions (cache reuse) */
   int32_t enable_upsample_fold;      /* offer kernels that fold a fused 2x upsample into the weights: fewer multiplications, the
                                         summed weights rounded to binary16 once more (no counterpart in the reference) */
+  int32_t enable_implicit_concat;    /* Features::enableImplicitConcat: a concat source whose only consumer is the concat may be
+                                        written by its producer straight into the concat's output (no copy dispatch) */
   int32_t input_format;              /* DENOX_HIP_FORMAT_* of every model input  (0 = HWC) */
   int32_t output_format;             /* DENOX_HIP_FORMAT_* of every model output (0 = HWC) */
   uint32_t assumption_count;         /* extents assumed for cost estimates */

@@ -284,3 +284,81 @@ def test_fused_patterns_agree(oracle, features, CA, CB, K, H, W):
     assert_conv_close(got, env[t.name], str(features))
     n = mod.runtime_model.dispatch_count
     assert n == (1 if not features else n)  # the default schedule is a single dispatch
+
+
+IN_PLACE_CASES = [  # (C, K0, K1, tail): channel range aligned / not aligned to 16 bytes, narrow and wide, a pooled and an activated producer
+    (8, 16, 24, "none"), (8, 16, 24, "conv"), (3, 3, 4, "none"), (9, 9, 16, "conv"), (16, 8, 3, "none"), (16, 64, 32, "conv"),
+    (8, 16, 16, "pool"), (12, 40, 24, "relu"), (32, 48, 80, "conv")]
+
+
+@pytest.mark.parametrize("config", [None, "s8r2k16", "m4r2k32x2", "t16r1k16", "q8r2k32x2"])
+@pytest.mark.parametrize("C,K0,K1,tail", IN_PLACE_CASES)
+def test_concat_sources_written_in_place(oracle, config, C, K0, K1, tail):
+    """concat(conv(x), conv(x)): each conv stores into its channel range of the concat's tensor (pixel pitch K0 + K1),
+    no copy runs, and the bits equal those of the schedule that copies."""
+    rng = np.random.default_rng(C + K0 + 3 * K1)
+    H, W = 37, 70
+    x = rng.standard_normal((H, W, C)).astype(np.float16)
+    m = dx.Model()
+    t = m.input("input", "W", "H", C)
+
+    def branch(K):
+        y = m.conv2d(t, he_weights(rng, K, C), small_bias(rng, K))
+        if tail == "relu":
+            y = m.relu(y)
+        if tail == "pool":
+            y = m.pool(m.relu(y))
+        return y
+    c = m.concat(branch(K0), branch(K1))
+    out = m.conv2d(c, he_weights(rng, 8, K0 + K1), small_bias(rng, 8)) if tail == "conv" else c
+    m.output(out)
+    # the consumer conv would otherwise read both sources itself (concat fused into the conv): keep the concat a tensor
+    feats = {"concat_conv_fusion": False}
+    try:
+        mod = dx.Module.compile(m, conv_config=config, features=feats)
+        ref = dx.Module.compile(m, conv_config=config, features={**feats, "implicit_concat": False})
+    except dx.DenoxHipError as e:
+        assert e.status == 5 and config is not None
+        pytest.skip(str(e))
+    n = 2 + (tail == "conv")
+    assert mod.runtime_model.dispatch_count == n and ref.runtime_model.dispatch_count == n + 2
+    got = mod.instance(H=H, W=W).infer(x)[0]
+    assert_bits_equal(got, ref.instance(H=H, W=W).infer(x)[0], "in place against copied")
+    want = oracle.run_graph(m.to_ops({"H": H, "W": W}), {"input": x}, "fp32")[out.name]
+    assert_conv_close(got, want, f"in-place concat {config}")
+
+
+def test_concat_with_one_source_in_place(oracle):
+    """concat(conv(x), x): the model input cannot live inside another tensor, the conv output can -- one copy instead of two."""
+    rng = np.random.default_rng(11)
+    H, W = 20, 33
+    x = rng.standard_normal((H, W, 8)).astype(np.float16)
+    m = dx.Model()
+    t = m.input("input", "W", "H", 8)
+    c = m.concat(t, m.relu(m.conv2d(t, he_weights(rng, 24, 8), small_bias(rng, 24))))
+    m.output(c)
+    mod = dx.Module.compile(m)
+    rep = dx.last_compile_report()
+    assert mod.runtime_model.dispatch_count == 2 and "copy/in-place" in rep
+    got = mod.instance(H=H, W=W).infer(x)[0]
+    assert_bits_equal(got[:, :, :8], x, "copied source")
+    want = oracle.run_graph(m.to_ops({"H": H, "W": W}), {"input": x}, "fp32")[c.name]
+    assert_conv_close(got, want, "half in-place concat")
+
+
+def test_timing_table_runs_in_place_candidates(tmp_path):
+    """The candidates that store with a foreign pixel pitch are benchmarked like any other: their scratch buffers span
+    the wider tensor, and a schedule compiled against the table still gives the same bits."""
+    rng = np.random.default_rng(2)
+    m = dx.Model()
+    t = m.input("input", "W", "H", 8)
+    c = m.concat(m.conv2d(t, he_weights(rng, 16, 8)), m.conv2d(t, he_weights(rng, 9, 8)))
+    m.output(c)
+    db = dx.Db(str(tmp_path / "t.db"))
+    assert db.populate(m, assume={"H": 48, "W": 64}, conv_config="w4r2k16") >= 6
+    r = db.bench(min_samples=2, max_relative_error=1.0)
+    assert r["failed"] == 0 and r["benchmarked"] >= 6
+    x = rng.standard_normal((48, 64, 8)).astype(np.float16)
+    got = dx.Module.load(dx.compile_model(m, assume={"H": 48, "W": 64}, conv_config="w4r2k16", db=db)).instance(H=48, W=64).infer(x)[0]
+    ref = dx.Module.compile(m, conv_config="w4r2k16", features={"implicit_concat": False}).instance(H=48, W=64).infer(x)[0]
+    assert_bits_equal(got, ref, "table-driven schedule")

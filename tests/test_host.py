@@ -128,6 +128,63 @@ def test_missing_kernel_is_reported():
     assert e.value.status == 5 and "no kernel implements" in str(e.value)
 
 
+# ----------------------------------------------------------------------------- concat without copies
+def _w(rng, k, c):
+    return (rng.standard_normal((k, c, 3, 3)) * 0.1).astype(np.float16)
+
+
+def test_concat_sources_are_placed_inside_the_result():
+    rng = np.random.default_rng(0)
+    m = dx.Model()
+    x = m.input("input", "W", "H", 8)
+    a, b = m.conv2d(x, _w(rng, 16, 8)), m.relu(m.conv2d(x, _w(rng, 24, 8)))
+    c = m.concat(a, b)
+    m.output(c)
+    d = dx.describe(dx.compile_model(m, conv_config="w4r2k16"), H=20, W=30)
+    assert [x_["name"] for x_ in d["dispatches"]] == ["conv3x3+concat", "conv3x3+relu+concat"]
+    assert all("OPITCH=40" in x_["debug_info"] and "OVEC=1" in x_["debug_info"] for x_ in d["dispatches"])
+    out = d["tensors"][d["outputs"][0]]
+    views = [t for t in d["tensors"] if not t["param"] and t.get("channels") in (16, 24)]
+    assert len(views) == 2 and all(t["buffer"] == out["buffer"] for t in views)
+    by_c = {t["channels"]: t for t in views}
+    assert (by_c[16]["offset"], by_c[24]["offset"]) == (0, 32)  # channel 16 of pixel 0
+    assert by_c[24]["size"] == out["size"] - 32 and out["size"] == 20 * 30 * 40 * 2
+    assert len(d["buffers"]) == 2 + 2  # input, result, two weight blobs: no buffer is left for the sources
+    # switched off: the convs write tensors of their own and two copies follow
+    d = dx.describe(dx.compile_model(m, conv_config="w4r2k16", features={"implicit_concat": False}), H=20, W=30)
+    assert [x_["name"] for x_ in d["dispatches"]] == ["conv3x3", "conv3x3+relu", "concat-copy-src0", "concat-copy-src1"]
+
+
+def test_concat_sources_that_cannot_move():
+    rng = np.random.default_rng(1)
+    # a source with a second consumer, a model input, a model output and concat(t, t) keep their own buffers
+    m = dx.Model()
+    x = m.input("input", "W", "H", 8)
+    a = m.conv2d(x, _w(rng, 8, 8))
+    c = m.concat(a, x)          # x: model input; a: also read by the conv below
+    e = m.conv2d(a, _w(rng, 8, 8))
+    f = m.concat(e, e)          # the same tensor twice
+    m.output(c)
+    m.output(f)
+    blob = dx.compile_model(m, conv_config="w4r2k16")
+    assert "in-place" not in dx.last_compile_report()
+    d = dx.describe(blob, H=16, W=16)
+    assert sum(x_["name"].startswith("concat-copy") for x_ in d["dispatches"]) == 4
+    m = dx.Model()
+    x = m.input("input", "W", "H", 8)
+    a = m.conv2d(x, _w(rng, 8, 8))
+    m.output(a)                 # a model output stays a tensor of its own
+    m.output(m.concat(a, m.conv2d(x, _w(rng, 16, 8))))
+    dx.compile_model(m, conv_config="w4r2k16")
+    assert "copy/in-place" in dx.last_compile_report()
+    # an unaligned channel range is stored element by element
+    m = dx.Model()
+    x = m.input("input", "W", "H", 8)
+    m.output(m.concat(m.conv2d(x, _w(rng, 3, 8)), m.conv2d(x, _w(rng, 8, 8))))
+    d = dx.describe(dx.compile_model(m, conv_config="w4r2k16"), H=16, W=16)
+    assert all("OPITCH=11" in x_["debug_info"] and "OVEC=0" in x_["debug_info"] for x_ in d["dispatches"]) and len(d["dispatches"]) == 2
+
+
 # ----------------------------------------------------------------------------- serialised model
 def test_dnx_round_trip_and_corruption():
     m, _ = networks.build("tiny_unet")
