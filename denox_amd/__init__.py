@@ -14,5 +14,5 @@ computes on the CPU.
 """
 from ._capi import DenoxHipError, LIB_PATH, build  # noqa: F401
 from .graph import Model, Sym, Tensor  # noqa: F401
-from .module import (Context, Db, Instance, Layout, Module, RuntimeModel, Shape, compile_model, describe, device_info,  # noqa: F401
+from .module import (Context, Db, Instance, Layout, Module, RuntimeModel, Shape, compile_model, describe, device_info, pinned_empty,  # noqa: F401
                      last_compile_report, report)

@@ -482,6 +482,18 @@ int denox_hip_instance_output_desc(const denox_hip_instance *inst, uint32_t i, d
 int denox_hip_instance_infer(denox_hip_instance *inst, const void *const *in, void *const *out) {
   return guarded([&] { need(inst, "instance"); inst->inst->infer(in, out); });
 }
+int denox_hip_instance_infer_many(denox_hip_instance *inst, uint32_t frames, const void *const *in, void *const *out) {
+  return guarded([&] { need(inst, "instance"); inst->inst->inferMany(frames, in, out); });
+}
+int denox_hip_host_alloc(size_t bytes, void **out) {
+  return guarded([&] {
+    need(out, "out");
+    void *p = nullptr;
+    runtime::hipCheck(hipHostMalloc(&p, bytes ? bytes : 1, hipHostMallocDefault), "hipHostMalloc");
+    *out = p;
+  });
+}
+void denox_hip_host_free(void *p) { if (p) (void)hipHostFree(p); }
 int denox_hip_instance_infer_device(denox_hip_instance *inst, const void *const *in, void *const *out) {
   return guarded([&] { need(inst, "instance"); inst->inst->inferDevice(in, out); });
 }

@@ -175,9 +175,25 @@ Instance::~Instance() {
     (void)hipSetDevice(m_model->context()->device());
     (void)hipStreamSynchronize(m_model->context()->stream());
   }
+  destroyPipeline();
   if (m_graphExec) (void)hipGraphExecDestroy(m_graphExec);
   if (m_graph) (void)hipGraphDestroy(m_graph);
   for (void *b : m_buffers) if (b) (void)hipFree(b);
+}
+
+void Instance::destroyPipeline() {
+  if (m_pipe.exec) (void)hipGraphExecDestroy(m_pipe.exec);
+  if (m_pipe.graph) (void)hipGraphDestroy(m_pipe.graph);
+  for (void *p : m_pipe.in) if (p) (void)hipFree(p);
+  for (void *p : m_pipe.out) if (p) (void)hipFree(p);
+  for (int s = 0; s < 2; ++s) {
+    if (m_pipe.inReady[s]) (void)hipEventDestroy(m_pipe.inReady[s]);
+    if (m_pipe.computed[s]) (void)hipEventDestroy(m_pipe.computed[s]);
+    if (m_pipe.outRead[s]) (void)hipEventDestroy(m_pipe.outRead[s]);
+  }
+  if (m_pipe.h2d) (void)hipStreamDestroy(m_pipe.h2d);
+  if (m_pipe.d2h) (void)hipStreamDestroy(m_pipe.d2h);
+  m_pipe = Pipeline{};
 }
 
 void *Instance::tensorPtr(uint32_t tensor) const {
@@ -256,6 +272,128 @@ void Instance::rebind(const void *const *inputs, void *const *outputs) {
     m_graph = nullptr;
     buildGraph();
   }
+}
+
+// Writes the given interface addresses into the argument buffers (no graph is touched).
+void Instance::patchInterface(const std::vector<void *> &inputs, const std::vector<void *> &outputs) {
+  const dnx::Model &m = m_model->dnx();
+  for (auto &l : m_launches)
+    for (const auto &[off, tensor] : l.ptrSlots) {
+      for (size_t i = 0; i < m.inputs.size(); ++i)
+        if (m.inputs[i] == tensor) std::memcpy(l.args.data() + off, &inputs[i], sizeof(void *));
+      for (size_t i = 0; i < m.outputs.size(); ++i)
+        if (m.outputs[i] == tensor) std::memcpy(l.args.data() + off, &outputs[i], sizeof(void *));
+    }
+}
+
+void Instance::preparePipeline() {
+  if (m_pipe.ready) return;
+  const dnx::Model &m = m_model->dnx();
+  try {
+    // default-priority streams that do not synchronise with the legacy stream
+    hipCheck(hipStreamCreateWithFlags(&m_pipe.h2d, hipStreamNonBlocking), "hipStreamCreateWithFlags");
+    hipCheck(hipStreamCreateWithFlags(&m_pipe.d2h, hipStreamNonBlocking), "hipStreamCreateWithFlags");
+    for (int s = 0; s < 2; ++s) {
+      hipCheck(hipEventCreateWithFlags(&m_pipe.inReady[s], hipEventDisableTiming), "hipEventCreate");
+      hipCheck(hipEventCreateWithFlags(&m_pipe.computed[s], hipEventDisableTiming), "hipEventCreate");
+      hipCheck(hipEventCreateWithFlags(&m_pipe.outRead[s], hipEventDisableTiming), "hipEventCreate");
+    }
+    auto alloc = [&](uint32_t tensor) {
+      void *p = nullptr;
+      const uint64_t bytes = std::max<uint64_t>(static_cast<uint64_t>(m.tensors[tensor].size.eval(m_sym)), 16) + 256;
+      hipCheck(hipMalloc(&p, bytes), "hipMalloc(second interface tensor)");
+      m_deviceBytes += bytes;
+      return p;
+    };
+    m_pipe.in.assign(m.inputs.size(), nullptr);
+    m_pipe.out.assign(m.outputs.size(), nullptr);
+    for (size_t i = 0; i < m.inputs.size(); ++i) m_pipe.in[i] = alloc(m.inputs[i]);
+    for (size_t i = 0; i < m.outputs.size(); ++i) m_pipe.out[i] = alloc(m.outputs[i]);
+    if (m_graphExec) {
+      // the same dispatch list captured once more with the second set's addresses
+      std::vector<void *> in0, out0;
+      for (uint32_t t : m.inputs) in0.push_back(tensorPtr(t));
+      for (uint32_t t : m.outputs) out0.push_back(tensorPtr(t));
+      hipGraph_t g0 = m_graph;
+      hipGraphExec_t e0 = m_graphExec;
+      m_graph = nullptr;
+      m_graphExec = nullptr;
+      patchInterface(m_pipe.in, m_pipe.out);
+      try {
+        buildGraph();
+      } catch (...) {
+        patchInterface(in0, out0);
+        m_graph = g0;
+        m_graphExec = e0;
+        throw;
+      }
+      m_pipe.graph = m_graph;
+      m_pipe.exec = m_graphExec;
+      m_graph = g0;
+      m_graphExec = e0;
+      patchInterface(in0, out0);
+    }
+    m_pipe.ready = true;
+  } catch (...) {
+    destroyPipeline();
+    throw;
+  }
+}
+
+void Instance::inferMany(size_t frames, const void *const *inputs, void *const *outputs) {
+  const dnx::Model &m = m_model->dnx();
+  if (frames == 0) return;
+  if (!inputs || !outputs) fail(Status::InvalidArgument, "infer: null pointer array");
+  const size_t nin = m.inputs.size(), nout = m.outputs.size();
+  for (size_t i = 0; i < frames * nin; ++i) if (!inputs[i]) fail(Status::InvalidArgument, "infer: null input pointer");
+  for (size_t i = 0; i < frames * nout; ++i) if (!outputs[i]) fail(Status::InvalidArgument, "infer: null output pointer");
+  m_model->context()->makeCurrent();
+  rebind(nullptr, nullptr); // set 0 is the instance's own interface tensors
+  preparePipeline();
+  hipStream_t cs = m_model->context()->stream();
+  std::vector<void *> in0, out0;
+  for (uint32_t t : m.inputs) in0.push_back(tensorPtr(t));
+  for (uint32_t t : m.outputs) out0.push_back(tensorPtr(t));
+  // nothing enqueued earlier on the context's stream may still use the interface tensors
+  hipCheck(hipStreamSynchronize(cs), "hipStreamSynchronize");
+  bool patched = false;
+  try {
+    for (size_t f = 0; f < frames; ++f) {
+      const int s = static_cast<int>(f & 1);
+      const std::vector<void *> &din = s ? m_pipe.in : in0, &dout = s ? m_pipe.out : out0;
+      // upload: the dispatches of frame f-2 have read this set's inputs
+      if (f >= 2) hipCheck(hipStreamWaitEvent(m_pipe.h2d, m_pipe.computed[s], 0), "hipStreamWaitEvent");
+      for (size_t i = 0; i < nin; ++i)
+        hipCheck(hipMemcpyAsync(din[i], inputs[f * nin + i], static_cast<uint64_t>(m.tensors[m.inputs[i]].size.eval(m_sym)), hipMemcpyHostToDevice, m_pipe.h2d), "hipMemcpyAsync(input)");
+      hipCheck(hipEventRecord(m_pipe.inReady[s], m_pipe.h2d), "hipEventRecord");
+      // dispatches: inputs are up, and the download of frame f-2 has read this set's outputs
+      hipCheck(hipStreamWaitEvent(cs, m_pipe.inReady[s], 0), "hipStreamWaitEvent");
+      if (f >= 2) hipCheck(hipStreamWaitEvent(cs, m_pipe.outRead[s], 0), "hipStreamWaitEvent");
+      if (m_graphExec) {
+        hipCheck(hipGraphLaunch(s ? m_pipe.exec : m_graphExec, cs), "hipGraphLaunch");
+      } else { // without a graph the argument buffers are read at launch time: patch them per frame
+        patchInterface(din, dout);
+        patched = s != 0;
+        launchAll(cs);
+      }
+      hipCheck(hipEventRecord(m_pipe.computed[s], cs), "hipEventRecord");
+      // download
+      hipCheck(hipStreamWaitEvent(m_pipe.d2h, m_pipe.computed[s], 0), "hipStreamWaitEvent");
+      for (size_t i = 0; i < nout; ++i)
+        hipCheck(hipMemcpyAsync(outputs[f * nout + i], dout[i], static_cast<uint64_t>(m.tensors[m.outputs[i]].size.eval(m_sym)), hipMemcpyDeviceToHost, m_pipe.d2h), "hipMemcpyAsync(output)");
+      hipCheck(hipEventRecord(m_pipe.outRead[s], m_pipe.d2h), "hipEventRecord");
+    }
+  } catch (...) {
+    (void)hipStreamSynchronize(m_pipe.h2d);
+    (void)hipStreamSynchronize(cs);
+    (void)hipStreamSynchronize(m_pipe.d2h);
+    if (patched) patchInterface(in0, out0);
+    throw;
+  }
+  hipCheck(hipStreamSynchronize(m_pipe.h2d), "hipStreamSynchronize");
+  hipCheck(hipStreamSynchronize(cs), "hipStreamSynchronize");
+  hipCheck(hipStreamSynchronize(m_pipe.d2h), "hipStreamSynchronize");
+  if (patched) patchInterface(in0, out0);
 }
 
 void Instance::inferDevice(const void *const *inputs, void *const *outputs) {

@@ -94,6 +94,13 @@ public:
   // stream and returns without synchronising.  A null entry means "use the
   // instance's own buffer for that tensor" (see inputDevicePtr/outputDevicePtr).
   void inferDevice(const void *const *inputs, void *const *outputs);
+  // A sequence of frames from host memory, arrays frame-major (inputs[f * inputCount() + i]); blocking.
+  // Upload of frame f+1, the dispatches of frame f and the download of frame f-1 run at the same time on three
+  // streams: the interface tensors exist twice, everything in between once (the dispatches of consecutive frames
+  // are serialised on the context's stream anyway).  The copies overlap only when the host memory is pinned
+  // (hipHostMalloc); with pageable memory the result is the same and the transfers are staged by the driver.
+  // The reference has no counterpart: its infer() is one blocking frame (instance.cpp:322-430).
+  void inferMany(size_t frames, const void *const *inputs, void *const *outputs);
   void synchronize();
   // Per-dispatch timings with hipEvents after warm-up passes (instance.cpp:432-654).
   std::vector<DispatchTiming> bench(int warmup);
@@ -120,6 +127,8 @@ private:
   void launchAll(hipStream_t s);
   void buildGraph();
   void rebind(const void *const *inputs, void *const *outputs);
+  void patchInterface(const std::vector<void *> &inputs, const std::vector<void *> &outputs);
+  void preparePipeline();
 
   ModelHandle m_model;
   std::vector<int64_t> m_sym;
@@ -130,6 +139,16 @@ private:
   hipGraph_t m_graph = nullptr;
   hipGraphExec_t m_graphExec = nullptr;
   uint64_t m_deviceBytes = 0;
+  // inferMany: the second set of interface tensors with its own captured graph, copy streams, per-set events
+  struct Pipeline {
+    std::vector<void *> in, out;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    hipStream_t h2d = nullptr, d2h = nullptr;
+    hipEvent_t inReady[2] = {nullptr, nullptr}, computed[2] = {nullptr, nullptr}, outRead[2] = {nullptr, nullptr};
+    bool ready = false;
+  } m_pipe;
+  void destroyPipeline();
 };
 
 } // namespace denox::runtime

@@ -278,6 +278,36 @@ class Instance:
         _capi.check(_capi.lib().denox_hip_instance_infer(self._h, pin, pout))
         return outs
 
+    def infer_many(self, frames: Sequence[Sequence[np.ndarray]], outputs: Optional[Sequence[Sequence[np.ndarray]]] = None) -> List[List[np.ndarray]]:
+        """Blocking inference on a sequence of frames (each a sequence of host arrays, one per model input) with uploads,
+        dispatches and downloads of neighbouring frames overlapped.  The overlap needs page-locked arrays (`pinned_empty`)
+        on both sides; `outputs` may supply them, else pageable arrays are allocated."""
+        nin, nout = self.input_count, self.output_count
+        ins = []
+        for f, frame in enumerate(frames):
+            if len(frame) != nin:
+                raise ValueError(f"frame {f}: model takes {nin} inputs")
+            for i, a in enumerate(frame):
+                arr = a if (isinstance(a, np.ndarray) and a.dtype == np.float16 and a.flags.c_contiguous) else np.ascontiguousarray(a, dtype=np.float16)
+                d = self.input_desc(i)
+                if arr.nbytes != d["byte_size"]:
+                    raise ValueError(f"frame {f} input {i}: expected {d['byte_size']} bytes, got {arr.nbytes}")
+                ins.append(arr)
+        if outputs is None:
+            outs = [[np.empty(self._np_shape(self.output_desc(i)), np.float16) for i in range(nout)] for _ in frames]
+        else:
+            outs = [list(o) for o in outputs]
+            for f, o in enumerate(outs):
+                if len(o) != nout or any(a.dtype != np.float16 or not a.flags.c_contiguous or a.nbytes != self.output_desc(i)["byte_size"] for i, a in enumerate(o)):
+                    raise ValueError(f"frame {f}: outputs must be contiguous float16 arrays of the model's output sizes")
+        if len(outs) != len(frames):
+            raise ValueError("one set of outputs per frame expected")
+        pin = (c_void_p * max(len(ins), 1))(*[a.ctypes.data for a in ins])
+        flat = [a for o in outs for a in o]
+        pout = (c_void_p * max(len(flat), 1))(*[a.ctypes.data for a in flat])
+        _capi.check(_capi.lib().denox_hip_instance_infer_many(self._h, len(frames), pin, pout))
+        return outs
+
     def infer_device(self, inputs: Optional[Sequence[int]] = None, outputs: Optional[Sequence[int]] = None) -> None:
         """Asynchronous inference on device addresses (ints); None = the instance's own tensors."""
         pin = (c_void_p * self.input_count)(*inputs) if inputs is not None else None
@@ -317,6 +347,31 @@ class Instance:
                         "GBps": (t.memory_reads + t.memory_writes) / ms * 1e-6 if ms > 0 else 0.0,
                         "TFLOPs": t.flops / ms * 1e-9 if ms > 0 else 0.0})
         return out
+
+
+class _PinnedBlock:
+    """Owner of one hipHostMalloc allocation; the arrays made from it keep it alive through their `base` chain."""
+
+    def __init__(self, nbytes: int):
+        p = c_void_p()
+        _capi.check(_capi.lib().denox_hip_host_alloc(max(int(nbytes), 1), byref(p)))
+        self.ptr, self.nbytes = p.value, int(nbytes)
+        self.buffer = (ctypes.c_uint8 * max(self.nbytes, 1)).from_address(self.ptr)
+        self.buffer._owner = self  # the ctypes view is what numpy holds on to
+
+    def __del__(self):
+        if getattr(self, "ptr", None):
+            _capi.lib().denox_hip_host_free(self.ptr)
+            self.ptr = None
+
+
+def pinned_empty(shape, dtype=np.float16) -> np.ndarray:
+    """An uninitialised array in page-locked host memory (denox_hip_host_alloc), from and to which `Instance.infer_many`
+    copies at bus speed and concurrently with the dispatches.  Needs a GPU."""
+    dt = np.dtype(dtype)
+    n = int(np.prod(shape)) * dt.itemsize
+    block = _PinnedBlock(n)
+    return np.frombuffer(block.buffer, dtype=dt, count=int(np.prod(shape))).reshape(shape)
 
 
 def report(timings: List[dict]) -> str:

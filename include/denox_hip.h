@@ -244,6 +244,16 @@ int denox_hip_instance_input_desc(const denox_hip_instance *inst, uint32_t i, de
 int denox_hip_instance_output_desc(const denox_hip_instance *inst, uint32_t i, denox_hip_tensor_desc *out);
 /* blocking; host arrays in model input / output order */
 int denox_hip_instance_infer(denox_hip_instance *inst, const void *const *host_inputs, void *const *host_outputs);
+/* `frames` consecutive frames, blocking; host arrays frame-major: host_inputs[f * input_count + i].  The upload of the next
+ * frame, the dispatches of the current one and the download of the previous one overlap on three streams (the interface
+ * tensors exist twice on the device).  The copies overlap only from / to pinned host memory (denox_hip_host_alloc); pageable
+ * memory gives the same result at the speed of denox_hip_instance_infer.  No counterpart in the reference, whose
+ * Instance::infer is one blocking frame (runtime/src/denox/runtime/instance.cpp:322-430): for callers that stream
+ * frames from host memory. */
+int denox_hip_instance_infer_many(denox_hip_instance *inst, uint32_t frames, const void *const *host_inputs, void *const *host_outputs);
+/* page-locked host memory for denox_hip_instance_infer_many / _infer (hipHostMalloc); release with denox_hip_host_free */
+int denox_hip_host_alloc(size_t bytes, void **out);
+void denox_hip_host_free(void *p);
 /* asynchronous on the context's stream; device arrays, entries (or the arrays
  * themselves) may be NULL to use the instance's own tensors */
 int denox_hip_instance_infer_device(denox_hip_instance *inst, const void *const *dev_inputs, void *const *dev_outputs);

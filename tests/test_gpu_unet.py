@@ -194,3 +194,36 @@ def test_model_file_round_trip_and_a_model_compiled_for_vulkan(tmp_path):
     with pytest.raises(dx.DenoxHipError) as e:
         dx.Module.load(as_written_for_vulkan(blob)).instance(H=32, W=48)
     assert e.value.status == 5 and "SPIR-V" in str(e.value)
+
+
+@pytest.mark.parametrize("net,H,W,layout", [("tiny_unet", 64, 96, "HWC"), ("oidn_unet", 40, 56, "HWC"), ("oidn_unet", 33, 47, "CHW")])
+@pytest.mark.parametrize("pinned", [False, True])
+def test_frame_sequence_matches_frame_by_frame(net, H, W, layout, pinned):
+    """infer_many overlaps upload, dispatches and download of neighbouring frames on three streams with the interface
+    tensors doubled: every frame's bits equal those of a blocking infer of that frame alone, for 1, 2 and 5 frames,
+    from pageable and from page-locked memory, and a plain infer afterwards still works."""
+    m, _ = networks.build(net, seed=1)
+    lay = dx.Layout[layout]
+    inst = dx.Module.compile(m, input_layout=lay, output_layout=lay).instance(H=H, W=W)
+    frames = [networks.synthetic_input(net, H, W, seed=10 + f) for f in range(5)]
+    if layout == "CHW":
+        frames = [np.ascontiguousarray(x.transpose(2, 0, 1)) for x in frames]
+    want = [inst.infer(x)[0].copy() for x in frames]
+    assert any(not np.array_equal(want[0], w) for w in want[1:])
+    for n in (1, 2, 5):
+        if pinned:
+            ins = [dx.pinned_empty(frames[f].shape) for f in range(n)]
+            outs = [[dx.pinned_empty(want[f].shape)] for f in range(n)]
+            for f in range(n):
+                ins[f][...] = frames[f]
+                outs[f][0][...] = 0
+            got = inst.infer_many([[a] for a in ins], outs)
+            assert got[0][0] is outs[0][0]
+        else:
+            got = inst.infer_many([[frames[f]] for f in range(n)])
+        for f in range(n):
+            assert_bits_equal(got[f][0], want[f], f"frame {f} of {n}")
+    assert_bits_equal(inst.infer(frames[3])[0], want[3], "blocking infer after the sequence")
+    inst.infer_device(None, None)
+    inst.synchronize()
+    assert inst.infer_many([]) == []
