@@ -255,7 +255,8 @@ std::vector<uint8_t> serialize(const Model &m) {
 }
 
 Model deserialize(const void *data, size_t size) {
-  const fb::Table root = fb::Table::root(data, size, IDENTIFIER);
+  size_t spent = 0;
+  const fb::Table root = fb::Table::root(data, size, IDENTIFIER, &spent);
   Reader r;
   Model m;
   m.version = root.scalar<uint16_t>(id::M_version, 0);

@@ -153,6 +153,16 @@ private:
 struct Buf {
   const uint8_t *p = nullptr;
   size_t n = 0;
+  // Bytes of tables, vectors and strings handed out so far.  Offsets may legally point at shared objects, so a small
+  // file can describe a huge object graph (a long vector whose elements all name one large table); a reader that
+  // copies what it visits would be made to allocate without bound.  Every object visited is charged here and the walk
+  // stops at a multiple of the buffer size that no honest file, whose objects are visited a few times each, reaches.
+  size_t *spent = nullptr;
+  void charge(size_t bytes) const {
+    if (!spent) return;
+    *spent += bytes + 4;
+    if (*spent > 16 * n + (1u << 16)) fail(Status::InvalidModel, "flatbuffer: object graph larger than the buffer allows");
+  }
   void check(size_t pos, size_t len, size_t align) const {
     if (pos > n || len > n - pos) fail(Status::InvalidModel, "flatbuffer: object outside the buffer");
     if (align > 1 && (pos & (align - 1))) fail(Status::InvalidModel, "flatbuffer: misaligned object");
@@ -181,6 +191,7 @@ public:
     m_data = pos + 4;
     if (elemSize && m_len > (b.n - m_data) / elemSize) fail(Status::InvalidModel, "flatbuffer: vector longer than the buffer");
     b.check(m_data, static_cast<size_t>(m_len) * elemSize, align);
+    b.charge(static_cast<size_t>(m_len) * elemSize);
   }
   bool present() const { return m_present; }
   uint32_t size() const { return m_len; }
@@ -221,10 +232,13 @@ public:
     m_tblSize = b.rd<uint16_t>(m_vt + 2);
     if (m_tblSize < 4) fail(Status::InvalidModel, "flatbuffer: bad table size");
     b.check(pos, m_tblSize, 4);
+    b.charge(m_tblSize);
   }
   // `identifier` may be null for a schema that declares none.
-  static Table root(const void *data, size_t size, const char *identifier) {
-    Buf b{static_cast<const uint8_t *>(data), size};
+  // `spent` (optional) is the caller's counter for Buf::charge; it must outlive every view made from the root.
+  static Table root(const void *data, size_t size, const char *identifier, size_t *spent = nullptr) {
+    Buf b{static_cast<const uint8_t *>(data), size, spent};
+    if (spent) *spent = 0;
     if (!data || size < 12) fail(Status::InvalidModel, "flatbuffer: buffer too short");
     if (size > 0x7FFFFFFFu) fail(Status::InvalidModel, "flatbuffer: buffer exceeds 2 GiB");
     if (identifier && std::memcmp(b.p + 4, identifier, 4) != 0) fail(Status::InvalidModel, std::string("flatbuffer: file identifier is not '") + std::string(identifier, 4) + "'");
@@ -254,6 +268,7 @@ public:
     const uint32_t len = m_b.rd<uint32_t>(pos);
     m_b.check(pos + 4, static_cast<size_t>(len) + 1, 1);
     if (m_b.p[pos + 4 + len] != 0) fail(Status::InvalidModel, "flatbuffer: string without terminator");
+    m_b.charge(len);
     return std::string(reinterpret_cast<const char *>(m_b.p + pos + 4), len);
   }
   Buf buf() const { return m_b; }

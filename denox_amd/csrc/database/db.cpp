@@ -195,7 +195,8 @@ Db Db::deserialize(const void *data, size_t size, const std::string &path) {
   Db db;
   db.m_path = path;
   try {
-    const fb::Table root = fb::Table::root(data, size, IDENTIFIER);
+    size_t spent = 0;
+    const fb::Table root = fb::Table::root(data, size, IDENTIFIER, &spent);
     if (root.scalar<uint32_t>(id::Db_version, 0) != 0) fail(Status::IoError, "unknown version");
     const fb::Vector envs = root.vector(id::Db_env, 4, 4);
     for (uint32_t i = 0; i < envs.size(); ++i) {

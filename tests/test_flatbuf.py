@@ -425,3 +425,73 @@ def test_db_written_the_reference_way_is_read(probe, tmp_path):
     db.writeback()
     again = dx.Db(str(path))
     assert [again.row_stats(i)[0] for i in range(3)] == [3, 1, 120] and again.row_stats(2)[1] == mean[2]
+
+
+def _shared_object_bomb(n: int, name_len: int) -> bytes:
+    """A valid dnx buffer, written by hand front to back, whose value_names vector names ONE table `n` times: a few
+    hundred KB on disk, n * name_len bytes for a reader that copies every element it visits."""
+    out = bytearray(8)
+    out[4:8] = b"dnxx"
+
+    def align(k):
+        while len(out) % k:
+            out.append(0)
+
+    def table(fields, nslots):
+        """fields: {slot: (fmt, value)} with 'O' = offset patched later; returns (table position, {slot: field position})."""
+        align(4)
+        vt = len(out)
+        inline = sorted(fields.items(), key=lambda kv: -struct.calcsize("I" if kv[1][0] == "O" else kv[1][0]))
+        offs, pos = {}, 4
+        for slot, (fmt, _) in inline:
+            size = struct.calcsize("I" if fmt == "O" else fmt)
+            pos = (pos + size - 1) // size * size
+            offs[slot] = pos
+            pos += size
+        tbl_size = (pos + 3) // 4 * 4
+        out.extend(struct.pack("<HH", 4 + 2 * nslots, tbl_size))
+        for slot in range(nslots):
+            out.extend(struct.pack("<H", offs.get(slot, 0)))
+        align(4)
+        t = len(out)
+        out.extend(struct.pack("<i", t - vt) + bytes(tbl_size - 4))
+        where = {}
+        for slot, (fmt, value) in fields.items():
+            where[slot] = t + offs[slot]
+            if fmt != "O":
+                struct.pack_into("<" + fmt, out, where[slot], value)
+        return t, where
+
+    def point(field_pos, target):
+        struct.pack_into("<I", out, field_pos, target - field_pos)
+
+    root, rw = table({11: ("O", None)}, 12)
+    struct.pack_into("<I", out, 0, root)
+    align(4)
+    vec = len(out)
+    point(rw[11], vec)
+    out.extend(struct.pack("<I", n) + bytes(4 * n))
+    vn, vw = table({0: ("O", None), 1: ("B", 1), 2: ("O", None)}, 3)  # ValueName{name, value: literal}
+    for i in range(n):
+        point(vec + 4 + 4 * i, vn)
+    lit, lw = table({0: ("B", 4), 1: ("O", None)}, 2)  # ScalarLiteral{dtype: I64, bytes}
+    point(vw[2], lit)
+    align(4)
+    point(lw[1], len(out))
+    out.extend(struct.pack("<Iq", 8, 7))
+    align(4)
+    point(vw[0], len(out))
+    out.extend(struct.pack("<I", name_len) + b"n" * name_len + b"\0")
+    align(8)
+    return bytes(out)
+
+
+def test_shared_objects_cannot_make_the_reader_allocate_without_bound():
+    small = _shared_object_bomb(3, 10)
+    d = dx.describe(small)
+    assert d["value_names"] == ["n" * 10] * 3 and d["dispatches"] == []  # the hand-written buffer is a valid (empty) model
+    bomb = _shared_object_bomb(100_000, 100_000)  # 0.5 MB on disk, 10 GB if every element were copied
+    assert len(bomb) < 1 << 20
+    with pytest.raises(dx.DenoxHipError) as e:
+        dx.describe(bomb)
+    assert e.value.status == 2 and "object graph" in str(e.value)
