@@ -47,7 +47,7 @@ std::string fmtFloat(float v) {
 // per workgroup (0 = none); mf: matrix shape 32 (32x32x16) or 16 (16x16x32); xb: 16-pixel blocks per row (mf 16).
 // pp: two-phase schedule of the persistent kernel (two wave groups alternate matrix work and everything else).
 // fold: the 2x upsample of source A folded into the weights (conv3x3_upfold.hip; rpw counts low-resolution rows).
-struct ConvConfig { unsigned waves, rpw, ck; bool resident; unsigned pw; unsigned maxKT; unsigned mf, xb; const char *name; bool pp = false; bool fold = false; };
+struct ConvConfig { unsigned waves, rpw, ck; bool resident; unsigned pw; unsigned maxKT; unsigned mf, xb; const char *name; bool pp = false; bool fold = false; bool wideHalo = false; };
 const ConvConfig kConvConfigs[] = {
     // weights streamed per step
     {4, 2, 16, false, 0, 0, 32, 1, "w4r2k16"}, {4, 2, 32, false, 0, 0, 32, 1, "w4r2k32"}, {4, 4, 16, false, 0, 0, 32, 1, "w4r4k16"}, {4, 4, 32, false, 0, 0, 32, 1, "w4r4k32"},
@@ -78,6 +78,10 @@ const ConvConfig kConvConfigs[] = {
     {8, 1, 16, true, 0, 0, 32, 1, "t8r1k16", true},   {8, 2, 32, true, 0, 0, 16, 2, "u8r2k32x2", true}, {16, 1, 32, true, 0, 0, 16, 2, "u16r1k32x2", true},
     // upsample folded into the weights (layers whose source A is upsampled; one parity class of output pixels per workgroup)
     {8, 1, 16, true, 0, 0, 32, 1, "f8r1", false, true},  {4, 2, 16, true, 0, 0, 32, 1, "f4r2", false, true}, {4, 1, 16, true, 0, 0, 32, 1, "f4r1", false, true},
+    // the smallest tiles, offered to strided layers only: a stride multiplies the halo of a tile, and a 7 x 7 filter with
+    // stride 4 fits the LDS next to its weights with nothing larger
+    {2, 1, 16, false, 0, 32, 32, 1, "w2r1k16n", false, false, true}, {2, 1, 32, false, 0, 16, 16, 1, "m2r1k32x1n", false, false, true},
+    {2, 2, 16, false, 0, 32, 32, 1, "w2r2k16n", false, false, true},
 };
 constexpr unsigned kNumConvConfigs = sizeof(kConvConfigs) / sizeof(kConvConfigs[0]);
 
@@ -85,7 +89,8 @@ enum ConvPatternBits : unsigned { PAT_CONCAT = 1, PAT_UPSAMPLE = 2, PAT_ACT = 4,
 
 struct ConvGeometry {
   unsigned CA, CB, C, CPAD, K, KOUTP, KT, slots;
-  unsigned R = 3, S = 3; // filter rows / columns (set before chooseKT)
+  unsigned R = 3, S = 3;   // filter rows / columns (set before chooseKT)
+  unsigned SY = 1, SX = 1; // stride (set before chooseKT)
   size_t ldsBytes;
 };
 
@@ -110,7 +115,7 @@ bool chooseKT(const ConvConfig &cfgIn, unsigned CA, unsigned CB, unsigned K, con
   if (cfg.ck > 192 || cfg.ck % kstep) return false; // staging registers; whole matrix steps only
   const unsigned th = cfg.waves * cfg.rpw;
   const unsigned tw = cfg.mf == 32 ? 32 : 16 * cfg.xb;
-  const unsigned haloPix = (th + g.R - 1) * (tw + g.S - 1), taps = g.R * g.S;
+  const unsigned haloPix = ((th - 1) * g.SY + g.R) * ((tw - 1) * g.SX + g.S), taps = g.R * g.S;
   const unsigned ckp = cfg.ck + 8;
   const unsigned blocks = g.KOUTP / blk;
   // registers per lane: 512 shared by the waves of one SIMD; a workgroup of `waves` waves puts waves/4 on each
@@ -125,7 +130,12 @@ bool chooseKT(const ConvConfig &cfgIn, unsigned CA, unsigned CB, unsigned K, con
                                      : (static_cast<size_t>(haloPix) + taps * kb * blk) * ckp * 2u) +
                        static_cast<size_t>(kb * blk) * 2u; // + the staged bias
     if (lds > dev.maxComputeSharedMemory) continue;
-    if (taps > 9) { // larger filters: the registers that stage one step's weights and halo share count as well
+    {
+      // a thread stages at most 64 halo vectors per step (the kernels' bookkeeping is one bit per vector)
+      const unsigned stagers = (cfg.pw ? cfg.pw : cfg.waves) * 64;
+      if ((haloPix * (cfg.ck / 8) + stagers - 1) / stagers > 64) continue;
+    }
+    if (taps > 9 || g.SY > 1 || g.SX > 1) { // larger filters / halos: the registers that stage one step's weights and halo share count as well
       const unsigned vppk = cfg.ck / 8, threads = cfg.waves * 64, stagers = (cfg.pw ? cfg.pw : cfg.waves) * 64;
       const unsigned stage = cfg.resident ? 2 * 4 * ((haloPix * vppk + stagers - 1) / stagers)
                                           : 4 * ((taps * kb * blk * vppk + threads - 1) / threads + (haloPix * vppk + threads - 1) / threads);
@@ -271,9 +281,10 @@ public:
     for (size_t i = 0; i < ops.size(); ++i) {
       const Op &conv = ops[i];
       if (conv.kind != OpKind::Conv) continue;
-      // odd filter extents up to 7 with "same" zero padding, stride 1, no dilation
-      if (conv.R % 2 == 0 || conv.S % 2 == 0 || conv.R > 7 || conv.S > 7 || conv.strideX != 1 || conv.strideY != 1 || conv.padX != (conv.S - 1) / 2 ||
-          conv.padY != (conv.R - 1) / 2 || conv.dilX != 1 || conv.dilY != 1) continue;
+      // filters up to 7 x 7, zero padding up to 15, strides up to 4, no dilation (the reference's conv shaders take
+      // kernel size, STRIDE_* and PADDING_* as parameters as well and have no dilation either)
+      if (conv.R < 1 || conv.S < 1 || conv.R > 7 || conv.S > 7 || conv.strideX < 1 || conv.strideY < 1 || conv.strideX > 4 || conv.strideY > 4 ||
+          conv.padX > 15 || conv.padY > 15 || conv.dilX != 1 || conv.dilY != 1) continue;
       // A fused-away tensor may have other consumers: whoever needs it materialised gets it
       // from another edge, and the selection weighs both.
       struct Pro { unsigned bits; std::vector<int> ops; std::vector<int> inputs; };
@@ -349,16 +360,18 @@ public:
       if (cfg.fold) {
         const unsigned others = PAT_POOL | PAT_CROP | PAT_PADA;
         FoldGeometry fg;
-        if ((m.pattern & PAT_UPSAMPLE) && !(m.pattern & others) && conv.R == 3 && conv.S == 3 && opt.features.enableUpsampleFold && chooseFold(cfg, CA, CB, conv.K, opt.deviceInfo, fg))
+        if ((m.pattern & PAT_UPSAMPLE) && !(m.pattern & others) && conv.R == 3 && conv.S == 3 && conv.padX == 1 && conv.padY == 1 && conv.strideX == 1 && conv.strideY == 1 &&
+            opt.features.enableUpsampleFold && chooseFold(cfg, CA, CB, conv.K, opt.deviceInfo, fg))
           out.push_back(c);
         continue;
       }
+      if (cfg.wideHalo && conv.strideX == 1 && conv.strideY == 1) continue;
       if (cfg.ck > cpad && cfg.ck != kstep) continue; // a larger stage than the whole reduction adds nothing
       if (cfg.ck <= 1 && cpad <= 32) continue;     // "whole / half reduction" duplicates a fixed-size stage for narrow layers
       if ((m.pattern & PAT_POOL) && (cfg.rpw % 2)) continue;
       if ((cfg.waves + cfg.pw) * 64 > opt.deviceInfo.maxComputeWorkGroupInvocations) continue;
       ConvGeometry g;
-      g.R = conv.R; g.S = conv.S;
+      g.R = conv.R; g.S = conv.S; g.SY = conv.strideY; g.SX = conv.strideX;
       if (!chooseKT(cfg, CA, CB, conv.K, opt.deviceInfo, g)) continue;
       out.push_back(c);
     }
@@ -383,7 +396,7 @@ public:
     const unsigned CA = tA.channels;
     const unsigned CB = m.inputs.size() > 1 ? model.tensors()[m.inputs[1]].channels : 0;
     ConvGeometry g;
-    g.R = conv.R; g.S = conv.S;
+    g.R = conv.R; g.S = conv.S; g.SY = conv.strideY; g.SX = conv.strideX;
     FoldGeometry fg{};
     if (cfg.fold) {
       if (!chooseFold(cfg, CA, CB, conv.K, opt.deviceInfo, fg)) fail(Status::Internal, "conv config rejected at implement time");
@@ -414,21 +427,27 @@ public:
     if (cfg.pw) k.define("PW", cfg.pw);
     if (cfg.pp) k.define("PP", 1);
     if (conv.R != 3 || conv.S != 3) { k.define("KR", conv.R); k.define("KS", conv.S); }
+    const bool samePad = conv.padY == (conv.R - 1) / 2 && conv.padX == (conv.S - 1) / 2, unitStride = conv.strideX == 1 && conv.strideY == 1;
+    if (!samePad) { k.define("PY", conv.padY); k.define("PX", conv.padX); }
+    if (!unitStride) { k.define("SY", conv.strideY); k.define("SX", conv.strideX); }
     if (cfg.mf != 32) { k.define("MF", cfg.mf); k.define("XB", cfg.xb); }
     const ConcatView view = m.outputVariant ? concatViewOf(model, m.output) : ConcatView{};
     if (m.outputVariant && !view.valid) fail(Status::Internal, "conv match writes into a concat that does not exist");
     const bool ovec = view.valid && view.pitch % 8 == 0 && view.channelOffset % 8 == 0;
     if (view.valid) { k.define("OPITCH", view.pitch); k.define("OVEC", ovec ? 1 : 0); }
-    std::string entry = "conv" + std::to_string(conv.R) + "x" + std::to_string(conv.S) + "_c" + std::to_string(CA) + (up ? "u" : "") + (padA ? "e" : "") + (CB ? "p" + std::to_string(CB) + (padB ? "e" : "") : "") + "_k" +
+    std::string entry = "conv" + std::to_string(conv.R) + "x" + std::to_string(conv.S) + (samePad ? "" : "p" + std::to_string(conv.padY) + "x" + std::to_string(conv.padX)) +
+                        (unitStride ? "" : "s" + std::to_string(conv.strideY) + "x" + std::to_string(conv.strideX)) + "_c" + std::to_string(CA) + (up ? "u" : "") + (padA ? "e" : "") + (CB ? "p" + std::to_string(CB) + (padB ? "e" : "") : "") + "_k" +
                         std::to_string(conv.K) + (act == 1 ? "_relu" : act == 2 ? "_lrelu" : "") + (pool ? "_pool" : "") + (crop ? "_crop" : "") +
                         (view.valid ? "_into" + std::to_string(view.pitch) + (ovec ? "" : "e") : "") + "_" + cfg.name;
     k.define("KERNEL_NAME", entry);
     const Sym W = convIn.width, H = convIn.height;
+    const TensorNode &convOut = model.tensors()[conv.output]; // the convolution's own result, whatever is fused behind it
+    const Sym OW = convOut.width, OH = convOut.height;
     const unsigned th = cfg.waves * cfg.rpw;
     const unsigned nkt = g.KOUTP / g.KT;
     auto d = cfg.fold ? impl.registerDispatch(k, entry, Sym::Const(opt.deviceInfo.xcdCount * 4 * nkt * g.slots), Sym::Const(1), Sym::Const(1), cfg.waves * 64)
            : cfg.resident ? impl.registerDispatch(k, entry, Sym::Const(opt.deviceInfo.xcdCount * nkt * g.slots), Sym::Const(1), Sym::Const(1), (cfg.waves + cfg.pw) * 64)
-                          : impl.registerDispatch(k, entry, sym.cdiv(W, cfg.mf == 32 ? 32 : 16 * cfg.xb), sym.cdiv(H, th), Sym::Const(nkt), cfg.waves * 64);
+                          : impl.registerDispatch(k, entry, sym.cdiv(OW, cfg.mf == 32 ? 32 : 16 * cfg.xb), sym.cdiv(OH, th), Sym::Const(nkt), cfg.waves * 64);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     if (CB) d.addBinding(dnx::Access::ReadOnly, m.inputs[1]);
     if (view.valid) {
@@ -486,7 +505,7 @@ public:
     reads = sym.add(reads, static_cast<int64_t>(conv.K) * conv.C * conv.R * conv.S * 2 + (conv.hasBias ? conv.K * 2 : 0));
     d.setMemoryReads(reads);
     d.setMemoryWrites(bytesOf(sym, model.tensors()[m.output]));
-    d.setFlops(sym.mul(sym.mul(W, H), static_cast<int64_t>(2) * conv.R * conv.S * conv.C * conv.K));
+    d.setFlops(sym.mul(sym.mul(OW, OH), static_cast<int64_t>(2) * conv.R * conv.S * conv.C * conv.K));
   }
 
 private:

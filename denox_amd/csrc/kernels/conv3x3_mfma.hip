@@ -74,7 +74,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   const int wv = tid >> 6;
   const int lane = tid & 63;
   const bool rev = (pc.FLAGS & 1u) != 0;
-  const int tilesX = (pc.IN_W + TW - 1) / TW, tilesY = (pc.IN_H + TH - 1) / TH;
+  const int tilesX = (CONV_OUT_W(pc) + TW - 1) / TW, tilesY = (CONV_OUT_H(pc) + TH - 1) / TH;
   const int x0 = (rev ? tilesX - 1 - (int)DNX_BID_X : (int)DNX_BID_X) * TW;
   const int y0 = (rev ? tilesY - 1 - (int)DNX_BID_Y : (int)DNX_BID_Y) * TH;
   const int kt = DNX_BID_Z; // output-channel tile

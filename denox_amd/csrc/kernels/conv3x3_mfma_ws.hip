@@ -58,8 +58,8 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   const int q = b / NXCD;
   const int kt = q % NKT;
   const int slot = q / NKT;
-  const int tilesX = (pc.IN_W + TW - 1) / TW;
-  const int tilesY = (pc.IN_H + TH - 1) / TH;
+  const int tilesX = (CONV_OUT_W(pc) + TW - 1) / TW;
+  const int tilesY = (CONV_OUT_H(pc) + TH - 1) / TH;
   const int numTiles = tilesX * tilesY;
   const int perXcd = (numTiles + NXCD - 1) / NXCD;
   const int first = xcd * perXcd;

@@ -21,7 +21,7 @@
 #ifndef KERNEL_NAME
 #define KERNEL_NAME conv3x3_upfold
 #endif
-static_assert(UPA == 1 && MF == 32 && !POOL && !CROP && !PADA && KR == 3 && KS == 3, "upsample-folded variant");
+static_assert(UPA == 1 && MF == 32 && !POOL && !CROP && !PADA && KR == 3 && KS == 3 && PY == 1 && PX == 1 && SY == 1 && SX == 1, "upsample-folded variant");
 static_assert(CA % 8 == 0 && (CB == 0 || CB >= 8), "whole 8-channel vectors of A; at least one whole vector of B");
 
 #define NKT (KOUTP / KT)

@@ -2,7 +2,7 @@
 // source loader (concat / upsample / replicate-pad folded into the addressing)
 // and the epilogue (bias, activation, rounding, 2x2 max pool or crop, store).
 //
-//   out[y,x,k] = act(bias[k] + sum_{r,s,c} src[y+r-PADY, x+s-PADX, c] * W[k,c,r,s])   (zero outside the image; KR x KS taps)
+//   out[y,x,k] = act(bias[k] + sum_{r,s,c} src[y*SY+r-PY, x*SX+s-PX, c] * W[k,c,r,s])   (zero outside the image; KR x KS taps)
 //   src[y,x,c] = c < CA ? A'[y,x,c] : B'[y,x,c-CA]
 //   A' = UPA ? A[y/2, x/2] : (PADA ? A[clamp(y-PAD_T), clamp(x-PAD_L)] : A[y,x]),   B' likewise with PADB
 //
@@ -63,8 +63,24 @@ typedef unsigned short ushort_t;
 #define KS 3
 #endif
 #define NTAPS (KR * KS)
-#define PADY ((KR - 1) / 2)
-#define PADX ((KS - 1) / 2)
+// Zero padding PY x PX (default: the image extent is kept for odd filters) and stride SY x SX (default 1):
+// out[y, x] = sum in[y * SY + r - PY, x * SX + s - PX] * w[r, s]; output extent (IN + 2 P - K) / S + 1
+// (direct_conv.comp:209-212,304-311 of the reference take STRIDE_* and PADDING_* the same way).
+#ifndef PY
+#define PY ((KR - 1) / 2)
+#endif
+#ifndef PX
+#define PX ((KS - 1) / 2)
+#endif
+#ifndef SY
+#define SY 1
+#endif
+#ifndef SX
+#define SX 1
+#endif
+// extent of the convolution's own output (before POOL / CROP); folds to IN_W / IN_H for the default padding and stride
+#define CONV_OUT_W(pc) (((pc).IN_W + 2u * PX - KS) / SX + 1u)
+#define CONV_OUT_H(pc) (((pc).IN_H + 2u * PY - KR) / SY + 1u)
 #ifndef MF
 #define MF 32
 #endif
@@ -78,8 +94,9 @@ typedef unsigned short ushort_t;
 #define TAIL (CPAD - (NCHUNK - 1) * CK)
 #define TW (MF == 32 ? 32 : 16 * XB)
 #define TH (WAVES * RPW)
-#define HALO_W (TW + KS - 1)
-#define HALO_H (TH + KR - 1)
+#define HALO_W ((TW - 1) * SX + KS)
+#define HALO_H ((TH - 1) * SY + KR)
+#define PXROWS ((RPW - 1) * SY + KR) // halo rows one wave's RPW output rows read
 #define HALO_PIX (HALO_W * HALO_H)
 #define CKP (CK + 8)
 #define KB (KT / MF)
@@ -314,8 +331,8 @@ struct Halo {
   static __device__ DNX_INLINE void src_init(Src &s, const Map &m, int y0, int x0, const PushConstants &pc) {
 #pragma unroll
     for (int it = 0; it < NV; ++it) {
-      const int gy = y0 + m.hy[it] - PADY;
-      const int gx = x0 + m.hx[it] - PADX;
+      const int gy = y0 * SY + m.hy[it] - PY; // (y0, x0): the tile's first output pixel
+      const int gx = x0 * SX + m.hx[it] - PX;
       size_t pa = 0, pb = 0;
       const bool inside = m.lds[it] >= 0 && gy >= 0 && gy < (int)pc.IN_H && gx >= 0 && gx < (int)pc.IN_W;
       if (inside)
@@ -442,11 +459,11 @@ typedef __amdgpu_buffer_rsrc_t OutBuf;
 
 __device__ DNX_INLINE OutBuf out_buffer(_Float16 *OUT, const PushConstants &pc) {
 #if POOL
-  const unsigned w = pc.IN_W >> 1, h = pc.IN_H >> 1;
+  const unsigned w = CONV_OUT_W(pc) >> 1, h = CONV_OUT_H(pc) >> 1;
 #elif CROP
   const unsigned w = pc.OUT_W, h = pc.OUT_H;
 #else
-  const unsigned w = pc.IN_W, h = pc.IN_H;
+  const unsigned w = CONV_OUT_W(pc), h = CONV_OUT_H(pc);
 #endif
   // the last pixel ends after its KOUT channels, not after a whole pitch: the rest belongs to another tensor's range
   const unsigned pixels = w * h;
@@ -544,7 +561,7 @@ __device__ DNX_INLINE void pack_tile(const Acc &acc, Packed &pk, const _Float16 
 __device__ DNX_INLINE void
 store_packed(const Packed &pk, OutBuf out, int y0, int x0, int kt, int wv, int lane, const PushConstants &pc, int part = 0, int nparts = 1,
              int ystep = 1, int xstep = 1) { // (steps of 2: a kernel that computes every other row / column of the output)
-  const unsigned W = pc.IN_W, H = pc.IN_H;
+  const unsigned W = CONV_OUT_W(pc), H = CONV_OUT_H(pc);
   const int l32 = lane & 31;
   const int x = x0 + l32 * xstep;
 #pragma unroll
@@ -585,10 +602,11 @@ mma_chunk(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, int wv, i
 #pragma unroll
     for (int ks = 0; ks < L / 16; ++ks) {
       const int kk = ks * 16 + kq;
-      half8 px[RPW + KR - 1];
+      half8 px[PXROWS];
 #pragma unroll
-      for (int hr = 0; hr < RPW + KR - 1; ++hr)
-        px[hr] = *reinterpret_cast<const half8 *>(sIn + ((wv * RPW + hr) * HALO_W + l32 + s) * CKP + kk);
+      for (int hr = 0; hr < PXROWS; ++hr)
+        if (SY == 1 || hr % SY < KR) // with a stride larger than the filter some halo rows are never read
+          px[hr] = *reinterpret_cast<const half8 *>(sIn + ((wv * RPW * SY + hr) * HALO_W + l32 * SX + s) * CKP + kk);
 #pragma unroll
       for (int r = 0; r < KR; ++r) {
         half8 wf[KB];
@@ -600,9 +618,9 @@ mma_chunk(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, int wv, i
 #pragma unroll
           for (int j = 0; j < RPW; ++j)
 #ifndef DBG_SKIP_MMA
-            acc.v[kb][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[kb], px[j + r], acc.v[kb][j], 0, 0, 0);
+            acc.v[kb][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[kb], px[j * SY + r], acc.v[kb][j], 0, 0, 0);
 #else
-            acc.v[kb][j][0] += (float)wf[kb][0] * (float)px[j + r][0]; // keeps the LDS reads alive without matrix work
+            acc.v[kb][j][0] += (float)wf[kb][0] * (float)px[j * SY + r][0]; // keeps the LDS reads alive without matrix work
 #endif
       }
     }
@@ -704,7 +722,7 @@ __device__ DNX_INLINE void pack_tile(const Acc &acc, Packed &pk, const _Float16 
 // together: a 128-byte line that is filled in two portions far apart in time is written to memory twice.
 __device__ DNX_INLINE void
 store_packed(const Packed &pk, OutBuf out, int y0, int x0, int kt, int wv, int lane, const PushConstants &pc, int part = 0, int nparts = 1) {
-  const unsigned W = pc.IN_W, H = pc.IN_H;
+  const unsigned W = CONV_OUT_W(pc), H = CONV_OUT_H(pc);
   const int l16 = lane & 15;
   const int g = lane >> 4;
 #pragma unroll
@@ -749,12 +767,13 @@ mma_chunk(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, int wv, i
 #pragma unroll
     for (int ks = 0; ks < L / 32; ++ks) {
       const int kk = ks * 32 + kq;
-      half8 px[RPW + KR - 1][XB];
+      half8 px[PXROWS][XB];
 #pragma unroll
-      for (int hr = 0; hr < RPW + KR - 1; ++hr)
+      for (int hr = 0; hr < PXROWS; ++hr)
 #pragma unroll
         for (int xb = 0; xb < XB; ++xb)
-          px[hr][xb] = *reinterpret_cast<const half8 *>(sIn + ((wv * RPW + hr) * HALO_W + xb * 16 + l16 + s) * CKP + kk);
+          if (SY == 1 || hr % SY < KR)
+            px[hr][xb] = *reinterpret_cast<const half8 *>(sIn + ((wv * RPW * SY + hr) * HALO_W + (xb * 16 + l16) * SX + s) * CKP + kk);
 #pragma unroll
       for (int r = 0; r < KR; ++r) {
         half8 wf[KB];
@@ -767,7 +786,7 @@ mma_chunk(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, int wv, i
           for (int j = 0; j < RPW; ++j)
 #pragma unroll
             for (int xb = 0; xb < XB; ++xb)
-              acc.v[kb][j][xb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[kb], px[j + r][xb], acc.v[kb][j][xb], 0, 0, 0);
+              acc.v[kb][j][xb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf[kb], px[j * SY + r][xb], acc.v[kb][j][xb], 0, 0, 0);
       }
     }
   }

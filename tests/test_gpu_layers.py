@@ -362,3 +362,65 @@ def test_timing_table_runs_in_place_candidates(tmp_path):
     got = dx.Module.load(dx.compile_model(m, assume={"H": 48, "W": 64}, conv_config="w4r2k16", db=db)).instance(H=48, W=64).infer(x)[0]
     ref = dx.Module.compile(m, conv_config="w4r2k16", features={"implicit_concat": False}).instance(H=48, W=64).infer(x)[0]
     assert_bits_equal(got, ref, "table-driven schedule")
+
+
+GEOMETRY_CASES = [  # (R, S, (pad_y, pad_x), (stride_y, stride_x))
+    (3, 3, (0, 0), (1, 1)),   # "valid"
+    (3, 3, (1, 1), (2, 2)),   # the usual strided downsampling
+    (3, 3, (0, 0), (2, 2)),
+    (2, 2, (0, 0), (2, 2)),   # even filter, patch embedding style
+    (4, 4, (1, 1), (2, 2)),
+    (1, 1, (0, 0), (2, 2)),   # stride larger than the filter: halo rows and columns nobody reads
+    (5, 3, (2, 0), (1, 2)),   # everything different in y and x
+    (3, 3, (2, 2), (1, 1)),   # more padding than "same": the output is larger than the input
+    (2, 3, (1, 1), (1, 1)),   # even rows
+    (7, 7, (3, 3), (4, 4)),
+    (3, 3, (1, 1), (3, 1)),
+]
+
+
+@pytest.mark.parametrize("config", [None, "w4r2k16", "s8r2k16", "m4r2k32x2", "p8r2k16", "t16r1k16", "p4r1k32", "q4r2k32x2", "m2r1k32x1n", "w2r2k16n"])
+@pytest.mark.parametrize("R,S,pad,stride", GEOMETRY_CASES)
+def test_conv_padding_and_stride(oracle, config, R, S, pad, stride):
+    """Filter extents 1..7 (even ones too), any zero padding, strides up to 4: out[y, x] reads in[y*sy + r - py, x*sx + s - px]."""
+    rng = np.random.default_rng(R * 100 + S * 10 + pad[0] + stride[1])
+    H, W, C, K = 45, 70, 24, 40
+    x = rng.standard_normal((H, W, C)).astype(np.float16)
+    m = dx.Model()
+    t = m.relu(m.conv2d(m.input("input", "W", "H", C), he_weights(rng, K, C, R, S), small_bias(rng, K), stride=stride, padding=pad))
+    m.output(t)
+    try:
+        mod = dx.Module.compile(m, conv_config=config)
+    except dx.DenoxHipError as e:
+        assert e.status == 5 and config is not None
+        pytest.skip(str(e))
+    assert mod.runtime_model.dispatch_count == 1
+    inst = mod.instance(H=H, W=W)
+    got = inst.infer(x)[0]
+    want = oracle.run_graph(m.to_ops({"H": H, "W": W}), {"input": x}, "fp32")[t.name]
+    assert got.shape == want.shape == ((H + 2 * pad[0] - R) // stride[0] + 1, (W + 2 * pad[1] - S) // stride[1] + 1, K)
+    assert_conv_close(got, want, f"conv {R}x{S} pad {pad} stride {stride} {config}")
+
+
+@pytest.mark.parametrize("config", [None, "p8r2k16", "m4r2k32x2"])
+def test_strided_conv_with_fused_neighbours(oracle, config):
+    """A stride-2 valid conv between a fused upsample + concat in front and a fused ReLU + 2x2 max pool behind, odd
+    extents everywhere, channel counts that are not multiples of 8."""
+    rng = np.random.default_rng(5)
+    H, W = 38, 54
+    lo = rng.standard_normal((H // 2, W // 2, 16)).astype(np.float16)
+    x = rng.standard_normal((H, W, 9)).astype(np.float16)
+    m = dx.Model()
+    t = m.concat(m.upsample(m.input("lo", m.sym("W") // 2, m.sym("H") // 2, 16)), m.input("x", "W", "H", 9))
+    t = m.pool(m.relu(m.conv2d(t, he_weights(rng, 19, 25), small_bias(rng, 19), stride=(2, 2), padding=(0, 0))))
+    m.output(t)
+    try:
+        mod = dx.Module.compile(m, conv_config=config)
+    except dx.DenoxHipError as e:
+        assert e.status == 5 and config is not None
+        pytest.skip(str(e))
+    assert mod.runtime_model.dispatch_count == 1
+    got = mod.instance(H=H, W=W).infer(lo, x)[0]
+    want = oracle.run_graph(m.to_ops({"H": H, "W": W}), {"lo": lo, "x": x}, "fp32")[t.name]
+    assert got.shape == want.shape == (9, 13, 19)
+    assert_conv_close(got, want, f"strided conv with fused neighbours {config}")

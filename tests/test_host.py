@@ -122,7 +122,7 @@ def test_oidn_unet_schedule_dispatch_geometry_covers_every_pixel():
 def test_missing_kernel_is_reported():
     m = dx.Model()
     x = m.input("input", "W", "H", 8)
-    m.output(m.conv2d(x, np.zeros((8, 8, 3, 3), np.float16), stride=(2, 2)))  # strided convolutions have no kernel
+    m.output(m.conv2d(x, np.zeros((8, 8, 3, 3), np.float16), dilation=(2, 2)))  # dilated convolutions have no kernel
     with pytest.raises(dx.DenoxHipError) as e:
         dx.compile_model(m)
     assert e.value.status == 5 and "no kernel implements" in str(e.value)

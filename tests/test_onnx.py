@@ -168,8 +168,14 @@ def test_one_by_one_and_five_by_five_convs_import():
              node("Conv", ["a", "w5"], ["y"], attr_ints("kernel_shape", [5, 5]), attr_ints("pads", [2, 2, 2, 2]))]
     onnx = model(nodes, [value_info("x", (1, 8, "H", "W"))], [value_info("y", (1, 8, "H", "W"))], [tensor("w1", w1), tensor("w5", w5)])
     assert dispatch_names(dx.compile_model(dx.Model.from_onnx(onnx)), H=9, W=9) == ["conv1x1", "conv5x5"]
-    # a 5x5 filter without padding changes the extent: no kernel for that
-    nodes[1] = node("Conv", ["a", "w5"], ["y"], attr_ints("kernel_shape", [5, 5]))
+    # a 5x5 filter without padding and with a stride: the extents follow (H - 5) // 2 + 1
+    nodes[1] = node("Conv", ["a", "w5"], ["y"], attr_ints("kernel_shape", [5, 5]), attr_ints("strides", [2, 2]))
+    onnx = model(nodes, [value_info("x", (1, 8, "H", "W"))], [value_info("y", (1, 8, "h", "w"))], [tensor("w1", w1), tensor("w5", w5)])
+    d = dx.describe(dx.compile_model(dx.Model.from_onnx(onnx)), H=20, W=31)
+    out = d["tensors"][d["outputs"][0]]
+    assert (out["height"], out["width"], out["channels"]) == (8, 14, 8) and "SY=2" in d["dispatches"][1]["debug_info"]
+    # a dilated filter has no kernel
+    nodes[1] = node("Conv", ["a", "w5"], ["y"], attr_ints("kernel_shape", [5, 5]), attr_ints("dilations", [2, 2]))
     onnx = model(nodes, [value_info("x", (1, 8, "H", "W"))], [value_info("y", (1, 8, "h", "w"))], [tensor("w1", w1), tensor("w5", w5)])
     with pytest.raises(dx.DenoxHipError) as e:
         dx.compile_model(dx.Model.from_onnx(onnx))
