@@ -547,6 +547,47 @@ struct Importer {
     setHost(n, std::move(h));
   }
 
+  // Clip(X, [min], [max]) on a host tensor (details/ops/clip.cpp of the reference handles host tensors only, too);
+  // before opset 11 the bounds are the attributes `min` / `max`.
+  void opClip(const Node &n) {
+    HostTensor h = host(n, 0);
+    auto bound = [&](size_t input, const char *attr, bool &present) -> HostTensor {
+      HostTensor b;
+      present = false;
+      if (has(n, input)) {
+        b = host(n, input);
+        if (b.count() != 1) bad("Clip '" + n.name + "': bounds must be scalars");
+        present = true;
+      } else if (const Attr *a = n.attr(attr)) {
+        b.isFloat = true;
+        b.fv = {static_cast<double>(a->f)};
+        present = true;
+      }
+      return b;
+    };
+    bool hasLo = false, hasHi = false;
+    HostTensor lo = bound(1, "min", hasLo), hi = bound(2, "max", hasHi);
+    if (h.isFloat) {
+      if (hasLo) lo = toFloat(n, lo);
+      if (hasHi) hi = toFloat(n, hi);
+      for (double &v : h.fv) {
+        if (hasLo) v = std::max(v, lo.fv[0]);
+        if (hasHi) v = std::min(v, hi.fv[0]);
+      }
+    } else {
+      auto asInt = [&](const HostTensor &b) -> Sym {
+        if (!b.isFloat) return b.iv[0];
+        if (b.fv[0] != std::floor(b.fv[0]) || std::fabs(b.fv[0]) > 9e15) unsupported("Clip '" + n.name + "': fractional bound on an integer tensor");
+        return Sym::Const(static_cast<int64_t>(b.fv[0]));
+      };
+      for (Sym &s : h.iv) {
+        if (hasLo) s = sg.max(s, asInt(lo));
+        if (hasHi) s = sg.min(s, asInt(hi));
+      }
+    }
+    setHost(n, std::move(h));
+  }
+
   void opConstant(const Node &n) {
     HostTensor h;
     if (const Attr *a = n.attr("value")) {
@@ -1052,6 +1093,7 @@ struct Importer {
     else if (op == "Concat") opConcat(n);
     else if (op == "Identity") values[n.out[0]] = get(n, 0);
     else if (op == "Add" || op == "Sub" || op == "Mul" || op == "Div" || op == "Mod" || op == "Min" || op == "Max" || op == "Pow") binary(n);
+    else if (op == "Clip") opClip(n);
     else if (op == "Neg" || op == "Abs" || op == "Floor" || op == "Ceil" || op == "Round" || op == "Sqrt" || op == "Reciprocal" || op == "Sign") unary(n);
     else if (op == "Conv") opConv(n);
     else if (op == "Relu") setDevice(n, model.activation(device(n, 0), compiler::ActivationFunction::ReLU, 0.0f));

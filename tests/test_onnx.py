@@ -152,6 +152,25 @@ def test_integer_mod_takes_the_sign_of_the_divisor():
     assert out["width"] == 10
 
 
+def test_clip_on_shape_arithmetic():
+    # crop offset = Clip(W - 20, 0, 3): 0 for narrow images, 3 for wide ones, the symbolic value in between
+    c = lambda name, arr: node("Constant", [], [name], attr_tensor("value", arr), name=name)
+    nodes = [node("Shape", ["c"], ["shp"]), c("i3", np.array([3], np.int64)), node("Gather", ["shp", "i3"], ["w"], attr_int("axis", 0)),
+             c("k20", np.array([20], np.int64)), node("Sub", ["w", "k20"], ["d"]),
+             c("lo", np.array(0, np.int64)), c("hi", np.array(3, np.int64)), node("Clip", ["d", "lo", "hi"], ["st"]),
+             c("en", np.array([np.iinfo(np.int64).max], np.int64)), c("ax", np.array([3], np.int64)), node("Slice", ["c", "st", "en", "ax"], ["y"])]
+    blob = dx.compile_model(dx.Model.from_onnx(conv_model(nodes, "y", (1, 8, "h", "w"))))
+    for W, want in ((12, 12), (21, 20), (22, 20), (40, 37)):
+        out = [t for t in dx.describe(blob, H=9, W=W)["tensors"] if t.get("name") == "y"][0]
+        assert out["width"] == want, W
+    # only an upper bound (the lower one omitted with an empty name), on constants
+    nodes = [c("a", np.array([7], np.int64)), c("hi", np.array(2, np.int64)), node("Clip", ["a", "", "hi"], ["st"]),
+             c("en", np.array([np.iinfo(np.int64).max], np.int64)), c("ax", np.array([2], np.int64)), node("Slice", ["c", "st", "en", "ax"], ["y"])]
+    blob = dx.compile_model(dx.Model.from_onnx(conv_model(nodes, "y", (1, 8, "h", "w"))))
+    out = [t for t in dx.describe(blob, H=9, W=12)["tensors"] if t.get("name") == "y"][0]
+    assert out["height"] == 7
+
+
 @pytest.mark.parametrize("opset,scales_at", [(10, 1), (13, 2)])
 def test_resize_scales_input_position_follows_the_opset(opset, scales_at):
     ins = ["c", "sc"] if scales_at == 1 else ["c", "", "sc"]
