@@ -73,3 +73,57 @@ def one_case(oracle, seed):
 def test_random_fused_conv_graphs(oracle, block):
     for seed in range(block * 25, block * 25 + 25):
         one_case(oracle, seed)
+
+
+GEOMETRY_CONFIGS = [None, None, "w4r2k16", "w4r1k32", "w2r2kfn", "p8r1k16", "p4r2k32n", "m4r2k32x2", "m4r2kfx1n", "q4r2k32x1n", "t8r1k16", "w2r1k16n", "m2r1k32x1n", "w2r2k16n"]
+
+
+def one_geometry_case(oracle, seed):
+    """A conv with a random filter extent, padding and stride; half of the time twice, concatenated (each branch then
+    stores straight into the concat's tensor), with a pool, a crop or another conv behind."""
+    rng = np.random.default_rng(10_000 + seed)
+    H, W = int(rng.integers(6, 41)), int(rng.integers(6, 61))
+    C, K0, K1 = (int(rng.choice(CHANNELS[:14])) for _ in range(3))
+    R, S = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+    py, px = int(rng.integers(0, 4)), int(rng.integers(0, 4))
+    sy, sx = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+    Ho, Wo = (H + 2 * py - R) // sy + 1, (W + 2 * px - S) // sx + 1
+    two, act, tail = bool(rng.integers(0, 2)), ["none", "relu", "leaky"][int(rng.integers(0, 3))], ["none", "pool", "crop", "conv"][int(rng.integers(0, 4))]
+    config = GEOMETRY_CONFIGS[int(rng.integers(0, len(GEOMETRY_CONFIGS)))]
+    feats = {k: bool(rng.integers(0, 4)) for k in ("conv_relu_fusion", "concat_conv_fusion", "pool_fusion", "slice_fusion", "implicit_concat")}
+    print(f"geometry seed={seed} H={H} W={W} C={C} K={K0},{K1 if two else 0} filter={R}x{S} pad={(py, px)} stride={(sy, sx)} act={act} tail={tail} config={config} feats={feats}", flush=True)
+    assert Ho >= 1 and Wo >= 1
+    m = dx.Model()
+    x = m.input("a", "W", "H", C)
+    feeds = {"a": rng.standard_normal((H, W, C)).astype(np.float16)}
+
+    def branch(K):
+        y = m.conv2d(x, he_weights(rng, K, C, R, S), small_bias(rng, K) if rng.integers(0, 4) else None, stride=(sy, sx), padding=(py, px))
+        return m.relu(y) if act == "relu" else m.activation(y, "leaky_relu", 0.125) if act == "leaky" else y
+    t = branch(K0)
+    Kt = K0
+    if two:
+        t = m.concat(t, branch(K1))
+        Kt += K1
+    if tail == "pool" and Ho >= 2 and Wo >= 2:
+        t = m.pool(t)
+    elif tail == "crop" and Ho >= 2 and Wo >= 2:
+        l, tp = int(rng.integers(0, Wo // 2)), int(rng.integers(0, Ho // 2))
+        t = m.slice(t, l, int(rng.integers(l + 1, Wo + 1)), tp, int(rng.integers(tp + 1, Ho + 1)))
+    elif tail == "conv":
+        t = m.conv2d(t, he_weights(rng, 8, Kt), small_bias(rng, 8))
+    m.output(t)
+    try:
+        mod = dx.Module.compile(m, features=feats, conv_config=config)
+    except dx.DenoxHipError as e:
+        assert e.status == 5, str(e)
+        mod = dx.Module.compile(m, features=feats)
+    got = mod.instance(H=H, W=W).infer(feeds["a"])[0]
+    want = oracle.run_graph(m.to_ops({"H": H, "W": W}), feeds, "fp32")[t.name]
+    assert_conv_close(got, want, f"geometry seed {seed}")
+
+
+@pytest.mark.parametrize("block", range(6))
+def test_random_conv_geometry(oracle, block):
+    for seed in range(block * 25, block * 25 + 25):
+        one_geometry_case(oracle, seed)
