@@ -521,7 +521,7 @@ Sym rowGrid(SymGraph &sym, Sym w, unsigned vectorsPerPixel) {
 class SingleOpShader : public IShader {
 public:
   SingleOpShader(const hip::HipCompiler *c, OpKind kind) : m_compiler(c), m_kind(kind) {}
-  std::vector<Match> matchAll(const Model &model, const CompileOptions &) const override {
+  std::vector<Match> matchAll(const Model &model, const CompileOptions &opt) const override {
     std::vector<Match> out;
     for (size_t i = 0; i < model.ops().size(); ++i) {
       const Op &op = model.ops()[i];
@@ -530,9 +530,37 @@ public:
       m.ops = {static_cast<int>(i)};
       m.inputs = op.inputs;
       m.output = op.output;
+      // the same dispatch storing straight into the channel range of the concat that consumes its result
+      if (m_kind != OpKind::Concat && opt.features.enableImplicitConcat && concatViewOf(model, m.output).valid) {
+        Match v = m;
+        v.outputVariant = 1;
+        out.push_back(std::move(v));
+      }
       out.push_back(std::move(m));
     }
     return out;
+  }
+
+  // Where a single-source dispatch stores: vector width (16-byte stores need an aligned channel range), the kernel
+  // definition and name suffix, and the output binding with the bytes it may touch.
+  struct Placement { ConcatView view; unsigned vec; std::string suffix; };
+  static Placement placementOf(const Model &model, const Match &m, unsigned channels) {
+    Placement p;
+    p.view = m.outputVariant ? concatViewOf(model, m.output) : ConcatView{};
+    if (m.outputVariant && !p.view.valid) fail(Status::Internal, "match writes into a concat that does not exist");
+    const bool aligned = !p.view.valid || (p.view.pitch % 8 == 0 && p.view.channelOffset % 8 == 0);
+    p.vec = channels % 8 == 0 && aligned ? 8 : 1;
+    if (p.view.valid) p.suffix = "_into" + std::to_string(p.view.pitch);
+    return p;
+  }
+  static void defineOutput(hip::HipCompilerInstance &k, const Placement &p) {
+    if (p.view.valid) k.define("OPITCH", p.view.pitch);
+  }
+  static void bindOutput(ComputeDispatchBuilder &d, SymGraph &sym, const Model &model, const Match &m, const Placement &p) {
+    if (!p.view.valid) { d.addBinding(dnx::Access::WriteOnly, m.output); return; }
+    const TensorNode &o = model.tensors()[m.output];
+    d.addBinding(dnx::Access::WriteOnly, m.output,
+                 sym.sub(sym.mul(sym.mul(o.width, o.height), static_cast<int64_t>(p.view.pitch) * 2), static_cast<int64_t>(p.view.pitch - o.channels) * 2));
   }
   std::vector<unsigned> acceptMatch(const Model &, const Match &, const CompileOptions &) const override { return {0}; }
   virtual bool supports(const Op &) const { return true; }
@@ -551,16 +579,18 @@ public:
   void implement(OpImpl &impl, const Model &model, const Match &m, unsigned, SymGraph &sym, const CompileOptions &) const override {
     const Op &op = model.ops()[m.ops[0]];
     const TensorNode &in = model.tensors()[m.inputs[0]], &out = model.tensors()[m.output];
-    const unsigned vec = in.channels % 8 == 0 ? 8 : 1;
+    const Placement place = placementOf(model, m, in.channels);
+    const unsigned vec = place.vec;
     auto k = m_compiler->read("pool.hip");
     k.define("CH", in.channels); k.define("KX", op.kernelX); k.define("KY", op.kernelY); k.define("VEC", vec);
-    const std::string entry = "pool_max_c" + std::to_string(in.channels) + "v" + std::to_string(vec);
+    defineOutput(k, place);
+    const std::string entry = "pool_max_c" + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
     k.define("KERNEL_NAME", entry);
     auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, in.channels / vec), out.height, Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
-    d.addBinding(dnx::Access::WriteOnly, m.output);
+    bindOutput(d, sym, model, m, place);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
-    d.setName("maxpool"); d.setOperation("maxpool"); d.setConfig("vec" + std::to_string(vec));
+    d.setName(std::string("maxpool") + (place.view.valid ? "+concat" : "")); d.setOperation("maxpool"); d.setConfig("vec" + std::to_string(vec));
     d.setMemoryReads(bytesOf(sym, in)); d.setMemoryWrites(bytesOf(sym, out)); d.setFlops(Sym::Const(0));
   }
 };
@@ -572,16 +602,18 @@ public:
   void implement(OpImpl &impl, const Model &model, const Match &m, unsigned, SymGraph &sym, const CompileOptions &) const override {
     const Op &op = model.ops()[m.ops[0]];
     const TensorNode &in = model.tensors()[m.inputs[0]], &out = model.tensors()[m.output];
-    const unsigned vec = in.channels % 8 == 0 ? 8 : 1;
+    const Placement place = placementOf(model, m, in.channels);
+    const unsigned vec = place.vec;
     auto k = m_compiler->read("upsample.hip");
     k.define("CH", in.channels); k.define("SCALE", op.scale); k.define("VEC", vec);
-    const std::string entry = "upsample_c" + std::to_string(in.channels) + "v" + std::to_string(vec);
+    defineOutput(k, place);
+    const std::string entry = "upsample_c" + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
     k.define("KERNEL_NAME", entry);
     auto d = impl.registerDispatch(k, entry, rowGrid(sym, in.width, in.channels / vec), in.height, Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
-    d.addBinding(dnx::Access::WriteOnly, m.output);
+    bindOutput(d, sym, model, m, place);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
-    d.setName("upsample"); d.setOperation("upsample"); d.setConfig("vec" + std::to_string(vec));
+    d.setName(std::string("upsample") + (place.view.valid ? "+concat" : "")); d.setOperation("upsample"); d.setConfig("vec" + std::to_string(vec));
     d.setMemoryReads(bytesOf(sym, in)); d.setMemoryWrites(bytesOf(sym, out)); d.setFlops(Sym::Const(0));
   }
 };
@@ -647,18 +679,20 @@ public:
   void implement(OpImpl &impl, const Model &model, const Match &m, unsigned, SymGraph &sym, const CompileOptions &) const override {
     const Op &op = model.ops()[m.ops[0]];
     const TensorNode &in = model.tensors()[m.inputs[0]];
-    const unsigned vec = in.channels % 8 == 0 ? 8 : 1;
+    const Placement place = placementOf(model, m, in.channels);
+    const unsigned vec = place.vec;
     auto k = m_compiler->read("activation.hip");
     k.define("CH", in.channels); k.define("VEC", vec); k.define("ACT", op.func == ActivationFunction::ReLU ? 1 : 2);
     if (op.func == ActivationFunction::LeakyReLU) k.define("ALPHA", fmtFloat(op.alpha));
-    const std::string entry = std::string(op.func == ActivationFunction::ReLU ? "relu_c" : "leaky_relu_c") + std::to_string(in.channels) + "v" + std::to_string(vec);
+    defineOutput(k, place);
+    const std::string entry = std::string(op.func == ActivationFunction::ReLU ? "relu_c" : "leaky_relu_c") + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
     k.define("KERNEL_NAME", entry);
     auto d = impl.registerDispatch(k, entry, rowGrid(sym, in.width, in.channels / vec), in.height, Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
-    d.addBinding(dnx::Access::WriteOnly, m.output);
+    bindOutput(d, sym, model, m, place);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
     const char *nm = op.func == ActivationFunction::ReLU ? "relu" : "leaky_relu";
-    d.setName(nm); d.setOperation(nm); d.setConfig("vec" + std::to_string(vec));
+    d.setName(std::string(nm) + (place.view.valid ? "+concat" : "")); d.setOperation(nm); d.setConfig("vec" + std::to_string(vec));
     d.setMemoryReads(bytesOf(sym, in)); d.setMemoryWrites(bytesOf(sym, in));
     d.setFlops(sym.mul(sym.mul(in.width, in.height), static_cast<int64_t>(in.channels))); // one FLOP per element, as the reference counts it
   }
@@ -671,17 +705,19 @@ public:
   void implement(OpImpl &impl, const Model &model, const Match &m, unsigned, SymGraph &sym, const CompileOptions &) const override {
     const Op &op = model.ops()[m.ops[0]];
     const TensorNode &in = model.tensors()[m.inputs[0]], &out = model.tensors()[m.output];
-    const unsigned vec = in.channels % 8 == 0 ? 8 : 1;
+    const Placement place = placementOf(model, m, in.channels);
+    const unsigned vec = place.vec;
     auto k = m_compiler->read("pad.hip");
     k.define("CH", in.channels); k.define("VEC", vec);
-    const std::string entry = "memory_pad_c" + std::to_string(in.channels) + "v" + std::to_string(vec);
+    defineOutput(k, place);
+    const std::string entry = "memory_pad_c" + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
     k.define("KERNEL_NAME", entry);
     auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, in.channels / vec), out.height, Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
-    d.addBinding(dnx::Access::WriteOnly, m.output);
+    bindOutput(d, sym, model, m, place);
     d.addPushConstant(out.width); d.addPushConstant(out.height);
     d.addPushConstant(op.left); d.addPushConstant(op.right); d.addPushConstant(op.top); d.addPushConstant(op.bottom);
-    d.setName("pad"); d.setOperation("pad"); d.setConfig("vec" + std::to_string(vec));
+    d.setName(std::string("pad") + (place.view.valid ? "+concat" : "")); d.setOperation("pad"); d.setConfig("vec" + std::to_string(vec));
     d.setMemoryReads(bytesOf(sym, in)); d.setMemoryWrites(bytesOf(sym, out)); d.setFlops(Sym::Const(0));
   }
 };
@@ -693,18 +729,20 @@ public:
   void implement(OpImpl &impl, const Model &model, const Match &m, unsigned, SymGraph &sym, const CompileOptions &) const override {
     const Op &op = model.ops()[m.ops[0]];
     const TensorNode &in = model.tensors()[m.inputs[0]], &out = model.tensors()[m.output];
-    const unsigned vec = in.channels % 8 == 0 ? 8 : 1;
+    const Placement place = placementOf(model, m, in.channels);
+    const unsigned vec = place.vec;
     auto k = m_compiler->read("slice.hip");
     k.define("CH", in.channels); k.define("VEC", vec);
-    const std::string entry = "memory_slice_c" + std::to_string(in.channels) + "v" + std::to_string(vec);
+    defineOutput(k, place);
+    const std::string entry = "memory_slice_c" + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
     k.define("KERNEL_NAME", entry);
     auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, in.channels / vec), out.height, Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
-    d.addBinding(dnx::Access::WriteOnly, m.output);
+    bindOutput(d, sym, model, m, place);
     d.addPushConstant(op.top); d.addPushConstant(op.left);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
     d.addPushConstant(out.width); d.addPushConstant(out.height);
-    d.setName("slice"); d.setOperation("slice"); d.setConfig("vec" + std::to_string(vec));
+    d.setName(std::string("slice") + (place.view.valid ? "+concat" : "")); d.setOperation("slice"); d.setConfig("vec" + std::to_string(vec));
     d.setMemoryReads(bytesOf(sym, out)); d.setMemoryWrites(bytesOf(sym, out)); d.setFlops(Sym::Const(0));
   }
 };

@@ -24,13 +24,15 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
   const unsigned i = DNX_ROW_INDEX();
   if (i >= pc.W * CV) return;
   const size_t idx = ((size_t)DNX_BID_Y * pc.W * CV + i) * VEC;
+  const unsigned w = i / CV, cv = i - w * CV;
+  const size_t odx = OPITCH == CH ? idx : ((size_t)DNX_BID_Y * pc.W + w) * OPITCH + cv * VEC;
   const vec_t v = ldv(IN + idx);
 #if VEC == 8
   half8 a = __builtin_bit_cast(half8, v);
 #pragma unroll
   for (int e = 0; e < 8; ++e) a[e] = act1(a[e]);
-  stv(OUT + idx, __builtin_bit_cast(uint4v, a));
+  stv(OUT + odx, __builtin_bit_cast(uint4v, a));
 #else
-  stv(OUT + idx, __builtin_bit_cast(ushort_t, act1(__builtin_bit_cast(_Float16, v))));
+  stv(OUT + odx, __builtin_bit_cast(ushort_t, act1(__builtin_bit_cast(_Float16, v))));
 #endif
 }

@@ -13,6 +13,12 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 #ifndef WG
 #define WG 256
 #endif
+// Channels between consecutive OUTPUT pixels of the single-source kernels (pool, upsample, activation, pad, slice):
+// their own channel count CH, or the channel count of a wider tensor when the result is stored straight into its
+// channel range of a concat's output (OUT then points at the range's first channel).
+#ifndef OPITCH
+#define OPITCH CH
+#endif
 
 #if VEC == 8
 typedef uint4v vec_t;

@@ -18,5 +18,5 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
   const int IN_H = (int)(pc.OUT_H - pc.PAD_T - pc.PAD_B);
   int hi = ho - (int)pc.PAD_T; hi = hi < 0 ? 0 : (hi > IN_H - 1 ? IN_H - 1 : hi);
   int wi = (int)wo - (int)pc.PAD_L; wi = wi < 0 ? 0 : (wi > IN_W - 1 ? IN_W - 1 : wi);
-  stv(OUT + ((size_t)ho * pc.OUT_W + wo) * CH + cv * VEC, ldv(IN + ((size_t)hi * IN_W + wi) * CH + cv * VEC));
+  stv(OUT + ((size_t)ho * pc.OUT_W + wo) * OPITCH + cv * VEC, ldv(IN + ((size_t)hi * IN_W + wi) * CH + cv * VEC));
 }

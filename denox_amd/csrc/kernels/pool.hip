@@ -33,5 +33,5 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
       acc = max_keep_first(acc, v);
 #endif
     }
-  stv(OUT + ((size_t)oh * W2 + ow) * CH + cv * VEC, acc);
+  stv(OUT + ((size_t)oh * W2 + ow) * OPITCH + cv * VEC, acc);
 }

@@ -14,6 +14,6 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
   const unsigned i = DNX_ROW_INDEX();
   if (i >= pc.OUT_W * CV) return;
   const unsigned w = i / CV, cv = i - w * CV;
-  stv(OUT + ((size_t)h * pc.OUT_W + w) * CH + cv * VEC,
+  stv(OUT + ((size_t)h * pc.OUT_W + w) * OPITCH + cv * VEC,
       ldv(IN + ((size_t)(h + pc.IN_TOP) * pc.IN_W + (w + pc.IN_LEFT)) * CH + cv * VEC));
 }

@@ -21,5 +21,5 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
   for (int r = 0; r < SCALE; ++r)
 #pragma unroll
     for (int s = 0; s < SCALE; ++s)
-      stv(OUT + (((size_t)h * SCALE + r) * W2 + (size_t)w * SCALE + s) * CH + cv * VEC, v);
+      stv(OUT + (((size_t)h * SCALE + r) * W2 + (size_t)w * SCALE + s) * OPITCH + cv * VEC, v);
 }

@@ -424,3 +424,36 @@ def test_strided_conv_with_fused_neighbours(oracle, config):
     want = oracle.run_graph(m.to_ops({"H": H, "W": W}), {"lo": lo, "x": x}, "fp32")[t.name]
     assert got.shape == want.shape == (9, 13, 19)
     assert_conv_close(got, want, f"strided conv with fused neighbours {config}")
+
+
+@pytest.mark.parametrize("C0,C1", [(8, 16), (16, 8), (3, 9), (8, 9), (24, 40)])
+def test_bandwidth_kernels_store_in_place(oracle, C0, C1):
+    """Pool, upsample, activation, pad and slice as producers of concat sources: each stores into its channel range of
+    the concat's tensor (16-byte stores when the range is aligned, element stores otherwise); bit-exact against the
+    oracle and against the schedule with copies."""
+    rng = np.random.default_rng(C0 * 7 + C1)
+    H, W = 22, 36
+    feeds = {"a": rng.standard_normal((H // 2, W // 2, C0)), "b": rng.standard_normal((H, W, C1)), "c": rng.standard_normal((2 * H, 2 * W, C0)),
+             "d": rng.standard_normal((H - 3, W - 5, C1)), "e": rng.standard_normal((H + 4, W + 6, C0))}
+    feeds = {k: v.astype(np.float16) for k, v in feeds.items()}
+    m = dx.Model()
+    a = m.input("a", m.sym("W") // 2, m.sym("H") // 2, C0)
+    b = m.input("b", "W", "H", C1)
+    c = m.input("c", m.sym("W") * 2, m.sym("H") * 2, C0)
+    d = m.input("d", m.sym("W") - 5, m.sym("H") - 3, C1)
+    e = m.input("e", m.sym("W") + 6, m.sym("H") + 4, C0)
+    o1 = m.concat(m.upsample(a), m.relu(b))
+    o2 = m.concat(m.pool(c), m.pad(d, 2, 3, 1, 2))
+    o3 = m.concat(m.slice(e, 1, m.sym("W") + 1, 3, m.sym("H") + 3), m.activation(b, "leaky_relu", 0.25))
+    for t in (o1, o2, o3):
+        m.output(t)
+    mod = dx.Module.compile(m)
+    ref = dx.Module.compile(m, features={"implicit_concat": False})
+    assert mod.runtime_model.dispatch_count == 6 and ref.runtime_model.dispatch_count == 12
+    order = ["a", "b", "c", "d", "e"]
+    got = mod.instance(H=H, W=W).infer(*[feeds[k] for k in order])
+    cop = ref.instance(H=H, W=W).infer(*[feeds[k] for k in order])
+    want = oracle.run_graph(m.to_ops({"H": H, "W": W}), feeds, "f16")
+    for g, r, t in zip(got, cop, (o1, o2, o3)):
+        assert_bits_equal(g, r, "in place against copied")
+        assert_bits_equal(g, want[t.name], "in place against the oracle")

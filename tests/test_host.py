@@ -80,9 +80,13 @@ def test_tiny_unet_schedule_and_geometry():
 def test_fusion_switches_change_the_schedule():
     m, _ = networks.build("tiny_unet")
     none = dict(conv_relu_fusion=False, concat_conv_fusion=False, upsample_fusion=False, pool_fusion=False)
-    names = _dispatch_names(dx.compile_model(m, features=none), H=64, W=64)
+    names = _dispatch_names(dx.compile_model(m, features=dict(none, implicit_concat=False)), H=64, W=64)
     assert names == ["conv3x3", "relu", "maxpool", "conv3x3", "relu", "upsample", "concat-copy-src0", "concat-copy-src1",
                      "conv3x3", "relu", "conv3x3"]
+    # the upsampled tensor is read by the concat only: the upsample stores straight into the concat's tensor; the skip
+    # tensor is also read by the pool and keeps its copy
+    names = _dispatch_names(dx.compile_model(m, features=none), H=64, W=64)
+    assert names == ["conv3x3", "relu", "maxpool", "conv3x3", "relu", "upsample+concat", "concat-copy-src1", "conv3x3", "relu", "conv3x3"]
     names = _dispatch_names(dx.compile_model(m, features=dict(upsample_fusion=False)), H=64, W=64)
     assert names == ["conv3x3+relu", "maxpool", "conv3x3+relu", "upsample", "concat+conv3x3+relu", "conv3x3"]
 
@@ -344,7 +348,7 @@ def test_measured_latencies_drive_the_selection(tmp_path):
         for _ in range(3):
             db.add_sample(i, lat)
     names = _dispatch_names(dx.compile_model(m, assume={"H": 64, "W": 64}, conv_config="w4r2k16", db=db), H=64, W=64)
-    assert "upsample" in names and "concat-copy-src0" in names and not any("concat+" in n for n in names)
+    assert "upsample+concat" in names and "concat-copy-src1" in names and not any(n.startswith("concat+") for n in names)
     assert "measured" in dx.last_compile_report()
     # without a table the roofline estimate prefers the fused kernel
     names = _dispatch_names(dx.compile_model(m, assume={"H": 64, "W": 64}, conv_config="w4r2k16"), H=64, W=64)
