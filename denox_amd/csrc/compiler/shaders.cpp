@@ -128,7 +128,7 @@ bool chooseKT(const ConvConfig &cfgIn, unsigned CA, unsigned CB, unsigned K, con
     if (accRegs + 64 + (cfg.mf == 16 ? kb * 4 : 0) > regBudget) continue;
     const size_t lds = (cfg.resident ? static_cast<size_t>(taps * kb * blk) * (g.CPAD + 8) * 2u + 2u * static_cast<size_t>(haloPix) * ckp * 2u
                                      : (static_cast<size_t>(haloPix) + taps * kb * blk) * ckp * 2u) +
-                       static_cast<size_t>(kb * blk) * 2u; // + the staged bias
+                       static_cast<size_t>(kb * blk) * 4u; // + the staged bias (fp32)
     if (lds > dev.maxComputeSharedMemory) continue;
     {
       // a thread stages at most 64 halo vectors per step (the kernels' bookkeeping is one bit per vector)
@@ -209,7 +209,7 @@ bool chooseFold(const ConvConfig &cfg, unsigned CA, unsigned CB, unsigned K, con
     if (kb * cfg.rpw * 24 + (nva + nvb) * 4 + 64 > regBudget) continue; // accumulators, converted tile, halo registers
     for (unsigned pitchPad : {8u, 0u}) { // the B halo gives up its bank-conflict padding where LDS is short
       const size_t lds = (static_cast<size_t>(4 * kt) * (g.CAP + 8) + (CB ? static_cast<size_t>(9 * kt) * (g.CBP + 8) : 8) + static_cast<size_t>(aPix) * (g.CAP + 8) +
-                          (CB ? static_cast<size_t>(bPix) * (g.CBP + pitchPad) : 8) + kt) * 2u;
+                          (CB ? static_cast<size_t>(bPix) * (g.CBP + pitchPad) : 8) + 2 * kt) * 2u; // the last term: the staged bias, fp32
       if (lds > dev.maxComputeSharedMemory) continue;
       g.KT = kt; g.bpitch = g.CBP + pitchPad; g.ldsBytes = lds;
       g.slots = std::max(1u, dev.computeUnits / (dev.xcdCount * 4 * (blocks / kb)));

@@ -61,7 +61,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     PushConstants pc) {
   __shared__ __attribute__((aligned(16))) _Float16 sIn[HALO_PIX * CKP];
   __shared__ __attribute__((aligned(16))) _Float16 sW[NTAPS * KT * CKP];
-  __shared__ __attribute__((aligned(16))) _Float16 sBias[KT];
+  __shared__ __attribute__((aligned(16))) bias_t sBias[KT];
 #if CB == 0
   const _Float16 *B = nullptr;
 #endif
@@ -80,7 +80,6 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   const int kt = DNX_BID_Z; // output-channel tile
 
   Acc acc;
-  zero_acc(acc);
   stage_bias(sBias, BIAS, kt, tid);
 
   // packed filter: [kt][chunk][tap][KT][len(chunk)]
@@ -105,6 +104,8 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     else
       weights_commit<TAIL>(stW, sW, tid);
     DNX_SYNC();
+    if (chunk == 0)
+      init_acc(acc, sBias, lane); // the staged bias is visible from here on
     if (chunk + 1 < NCHUNK) { // loads for the next step fly during the MFMAs below
       const _Float16 *wnext = wbase + (size_t)NTAPS * KT * (chunk + 1) * CK;
       H::fetch_step(srcs, stIn, map, src, chunk + 1);
@@ -116,5 +117,5 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     mma_step<CKP>(sIn, sW, 0, acc, wv, lane, chunk);
     DNX_SYNC();
   }
-  store_tile(acc, out, sBias, y0, x0, kt, wv, lane, pc);
+  store_tile(acc, out, y0, x0, kt, wv, lane, pc);
 }

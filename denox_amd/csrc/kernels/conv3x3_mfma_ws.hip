@@ -40,7 +40,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     PushConstants pc) {
   __shared__ __attribute__((aligned(16))) _Float16 sW[NTAPS * KT * CPADP];
   __shared__ __attribute__((aligned(16))) _Float16 sIn[2][HALO_PIX * CKP];
-  __shared__ __attribute__((aligned(16))) _Float16 sBias[KT];
+  __shared__ __attribute__((aligned(16))) bias_t sBias[KT];
 #if CB == 0
   const _Float16 *B = nullptr;
 #endif
@@ -134,8 +134,8 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   auto mma = [&](int buf) { mma_step<CPADP>(sIn[buf], sW, cchunk * CK, acc, wv, lane, cchunk); };
   auto post = [&]() { // after this wave's matrix work of a step
     if (++cchunk == NCHUNK) {
-      pack_tile(acc, done, sBias, lane);
-      zero_acc(acc);
+      pack_tile(acc, done);
+      init_acc(acc, sBias, lane);
       dtile = tile;
       dpart = 0;
       pend = tile < last; // false in the spare step
@@ -155,9 +155,9 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   issue(st0);
   __builtin_amdgcn_sched_barrier(0); // keep the two sets in issue order: the waits count loads in flight
   issue(st1);
-  zero_acc(acc);
   stage(st0, 0); // halo 0, by all waves
   DNX_SYNC();
+  init_acc(acc, sBias, lane); // the staged bias is visible from here on
   if (!groupB) {
     do {
       mma(0); DNX_SYNC(); post(); stage(st1, 1); DNX_SYNC();
@@ -172,12 +172,12 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
 #else
   int cchunk = 0, buf = 0;
   auto step = [&](H::Regs &regs) {
-    if (cchunk == 0)
-      zero_acc(acc);
     H::commit_step(regs, sIn[buf], map, cchunk);
     // One barrier per step: buffer `buf` was last read two steps ago, and every wave
     // has passed the barrier of the step in between since then.
     DNX_SYNC();
+    if (cchunk == 0)
+      init_acc(acc, sBias, lane);
     // A portion of the previous tile's stores, in front of this step's loads: when a later step waits for those
     // loads, it counts back over at most these stores, which are old by then.
     if (pend)
@@ -186,7 +186,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     mma_step<CPADP>(sIn[buf], sW, cchunk * CK, acc, wv, lane, cchunk);
     buf ^= 1;
     if (++cchunk == NCHUNK) {
-      pack_tile(acc, done, sBias, lane);
+      pack_tile(acc, done);
       dtile = tile;
       dpart = 0;
       pend = tile < last; // false in the spare step below
@@ -248,12 +248,12 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     Acc acc;
     int cchunk = 0;
     for (int g = 0; g < steps; ++g) {
-      if (cchunk == 0)
-        zero_acc(acc);
       DNX_SYNC();
+      if (cchunk == 0)
+        init_acc(acc, sBias, lane);
       mma_step<CPADP>(sIn[g & 1], sW, cchunk * CK, acc, wv, lane, cchunk);
       if (++cchunk == NCHUNK) {
-        store_tile(acc, out, sBias, tileY(tile), tileX(tile), kt, wv, lane, pc);
+        store_tile(acc, out, tileY(tile), tileX(tile), kt, wv, lane, pc);
         cchunk = 0;
         tile += SLOTS;
       }

@@ -57,7 +57,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   __shared__ __attribute__((aligned(16))) _Float16 sWB[CB > 0 ? 9 * KT * BWP : 8];
   __shared__ __attribute__((aligned(16))) _Float16 sA[AH * AW * APITCH];
   __shared__ __attribute__((aligned(16))) _Float16 sB[CB > 0 ? BH * BW * BPITCH : 8];
-  __shared__ __attribute__((aligned(16))) _Float16 sBias[KT];
+  __shared__ __attribute__((aligned(16))) bias_t sBias[KT];
 #if CB == 0
   const _Float16 *B = nullptr;
 #endif
@@ -207,10 +207,10 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   issueB(tile);
 #endif
   for (; tile < last; tile += SLOTS) {
-    zero_acc(acc);
     // ---- step A: the folded 2x2 taps over the low-resolution source
     commitA();
     DNX_SYNC();
+    init_acc(acc, sBias, lane);
     if (pend) { // the previous tile's stores, in front of this step's loads
       store_packed(done, out, 2 * tileY(dtile) + ca, 2 * tileX(dtile) + cb, kt, wv, lane, pc, 0, 1, 2, 2);
       pend = false;
@@ -268,7 +268,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
       }
     }
 #endif
-    pack_tile(acc, done, sBias, lane);
+    pack_tile(acc, done);
     dtile = tile;
     pend = true;
   }

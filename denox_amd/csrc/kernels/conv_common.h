@@ -133,6 +133,20 @@ __device__ DNX_INLINE uint4v ld16(const _Float16 *p) {
 
 __device__ DNX_INLINE int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
 
+// An LDS address the optimiser must take as it is.  A fragment read is `base that changes per step + per-lane part +
+// compile-time constant`; left alone, the compiler sums the per-lane part and each constant once, outside the step
+// loop (they do not change there), keeps 20-odd registers of such sums and adds the step's base to every one of them
+// again in every step -- one vector add per LDS read, in a loop whose matrix instructions wait for exactly those
+// slots.  With the step's base + per-lane part made opaque, the constants stay what the LDS instructions have a
+// field for: immediate offsets.
+typedef __attribute__((address_space(3))) const _Float16 lds_half_t;
+typedef __attribute__((address_space(3))) const half8 lds_half8_t;
+__device__ DNX_INLINE lds_half_t *lds_opaque(const _Float16 *p) {
+  unsigned a = (unsigned)(size_t)(lds_half_t *)p;
+  __asm__ volatile("" : "+v"(a));
+  return (lds_half_t *)(size_t)a;
+}
+
 // Element offsets of full-resolution pixel (gy, gx) inside A and B.
 __device__ DNX_INLINE void src_offsets(int gy, int gx, const PushConstants &pc, size_t &pa, size_t &pb) {
   const unsigned W = pc.IN_W;
@@ -445,6 +459,30 @@ __device__ DNX_INLINE float apply_act(float v) {
 #endif
 }
 
+// Activation and the one rounding fp32 -> binary16 of an accumulator (the bias is in it already, see init_acc).
+// ReLU commutes with the rounding -- both keep sign and zero -- so it is applied to the rounded values, where one
+// instruction handles two channels; LeakyReLU multiplies and therefore stays in fp32.
+__device__ DNX_INLINE _Float16 finish1(float v) {
+#if ACT == 1
+  return __builtin_fmaxf16((_Float16)v, (_Float16)0.0f);
+#else
+  return (_Float16)apply_act(v);
+#endif
+}
+__device__ DNX_INLINE half8 finish8(const float *v) {
+  half8 h;
+#if ACT == 1
+#pragma unroll
+  for (int i = 0; i < 8; ++i) h[i] = (_Float16)v[i];
+  const half8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  return __builtin_elementwise_max(h, zero);
+#else
+#pragma unroll
+  for (int i = 0; i < 8; ++i) h[i] = (_Float16)apply_act(v[i]);
+  return h;
+#endif
+}
+
 __device__ DNX_INLINE ushort_t dpp_xor1(ushort_t v) {
   // quad_perm [1,0,3,2]: exchange with the neighbouring lane
   return (ushort_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xF, 0xF, true);
@@ -492,12 +530,14 @@ __device__ DNX_INLINE void store16(OutBuf out, bool ok, unsigned pix, const half
   }
 }
 
-// The KT bias values of a workgroup's output channels are staged in LDS once (the global buffer is zero-padded to
-// KOUTP), so that the epilogue waits for no global load.  Visible after the first barrier.
-__device__ DNX_INLINE void stage_bias(_Float16 *sBias, const _Float16 *__restrict__ BIAS, int kt, int tid) {
+// The KT bias values of a workgroup's output channels are staged in LDS once, as fp32 (the global buffer is
+// zero-padded to KOUTP).  Visible after the first barrier: every tile's accumulators start from them (init_acc), as the
+// reference loads the bias straight into its accumulators (direct_conv_cm.comp:175-192), so the epilogue adds nothing.
+typedef float bias_t;
+__device__ DNX_INLINE void stage_bias(bias_t *sBias, const _Float16 *__restrict__ BIAS, int kt, int tid) {
 #if HAS_BIAS
   for (int i = tid; i < KT; i += NT)
-    sBias[i] = BIAS[kt * KT + i];
+    sBias[i] = (float)BIAS[kt * KT + i];
 #endif
 }
 
@@ -515,27 +555,17 @@ struct Packed {
   half8 o[KB][OROWS][2];
 };
 
-// bias, activation, rounding to fp16 and (POOL) the 2x2 maximum
-__device__ DNX_INLINE void pack_tile(const Acc &acc, Packed &pk, const _Float16 *sBias, int lane) {
-  const int hsel = lane >> 5;
+// activation, rounding to fp16 and (POOL) the 2x2 maximum
+__device__ DNX_INLINE void pack_tile(const Acc &acc, Packed &pk) {
 #pragma unroll
   for (int kb = 0; kb < KB; ++kb) {
-    float bias[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-#if HAS_BIAS
-      bias[i] = (float)sBias[kb * 32 + hsel * 16 + i];
-#else
-      bias[i] = 0.0f;
-#endif
-    }
 #if POOL
 #pragma unroll
     for (int j = 0; j < RPW; j += 2) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const _Float16 v0 = (_Float16)apply_act(acc.v[kb][j][i] + bias[i]);
-        const _Float16 v1 = (_Float16)apply_act(acc.v[kb][j + 1][i] + bias[i]);
+        const _Float16 v0 = finish1(acc.v[kb][j][i]);
+        const _Float16 v1 = finish1(acc.v[kb][j + 1][i]);
         const _Float16 n0 = __builtin_bit_cast(_Float16, dpp_xor1(__builtin_bit_cast(ushort_t, v0)));
         const _Float16 n1 = __builtin_bit_cast(_Float16, dpp_xor1(__builtin_bit_cast(ushort_t, v1)));
         // window order (0,0) (0,1) (1,0) (1,1); replace only on strictly greater
@@ -548,10 +578,13 @@ __device__ DNX_INLINE void pack_tile(const Acc &acc, Packed &pk, const _Float16 
     }
 #else
 #pragma unroll
-    for (int j = 0; j < RPW; ++j)
+    for (int j = 0; j < RPW; ++j) {
+      float v[16];
 #pragma unroll
-      for (int i = 0; i < 16; ++i)
-        pk.o[kb][j][i >> 3][i & 7] = (_Float16)apply_act(acc.v[kb][j][i] + bias[i]);
+      for (int i = 0; i < 16; ++i) v[i] = acc.v[kb][j][i];
+      pk.o[kb][j][0] = finish8(v);
+      pk.o[kb][j][1] = finish8(v + 8);
+    }
 #endif
   }
 }
@@ -597,22 +630,23 @@ __device__ DNX_INLINE void
 mma_chunk(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, int wv, int lane) {
   const int l32 = lane & 31;
   const int kq = (lane >> 5) * 8;
+  lds_half_t *pxb = lds_opaque(sIn + (wv * RPW * SY * HALO_W + l32 * SX) * CKP + kq);
+  lds_half_t *wb = lds_opaque(sW + l32 * WPITCH + wofs + kq);
 #pragma unroll
   for (int s = 0; s < KS; ++s) {
 #pragma unroll
     for (int ks = 0; ks < L / 16; ++ks) {
-      const int kk = ks * 16 + kq;
       half8 px[PXROWS];
 #pragma unroll
       for (int hr = 0; hr < PXROWS; ++hr)
         if (SY == 1 || hr % SY < KR) // with a stride larger than the filter some halo rows are never read
-          px[hr] = *reinterpret_cast<const half8 *>(sIn + ((wv * RPW * SY + hr) * HALO_W + l32 * SX + s) * CKP + kk);
+          px[hr] = *reinterpret_cast<lds_half8_t *>(pxb + (hr * HALO_W + s) * CKP + ks * 16);
 #pragma unroll
       for (int r = 0; r < KR; ++r) {
         half8 wf[KB];
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
-          wf[kb] = *reinterpret_cast<const half8 *>(sW + (((r * KS + s) * KT) + kb * 32 + l32) * WPITCH + wofs + kk);
+          wf[kb] = *reinterpret_cast<lds_half8_t *>(wb + ((r * KS + s) * KT + kb * 32) * WPITCH + ks * 16);
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -627,14 +661,21 @@ mma_chunk(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, int wv, i
   }
 }
 
-__device__ DNX_INLINE void zero_acc(Acc &acc) {
+// Start of a tile: every accumulator holds the bias of its output channel (zero without one).  Reads the staged bias,
+// so it runs after a barrier that follows stage_bias.
+__device__ DNX_INLINE void init_acc(Acc &acc, const bias_t *sBias, int lane) {
+  const int hsel = lane >> 5;
 #pragma unroll
   for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
     for (int j = 0; j < RPW; ++j)
 #pragma unroll
       for (int i = 0; i < 16; ++i)
+#if HAS_BIAS
+        acc.v[kb][j][i] = sBias[kb * 32 + hsel * 16 + i];
+#else
         acc.v[kb][j][i] = 0.0f;
+#endif
 }
 
 #else
@@ -672,23 +713,12 @@ struct Packed {
   _Float16 o[KPAIRS][XB][OROWS][8];
 };
 
-// bias, activation, rounding to fp16 and (POOL) the 2x2 maximum
-__device__ DNX_INLINE void pack_tile(const Acc &acc, Packed &pk, const _Float16 *sBias, int lane) {
-  const int g = lane >> 4;
+// activation, rounding to fp16 and (POOL) the 2x2 maximum
+__device__ DNX_INLINE void pack_tile(const Acc &acc, Packed &pk) {
 #pragma unroll
   for (int kp = 0; kp < KPAIRS; ++kp) {
     const bool paired = 2 * kp + 1 < KB;
     const int n = paired ? 8 : 4;
-    const int chl = paired ? 32 * kp + 8 * g : 16 * (2 * kp) + 4 * g; // first channel, relative to the workgroup's KT
-    float bias[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-#if HAS_BIAS
-      bias[i] = i < n ? (float)sBias[chl + i] : 0.0f;
-#else
-      bias[i] = 0.0f;
-#endif
-    }
 #pragma unroll
     for (int xb = 0; xb < XB; ++xb) {
 #pragma unroll
@@ -699,8 +729,8 @@ __device__ DNX_INLINE void pack_tile(const Acc &acc, Packed &pk, const _Float16 
           _Float16 m = (_Float16)0.0f;
           if (i < n) {
 #if POOL
-            const _Float16 v0 = (_Float16)apply_act(acc.v[kb][2 * r][xb][i & 3] + bias[i]);
-            const _Float16 v1 = (_Float16)apply_act(acc.v[kb][2 * r + 1][xb][i & 3] + bias[i]);
+            const _Float16 v0 = finish1(acc.v[kb][2 * r][xb][i & 3]);
+            const _Float16 v1 = finish1(acc.v[kb][2 * r + 1][xb][i & 3]);
             const _Float16 n0 = __builtin_bit_cast(_Float16, dpp_xor1(__builtin_bit_cast(ushort_t, v0)));
             const _Float16 n1 = __builtin_bit_cast(_Float16, dpp_xor1(__builtin_bit_cast(ushort_t, v1)));
             m = v0; // window order (0,0) (0,1) (1,0) (1,1); replace only on strictly greater
@@ -708,7 +738,7 @@ __device__ DNX_INLINE void pack_tile(const Acc &acc, Packed &pk, const _Float16 
             m = v1 > m ? v1 : m;
             m = n1 > m ? n1 : m;
 #else
-            m = (_Float16)apply_act(acc.v[kb][r][xb][i & 3] + bias[i]);
+            m = finish1(acc.v[kb][r][xb][i & 3]);
 #endif
           }
           pk.o[kp][xb][r][i] = m;
@@ -762,24 +792,25 @@ __device__ DNX_INLINE void
 mma_chunk(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, int wv, int lane) {
   const int l16 = lane & 15;
   const int kq = (lane >> 4) * 8;
+  lds_half_t *pxb = lds_opaque(sIn + (wv * RPW * SY * HALO_W + l16 * SX) * CKP + kq);
+  lds_half_t *wb = lds_opaque(sW + l16 * WPITCH + wofs + kq);
 #pragma unroll
   for (int s = 0; s < KS; ++s) {
 #pragma unroll
     for (int ks = 0; ks < L / 32; ++ks) {
-      const int kk = ks * 32 + kq;
       half8 px[PXROWS][XB];
 #pragma unroll
       for (int hr = 0; hr < PXROWS; ++hr)
 #pragma unroll
         for (int xb = 0; xb < XB; ++xb)
           if (SY == 1 || hr % SY < KR)
-            px[hr][xb] = *reinterpret_cast<const half8 *>(sIn + ((wv * RPW * SY + hr) * HALO_W + (xb * 16 + l16) * SX + s) * CKP + kk);
+            px[hr][xb] = *reinterpret_cast<lds_half8_t *>(pxb + (hr * HALO_W + xb * 16 * SX + s) * CKP + ks * 32);
 #pragma unroll
       for (int r = 0; r < KR; ++r) {
         half8 wf[KB];
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
-          wf[kb] = *reinterpret_cast<const half8 *>(sW + (((r * KS + s) * KT) + kb * 16 + l16) * WPITCH + wofs + kk);
+          wf[kb] = *reinterpret_cast<lds_half8_t *>(wb + ((r * KS + s) * KT + kb * 16) * WPITCH + ks * 32);
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -792,23 +823,34 @@ mma_chunk(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, int wv, i
   }
 }
 
-__device__ DNX_INLINE void zero_acc(Acc &acc) {
+// Start of a tile: every accumulator holds the bias of its output channel (zero without one); the channel of
+// acc.v[kb][..][..][e] is the one pack_tile / store_packed assign to it.  Runs after a barrier that follows stage_bias.
+__device__ DNX_INLINE void init_acc(Acc &acc, const bias_t *sBias, int lane) {
+  const int g = lane >> 4;
 #pragma unroll
-  for (int kb = 0; kb < KB; ++kb)
+  for (int kb = 0; kb < KB; ++kb) {
+    const int kp = kb >> 1;
+    const bool paired = 2 * kp + 1 < KB;
+    const int chl = paired ? 32 * kp + 8 * g + 4 * (kb & 1) : 16 * kb + 4 * g;
 #pragma unroll
     for (int j = 0; j < RPW; ++j)
 #pragma unroll
       for (int xb = 0; xb < XB; ++xb)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
+#if HAS_BIAS
+          acc.v[kb][j][xb][i] = sBias[chl + i];
+#else
           acc.v[kb][j][xb][i] = 0.0f;
+#endif
+  }
 }
 #endif // MF
 
 __device__ DNX_INLINE void
-store_tile(const Acc &acc, OutBuf out, const _Float16 *sBias, int y0, int x0, int kt, int wv, int lane, const PushConstants &pc) {
+store_tile(const Acc &acc, OutBuf out, int y0, int x0, int kt, int wv, int lane, const PushConstants &pc) {
   Packed pk;
-  pack_tile(acc, pk, sBias, lane);
+  pack_tile(acc, pk);
   store_packed(pk, out, y0, x0, kt, wv, lane, pc);
 }
 
