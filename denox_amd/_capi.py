@@ -81,6 +81,7 @@ SIGNATURES = {
     "denox_hip_builder_pool": (c_int, [c_void_p, c_int, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, POINTER(c_int)]),
     "denox_hip_builder_concat": (c_int, [c_void_p, c_int, c_int, POINTER(c_int)]),
     "denox_hip_builder_pad": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, POINTER(c_int)]),
+    "denox_hip_builder_pad_mode": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_int32, POINTER(c_int)]),
     "denox_hip_builder_slice": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, POINTER(c_int)]),
     "denox_hip_builder_output": (c_int, [c_void_p, c_int, c_char_p]),
     "denox_hip_builder_import_onnx": (c_int, [c_void_p, c_char_p, c_size_t]),

@@ -194,6 +194,13 @@ int denox_hip_builder_concat(denox_hip_builder *b, int src0, int src1, int *out_
 int denox_hip_builder_pad(denox_hip_builder *b, int src, int64_t l, int64_t r, int64_t t, int64_t bo, int *out_tensor) {
   return guarded([&] { need(b, "builder"); need(out_tensor, "out_tensor"); *out_tensor = b->model.pad(src, symFromHandle(l), symFromHandle(r), symFromHandle(t), symFromHandle(bo), compiler::PaddingMode::Replicate); });
 }
+int denox_hip_builder_pad_mode(denox_hip_builder *b, int src, int64_t l, int64_t r, int64_t t, int64_t bo, int32_t mode, int *out_tensor) {
+  return guarded([&] {
+    need(b, "builder"); need(out_tensor, "out_tensor");
+    if (mode != 0 && mode != 1) fail(Status::InvalidArgument, "pad mode must be 0 (replicate) or 1 (zero)");
+    *out_tensor = b->model.pad(src, symFromHandle(l), symFromHandle(r), symFromHandle(t), symFromHandle(bo), mode ? compiler::PaddingMode::Zero : compiler::PaddingMode::Replicate);
+  });
+}
 int denox_hip_builder_slice(denox_hip_builder *b, int src, int64_t l, int64_t r, int64_t t, int64_t bo, int *out_tensor) {
   return guarded([&] { need(b, "builder"); need(out_tensor, "out_tensor"); *out_tensor = b->model.slice(src, symFromHandle(l), symFromHandle(r), symFromHandle(t), symFromHandle(bo)); });
 }

@@ -99,12 +99,13 @@ TensorHandle Model::concat(TensorHandle src0, TensorHandle src1) {
   return m_ops.back().output;
 }
 
-TensorHandle Model::pad(TensorHandle src, Sym left, Sym right, Sym top, Sym bottom, PaddingMode) {
+TensorHandle Model::pad(TensorHandle src, Sym left, Sym right, Sym top, Sym bottom, PaddingMode mode) {
   const TensorNode in = get(src);
   Op op;
   op.kind = OpKind::Pad;
   op.inputs = {src};
   op.left = left; op.right = right; op.top = top; op.bottom = bottom;
+  op.padMode = mode;
   op.output = newTensor(m_sym.add(m_sym.add(in.width, left), right), m_sym.add(m_sym.add(in.height, top), bottom), in.channels, static_cast<int>(m_ops.size()));
   m_tensors[src].consumers.push_back(static_cast<int>(m_ops.size()));
   m_ops.push_back(std::move(op));

@@ -17,7 +17,7 @@ enum class OpKind { Conv, Activation, Upsample, Pool, Concat, Pad, Slice };
 enum class ActivationFunction { ReLU, LeakyReLU };
 enum class PoolFunction { Max };
 enum class FilterMode { Nearest };
-enum class PaddingMode { Replicate };
+enum class PaddingMode { Replicate, Zero }; // the reference's PaddingMode { Edge, Zero } (common/PaddingMode.hpp)
 
 using TensorHandle = int; // index into Model::tensors
 
@@ -48,6 +48,7 @@ struct Op {
   unsigned kernelX = 2, kernelY = 2, poolStrideX = 2, poolStrideY = 2, poolPadX = 0, poolPadY = 0;
   // Pad: border widths.  Slice: the half-open source ranges [left, right) x [top, bottom)
   Sym left, right, top, bottom;
+  PaddingMode padMode = PaddingMode::Replicate;
 };
 
 struct NamedValue { std::string name; Sym value; };

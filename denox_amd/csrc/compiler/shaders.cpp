@@ -270,7 +270,8 @@ public:
     if (prod >= 0) {
       const Op &p = model.ops()[prod];
       if (allowUpsample && p.kind == OpKind::Upsample && p.scale == 2 && opt.features.enableUpsampleFusion) out.push_back(Source{PAT_UPSAMPLE, {prod}, p.inputs[0]});
-      if (p.kind == OpKind::Pad && opt.features.enablePadFusion) out.push_back(Source{padBit, {prod}, p.inputs[0]});
+      // the conv loaders clamp coordinates, which is the replicate mode; a zero-mode pad stays a dispatch of its own
+      if (p.kind == OpKind::Pad && p.padMode == PaddingMode::Replicate && opt.features.enablePadFusion) out.push_back(Source{padBit, {prod}, p.inputs[0]});
     }
     return out;
   }
@@ -709,8 +710,10 @@ public:
     const unsigned vec = place.vec;
     auto k = m_compiler->read("pad.hip");
     k.define("CH", in.channels); k.define("VEC", vec);
+    const bool zeros = op.padMode == PaddingMode::Zero;
+    if (zeros) k.define("ZERO", 1);
     defineOutput(k, place);
-    const std::string entry = "memory_pad_c" + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
+    const std::string entry = std::string(zeros ? "memory_pad_zero_c" : "memory_pad_c") + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
     k.define("KERNEL_NAME", entry);
     auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, in.channels / vec), out.height, Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);

@@ -1050,11 +1050,20 @@ struct Importer {
       unsupported("Pad '" + n.name + "': only height and width of an image tensor can be padded");
     const bool none = before[2] == zero && after[2] == zero && before[3] == zero && after[3] == zero;
     if (none) { values[n.out.at(0)] = v; return; }
-    if (mode != "edge") unsupported("Pad '" + n.name + "': mode '" + mode + "' on an image tensor (only 'edge')");
+    if (mode != "edge" && mode != "constant") unsupported("Pad '" + n.name + "': mode '" + mode + "' on an image tensor (only 'edge' and 'constant')");
+    if (mode == "constant") { // the constant is input 2 (attribute `value` before opset 11); only 0 has a kernel
+      double value = n.floatAttr("value", 0.0f);
+      if (has(n, 2)) {
+        const HostTensor c = toFloat(n, host(n, 2));
+        if (c.count() != 1) bad("Pad '" + n.name + "': constant_value must be a scalar");
+        value = c.fv[0];
+      }
+      if (value != 0.0) unsupported("Pad '" + n.name + "': constant padding with a value other than 0");
+    }
     for (int ax = 2; ax < 4; ++ax)
       for (const Sym &s : {before[ax], after[ax]})
         if (s.isConst() && s.v < 0) unsupported("Pad '" + n.name + "': negative padding");
-    setDevice(n, model.pad(device(n, 0), before[3], after[3], before[2], after[2], compiler::PaddingMode::Replicate));
+    setDevice(n, model.pad(device(n, 0), before[3], after[3], before[2], after[2], mode == "edge" ? compiler::PaddingMode::Replicate : compiler::PaddingMode::Zero));
   }
 
   // ---------------------------------------------------------------- graph

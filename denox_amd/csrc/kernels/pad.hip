@@ -1,8 +1,12 @@
-// pad.hip -- replicate ("edge") padding, HWC binary16.
+// pad.hip -- replicate ("edge") or zero padding, HWC binary16.
 // Replaces compiler/src/denox/compiler/implement/shaders/pad/memory_pad.comp:31-133:
-//   out[ho, wo, c] = in[clamp(ho - PAD_T, 0, IN_H-1), clamp(wo - PAD_L, 0, IN_W-1), c].
-// Definitions: CH, VEC.  grid.y = output rows.
+//   out[ho, wo, c] = in[clamp(ho - PAD_T, 0, IN_H-1), clamp(wo - PAD_L, 0, IN_W-1), c];
+// with ZERO = 1 the border is 0 instead (PaddingMode::Zero of the reference's model, which its shader does not implement).
+// Definitions: CH, VEC, ZERO.  grid.y = output rows.
 #include "common.h"
+#ifndef ZERO
+#define ZERO 0
+#endif
 #ifndef KERNEL_NAME
 #define KERNEL_NAME memory_pad
 #endif
@@ -16,7 +20,16 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
   const unsigned wo = i / CV, cv = i - wo * CV;
   const int IN_W = (int)(pc.OUT_W - pc.PAD_L - pc.PAD_R);
   const int IN_H = (int)(pc.OUT_H - pc.PAD_T - pc.PAD_B);
-  int hi = ho - (int)pc.PAD_T; hi = hi < 0 ? 0 : (hi > IN_H - 1 ? IN_H - 1 : hi);
-  int wi = (int)wo - (int)pc.PAD_L; wi = wi < 0 ? 0 : (wi > IN_W - 1 ? IN_W - 1 : wi);
-  stv(OUT + ((size_t)ho * pc.OUT_W + wo) * OPITCH + cv * VEC, ldv(IN + ((size_t)hi * IN_W + wi) * CH + cv * VEC));
+  int hi = ho - (int)pc.PAD_T, wi = (int)wo - (int)pc.PAD_L;
+#if ZERO
+  const bool inside = hi >= 0 && hi < IN_H && wi >= 0 && wi < IN_W;
+#endif
+  hi = hi < 0 ? 0 : (hi > IN_H - 1 ? IN_H - 1 : hi);
+  wi = wi < 0 ? 0 : (wi > IN_W - 1 ? IN_W - 1 : wi);
+  vec_t v = ldv(IN + ((size_t)hi * IN_W + wi) * CH + cv * VEC); // the clamped read is in range in both modes
+#if ZERO
+  const vec_t zero = {};
+  v = inside ? v : zero;
+#endif
+  stv(OUT + ((size_t)ho * pc.OUT_W + wo) * OPITCH + cv * VEC, v);
 }

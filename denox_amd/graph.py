@@ -180,12 +180,14 @@ class Model:
         self._ops.append({"op": "concat", "src": [a.name, b.name], "dst": out.name})
         return out
 
-    def pad(self, src: Tensor, left, right, top, bottom) -> Tensor:
+    def pad(self, src: Tensor, left, right, top, bottom, mode: str = "replicate") -> Tensor:
+        """mode "replicate" repeats the border pixels (F.pad mode="replicate"), "zero" fills with zeros (mode="constant")."""
+        code = {"replicate": 0, "zero": 1}[mode]
         l, r, tp, bt = (self.sym(v) for v in (left, right, top, bottom))
         t = c_int()
-        _capi.check(_capi.lib().denox_hip_builder_pad(self._h, src.handle, l.handle, r.handle, tp.handle, bt.handle, byref(t)))
+        _capi.check(_capi.lib().denox_hip_builder_pad_mode(self._h, src.handle, l.handle, r.handle, tp.handle, bt.handle, code, byref(t)))
         out = Tensor(self, t.value, self._name("pad"), src.width + l + r, src.height + tp + bt, src.channels)
-        self._ops.append({"op": "pad", "src": src.name, "dst": out.name, "left": l, "right": r, "top": tp, "bottom": bt})
+        self._ops.append({"op": "pad", "src": src.name, "dst": out.name, "left": l, "right": r, "top": tp, "bottom": bt, "mode": mode})
         return out
 
     def slice(self, src: Tensor, left, right, top, bottom) -> Tensor:

@@ -110,6 +110,8 @@ int denox_hip_builder_pool(denox_hip_builder *b, int src, uint32_t kx, uint32_t 
                            uint32_t stride_x, uint32_t stride_y, int *out_tensor);                          /* max */
 int denox_hip_builder_concat(denox_hip_builder *b, int src0, int src1, int *out_tensor);
 int denox_hip_builder_pad(denox_hip_builder *b, int src, int64_t left_sym, int64_t right_sym, int64_t top_sym, int64_t bottom_sym, int *out_tensor); /* replicate */
+/* mode: 0 replicate the border (PaddingMode::Edge of the reference), 1 zeros (PaddingMode::Zero) */
+int denox_hip_builder_pad_mode(denox_hip_builder *b, int src, int64_t left_sym, int64_t right_sym, int64_t top_sym, int64_t bottom_sym, int32_t mode, int *out_tensor);
 /* half-open source ranges [left, right) x [top, bottom) */
 int denox_hip_builder_slice(denox_hip_builder *b, int src, int64_t left_sym, int64_t right_sym, int64_t top_sym, int64_t bottom_sym, int *out_tensor);
 int denox_hip_builder_output(denox_hip_builder *b, int src, const char *name);

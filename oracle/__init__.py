@@ -58,6 +58,7 @@ def lib() -> ctypes.CDLL:
         L.dnxo_copy_channels_hwc_f16.argtypes = [u16p, i64, i64, i64, i64, u16p, i64, i64, i64]
         L.dnxo_concat_hwc_f16.argtypes = [u16p, i64, u16p, i64, i64, i64, u16p]
         L.dnxo_pad_replicate_hwc_f16.argtypes = [u16p, i64, i64, i64, i64, i64, i64, i64, u16p]
+        L.dnxo_pad_zero_hwc_f16.argtypes = [u16p, i64, i64, i64, i64, i64, i64, i64, u16p]
         L.dnxo_slice_hwc_f16.argtypes = [u16p, i64, i64, i64, i64, i64, i64, i64, u16p]
         L.dnxo_activation_f16.argtypes = [u16p, ctypes.c_size_t, ctypes.c_int, f32, u16p]
         L.dnxo_symir_eval.argtypes = [i64, u16p, i64, u16p, u16p, u16p, u16p]
@@ -174,6 +175,14 @@ def pad_replicate(x: np.ndarray, left: int, right: int, top: int, bottom: int) -
     return out
 
 
+def pad_zero(x: np.ndarray, left: int, right: int, top: int, bottom: int) -> np.ndarray:
+    xin = _c(x, np.float16)
+    H, W, C = xin.shape
+    out = np.empty((H + top + bottom, W + left + right, C), np.float16)
+    _check(lib().dnxo_pad_zero_hwc_f16(_p(xin), H, W, C, left, right, top, bottom, _p(out)), "pad")
+    return out
+
+
 def slice_hw(x: np.ndarray, left: int, top: int, out_h: int, out_w: int) -> np.ndarray:
     xin = _c(x, np.float16)
     H, W, C = xin.shape
@@ -279,7 +288,10 @@ def run_graph(ops: Sequence[dict], inputs: Dict[str, np.ndarray], mode: str = "f
             elif kind == "pad":
                 x = env[src]
                 l, r, t, b = op["left"], op["right"], op["top"], op["bottom"]
-                env[op["dst"]] = pad_replicate(x, l, r, t, b) if f16 else np.pad(x, ((t, b), (l, r), (0, 0)), mode="edge")
+                if op.get("mode", "replicate") == "zero":
+                    env[op["dst"]] = pad_zero(x, l, r, t, b) if f16 else np.pad(x, ((t, b), (l, r), (0, 0)), mode="constant")
+                else:
+                    env[op["dst"]] = pad_replicate(x, l, r, t, b) if f16 else np.pad(x, ((t, b), (l, r), (0, 0)), mode="edge")
             else:
                 x = env[src]
                 l, t, oh, ow = op["left"], op["top"], op["out_h"], op["out_w"]

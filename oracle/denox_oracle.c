@@ -19,6 +19,7 @@
  *   dnxo_upsample_nearest_hwc_f16          pinned: F.interpolate(mode="nearest")
  *   dnxo_concat_hwc_f16 / dnxo_copy_channels_hwc_f16   pinned: torch.cat
  *   dnxo_pad_replicate_hwc_f16             pinned: F.pad(mode="replicate")
+ *   dnxo_pad_zero_hwc_f16                  pinned: F.pad(mode="constant", value=0)
  *   dnxo_slice_hwc_f16                     pinned: tensor slicing
  *   dnxo_activation_f16                    pinned: F.relu / F.leaky_relu on fp16
  *   dnxo_layout_index / dnxo_relayout_f16  pinned: permute/reshape round trips
@@ -357,6 +358,20 @@ DNXO_API int dnxo_pad_replicate_hwc_f16(const uint16_t *in, int64_t H,
       memcpy(out + (ho * Wo + wo) * C, in + (hi * W + wi) * C, (size_t)C * 2);
     }
   }
+  return 0;
+}
+
+/* Zero padding: the border is 0 (PaddingMode::Zero of the reference's model, common/src/denox/common/PaddingMode.hpp;
+ * torch: F.pad(mode="constant", value=0)). */
+DNXO_API int dnxo_pad_zero_hwc_f16(const uint16_t *in, int64_t H, int64_t W,
+                                   int64_t C, int64_t left, int64_t right,
+                                   int64_t top, int64_t bottom, uint16_t *out) {
+  if (left < 0 || right < 0 || top < 0 || bottom < 0)
+    return -1;
+  const int64_t Ho = H + top + bottom, Wo = W + left + right;
+  memset(out, 0, (size_t)(Ho * Wo * C) * 2);
+  for (int64_t h = 0; h < H; ++h)
+    memcpy(out + ((h + top) * Wo + left) * C, in + h * W * C, (size_t)(W * C) * 2);
   return 0;
 }
 

@@ -457,3 +457,25 @@ def test_bandwidth_kernels_store_in_place(oracle, C0, C1):
     for g, r, t in zip(got, cop, (o1, o2, o3)):
         assert_bits_equal(g, r, "in place against copied")
         assert_bits_equal(g, want[t.name], "in place against the oracle")
+
+
+@pytest.mark.parametrize("C", [3, 8, 9, 64])
+def test_zero_padding(oracle, C):
+    """Pad with zeros (F.pad mode="constant"): a dispatch of its own (the conv loaders fold only the replicate mode), bit-exact
+    alone and in front of a conv, whose own zero padding then sees zeros twice."""
+    rng = np.random.default_rng(C)
+    H, W = 23, 41
+    x = rng.standard_normal((H, W, C)).astype(np.float16)
+    m = dx.Model()
+    p = m.pad(m.input("input", "W", "H", C), 2, 5, 1, 3, mode="zero")
+    y = m.relu(m.conv2d(p, he_weights(rng, 16, C), small_bias(rng, 16)))
+    m.output(p)
+    m.output(y)
+    mod = dx.Module.compile(m)
+    names = [d_["name"] for d_ in dx.describe(mod.dnx, H=H, W=W)["dispatches"]]
+    assert names == ["pad", "conv3x3+relu"]
+    got_p, got_y = mod.instance(H=H, W=W).infer(x)
+    want = oracle.run_graph(m.to_ops({"H": H, "W": W}), {"input": x}, "f16")
+    assert_bits_equal(got_p, want[p.name], "zero pad")
+    assert got_p.shape == (H + 4, W + 7, C) and not got_p[0].any() and not got_p[:, :2].any()
+    assert_conv_close(got_y, oracle.run_graph(m.to_ops({"H": H, "W": W}), {"input": x}, "fp32")[y.name], "conv behind a zero pad")

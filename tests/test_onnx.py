@@ -205,8 +205,17 @@ def test_unsupported_and_malformed_models_are_reported():
     with pytest.raises(dx.DenoxHipError) as e:
         dx.Model.from_onnx(conv_model([node("Softmax", ["c"], ["y"], name="sm0")], "y", (1, 8, "h", "w")))
     assert e.value.status == 5 and "Softmax" in str(e.value) and "sm0" in str(e.value)
-    with pytest.raises(dx.DenoxHipError) as e:  # zero padding other than the conv's own
-        dx.Model.from_onnx(conv_model([node("Pad", ["c", "p"], ["y"])], "y", (1, 8, "h", "w"), [tensor("p", np.array([0, 0, 1, 1, 0, 0, 1, 1], np.int64))]))
+    # constant-mode Pad: zeros are a layer of their own, any other constant has no kernel
+    pads = tensor("p", np.array([0, 0, 1, 2, 0, 0, 3, 4], np.int64))
+    blob = dx.compile_model(dx.Model.from_onnx(conv_model([node("Pad", ["c", "p"], ["y"])], "y", (1, 8, "h", "w"), [pads])))
+    d = dx.describe(blob, H=10, W=20)
+    out = d["tensors"][d["outputs"][0]]
+    assert (out["height"], out["width"]) == (14, 26) and "ZERO=1" in d["dispatches"][-1]["debug_info"]
+    with pytest.raises(dx.DenoxHipError) as e:
+        dx.Model.from_onnx(conv_model([node("Pad", ["c", "p", "v"], ["y"])], "y", (1, 8, "h", "w"), [pads, tensor("v", np.array(1.5, np.float32))]))
+    assert e.value.status == 5 and "other than 0" in str(e.value)
+    with pytest.raises(dx.DenoxHipError) as e:
+        dx.Model.from_onnx(conv_model([node("Pad", ["c", "p"], ["y"], attr_str("mode", "reflect"))], "y", (1, 8, "h", "w"), [pads]))
     assert e.value.status == 5 and "mode" in str(e.value)
     with pytest.raises(dx.DenoxHipError) as e:  # batch of 2
         dx.Model.from_onnx(conv_model([], "c", (2, 8, "h", "w"), in_dims=(2, 8, "H", "W")))

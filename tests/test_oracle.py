@@ -197,6 +197,16 @@ def test_pad_replicate_vs_torch(oracle, l, r, t, b):
     assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
 
 
+@pytest.mark.parametrize("l,r,t,b", [(0, 0, 0, 8), (0, 3, 0, 11), (2, 1, 3, 0), (0, 0, 0, 0), (5, 5, 5, 5)])
+def test_pad_zero_vs_torch(oracle, l, r, t, b):
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((4, 5, 9)).astype(np.float16)
+    got = oracle.pad_zero(x, l, r, t, b)
+    want = nchw_to_hwc(F.pad(hwc_to_nchw(x.astype(np.float32)), (l, r, t, b), mode="constant", value=0.0)).astype(np.float16)
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    assert got[t:t + 4, l:l + 5].tobytes() == x.tobytes() and not got[:t].any() and not got[:, :l].any()  # interior kept, border 0
+
+
 def test_slice_vs_indexing(oracle):
     rng = np.random.default_rng(9)
     x = rng.standard_normal((9, 10, 3)).astype(np.float16)
