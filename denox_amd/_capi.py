@@ -79,6 +79,7 @@ SIGNATURES = {
     "denox_hip_builder_activation": (c_int, [c_void_p, c_int, c_int, c_float, POINTER(c_int)]),
     "denox_hip_builder_upsample": (c_int, [c_void_p, c_int, c_uint32, POINTER(c_int)]),
     "denox_hip_builder_pool": (c_int, [c_void_p, c_int, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, POINTER(c_int)]),
+    "denox_hip_builder_avg_pool": (c_int, [c_void_p, c_int, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, POINTER(c_int)]),
     "denox_hip_builder_concat": (c_int, [c_void_p, c_int, c_int, POINTER(c_int)]),
     "denox_hip_builder_pad": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, POINTER(c_int)]),
     "denox_hip_builder_pad_mode": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_int32, POINTER(c_int)]),

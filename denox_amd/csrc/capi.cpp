@@ -188,6 +188,9 @@ int denox_hip_builder_upsample(denox_hip_builder *b, int src, uint32_t scale, in
 int denox_hip_builder_pool(denox_hip_builder *b, int src, uint32_t kx, uint32_t ky, uint32_t px, uint32_t py, uint32_t sx, uint32_t sy, int *out_tensor) {
   return guarded([&] { need(b, "builder"); need(out_tensor, "out_tensor"); *out_tensor = b->model.pool(src, kx, ky, px, py, sx, sy, compiler::PoolFunction::Max); });
 }
+int denox_hip_builder_avg_pool(denox_hip_builder *b, int src, uint32_t kx, uint32_t ky, uint32_t px, uint32_t py, uint32_t sx, uint32_t sy, int *out_tensor) {
+  return guarded([&] { need(b, "builder"); need(out_tensor, "out_tensor"); *out_tensor = b->model.pool(src, kx, ky, px, py, sx, sy, compiler::PoolFunction::Avg); });
+}
 int denox_hip_builder_concat(denox_hip_builder *b, int src0, int src1, int *out_tensor) {
   return guarded([&] { need(b, "builder"); need(out_tensor, "out_tensor"); *out_tensor = b->model.concat(src0, src1); });
 }

@@ -70,13 +70,13 @@ TensorHandle Model::upsample(TensorHandle src, unsigned f, FilterMode) {
   return m_ops.back().output;
 }
 
-TensorHandle Model::pool(TensorHandle src, unsigned kx, unsigned ky, unsigned px, unsigned py, unsigned sx, unsigned sy, PoolFunction) {
+TensorHandle Model::pool(TensorHandle src, unsigned kx, unsigned ky, unsigned px, unsigned py, unsigned sx, unsigned sy, PoolFunction f) {
   const TensorNode in = get(src);
   if (kx == 0 || ky == 0 || sx == 0 || sy == 0) fail(Status::InvalidArgument, "pool: bad window");
   Op op;
   op.kind = OpKind::Pool;
   op.inputs = {src};
-  op.kernelX = kx; op.kernelY = ky; op.poolPadX = px; op.poolPadY = py; op.poolStrideX = sx; op.poolStrideY = sy;
+  op.kernelX = kx; op.kernelY = ky; op.poolPadX = px; op.poolPadY = py; op.poolStrideX = sx; op.poolStrideY = sy; op.poolFunc = f;
   op.output = newTensor(m_sym.pool(in.width, kx, px, sx, 1), m_sym.pool(in.height, ky, py, sy, 1), in.channels, static_cast<int>(m_ops.size()));
   m_tensors[src].consumers.push_back(static_cast<int>(m_ops.size()));
   m_ops.push_back(std::move(op));

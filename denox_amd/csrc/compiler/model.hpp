@@ -15,7 +15,7 @@ namespace denox::compiler {
 
 enum class OpKind { Conv, Activation, Upsample, Pool, Concat, Pad, Slice };
 enum class ActivationFunction { ReLU, LeakyReLU };
-enum class PoolFunction { Max };
+enum class PoolFunction { Max, Avg };
 enum class FilterMode { Nearest };
 enum class PaddingMode { Replicate, Zero }; // the reference's PaddingMode { Edge, Zero } (common/PaddingMode.hpp)
 
@@ -46,6 +46,7 @@ struct Op {
   unsigned scale = 2;
   // Pool
   unsigned kernelX = 2, kernelY = 2, poolStrideX = 2, poolStrideY = 2, poolPadX = 0, poolPadY = 0;
+  PoolFunction poolFunc = PoolFunction::Max;
   // Pad: border widths.  Slice: the half-open source ranges [left, right) x [top, bottom)
   Sym left, right, top, bottom;
   PaddingMode padMode = PaddingMode::Replicate;

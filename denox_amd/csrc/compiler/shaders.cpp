@@ -307,7 +307,7 @@ public:
       struct Epi { unsigned bits; std::vector<int> ops; int output; };
       std::vector<Epi> epis;
       epis.push_back(Epi{0, {}, conv.output});
-      auto poolOk = [](const Op &q) { return q.kind == OpKind::Pool && q.kernelX == 2 && q.kernelY == 2 && q.poolStrideX == 2 && q.poolStrideY == 2 && q.poolPadX == 0 && q.poolPadY == 0; };
+      auto poolOk = [](const Op &q) { return q.kind == OpKind::Pool && q.poolFunc == PoolFunction::Max && q.kernelX == 2 && q.kernelY == 2 && q.poolStrideX == 2 && q.poolStrideY == 2 && q.poolPadX == 0 && q.poolPadY == 0; };
       auto tails = [&](TensorHandle t, unsigned bits, std::vector<int> chain) {
         if (!singleUse(model, t)) return;
         const int c = model.tensors()[t].consumers[0];
@@ -575,7 +575,9 @@ class BasicPoolShader final : public SingleOpShader {
 public:
   explicit BasicPoolShader(const hip::HipCompiler *c) : SingleOpShader(c, OpKind::Pool) {}
   std::string name() const override { return "basic_pool"; }
-  // kernel == stride, no padding (the reference's restriction, BasicPoolShader.cpp:165-180)
+  // kernel == stride, no padding (the reference's restriction, BasicPoolShader.cpp:165-180).  The reference's shader
+  // also refuses PoolFunction::Avg (BasicPoolShader.cpp:170), which its model and ONNX importer accept
+  // (frontend/onnx/details/ops/average_pool.cpp:154); the kernel here has an averaging mode, so such models compile.
   bool supports(const Op &op) const override { return op.kernelX == op.poolStrideX && op.kernelY == op.poolStrideY && op.poolPadX == 0 && op.poolPadY == 0; }
   void implement(OpImpl &impl, const Model &model, const Match &m, unsigned, SymGraph &sym, const CompileOptions &) const override {
     const Op &op = model.ops()[m.ops[0]];
@@ -583,15 +585,17 @@ public:
     const Placement place = placementOf(model, m, in.channels);
     const unsigned vec = place.vec;
     auto k = m_compiler->read("pool.hip");
+    const bool avg = op.poolFunc == PoolFunction::Avg;
     k.define("CH", in.channels); k.define("KX", op.kernelX); k.define("KY", op.kernelY); k.define("VEC", vec);
+    if (avg) k.define("AVG", 1);
     defineOutput(k, place);
-    const std::string entry = "pool_max_c" + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
+    const std::string entry = std::string(avg ? "pool_avg_c" : "pool_max_c") + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
     k.define("KERNEL_NAME", entry);
     auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, in.channels / vec), out.height, Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     bindOutput(d, sym, model, m, place);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
-    d.setName(std::string("maxpool") + (place.view.valid ? "+concat" : "")); d.setOperation("maxpool"); d.setConfig("vec" + std::to_string(vec));
+    d.setName(std::string(avg ? "avgpool" : "maxpool") + (place.view.valid ? "+concat" : "")); d.setOperation(avg ? "avgpool" : "maxpool"); d.setConfig("vec" + std::to_string(vec));
     d.setMemoryReads(bytesOf(sym, in)); d.setMemoryWrites(bytesOf(sym, out)); d.setFlops(Sym::Const(0));
   }
 };

@@ -971,20 +971,23 @@ struct Importer {
                               static_cast<unsigned>(dil[1]), static_cast<unsigned>(dil[0])));
   }
 
-  void opMaxPool(const Node &n) {
+  // MaxPool and AveragePool (frontend/onnx/details/ops/max_pool.cpp:9-165, average_pool.cpp:9-156)
+  void opPool(const Node &n, compiler::PoolFunction func) {
     const TensorHandle x = device(n, 0);
-    if (n.out.size() > 1 && !n.out[1].empty()) unsupported("MaxPool '" + n.name + "': the indices output");
+    const std::string what = n.op + " '" + n.name + "'";
+    if (n.out.size() > 1 && !n.out[1].empty()) unsupported(what + ": the indices output");
     const auto ks = n.intsAttr("kernel_shape");
-    if (ks.size() != 2) unsupported("MaxPool '" + n.name + "': kernel_shape must have 2 entries");
+    if (ks.size() != 2) unsupported(what + ": kernel_shape must have 2 entries");
     std::vector<int64_t> strides = n.intsAttr("strides");
     if (strides.empty()) strides = {1, 1};
-    if (strides.size() != 2) bad("MaxPool '" + n.name + "': strides");
-    for (auto d : n.intsAttr("dilations")) if (d != 1) unsupported("MaxPool '" + n.name + "': dilation");
-    if (n.intAttr("ceil_mode", 0) != 0) unsupported("MaxPool '" + n.name + "': ceil_mode");
+    if (strides.size() != 2) bad(what + ": strides");
+    for (auto d : n.intsAttr("dilations")) if (d != 1) unsupported(what + ": dilation");
+    if (n.intAttr("ceil_mode", 0) != 0) unsupported(what + ": ceil_mode");
+    if (func == compiler::PoolFunction::Avg && n.intAttr("count_include_pad", 0) != 0) unsupported(what + ": count_include_pad");
     unsigned py, px;
     spatialPads(n, ks[0], ks[1], 1, 1, strides[0], strides[1], py, px);
     setDevice(n, model.pool(x, static_cast<unsigned>(ks[1]), static_cast<unsigned>(ks[0]), px, py, static_cast<unsigned>(strides[1]),
-                            static_cast<unsigned>(strides[0]), compiler::PoolFunction::Max));
+                            static_cast<unsigned>(strides[0]), func));
   }
 
   void opResize(const Node &n) {
@@ -1107,7 +1110,8 @@ struct Importer {
     else if (op == "Conv") opConv(n);
     else if (op == "Relu") setDevice(n, model.activation(device(n, 0), compiler::ActivationFunction::ReLU, 0.0f));
     else if (op == "LeakyRelu") setDevice(n, model.activation(device(n, 0), compiler::ActivationFunction::LeakyReLU, n.floatAttr("alpha", 0.01f)));
-    else if (op == "MaxPool") opMaxPool(n);
+    else if (op == "MaxPool") opPool(n, compiler::PoolFunction::Max);
+    else if (op == "AveragePool") opPool(n, compiler::PoolFunction::Avg);
     else if (op == "Resize" || op == "Upsample") opResize(n);
     else if (op == "Pad") opPad(n);
     else unsupported("operator '" + op + "' (node '" + n.name + "')");

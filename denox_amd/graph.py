@@ -162,15 +162,18 @@ class Model:
         self._ops.append({"op": "upsample", "src": src.name, "dst": out.name, "factor": scale})
         return out
 
-    def pool(self, src: Tensor, kernel=(2, 2), padding=(0, 0), stride=None) -> Tensor:
+    def pool(self, src: Tensor, kernel=(2, 2), padding=(0, 0), stride=None, func: str = "max") -> Tensor:
+        """``func`` is ``"max"`` or ``"avg"`` (the window's mean, summed in fp32 and rounded once)."""
         stride = tuple(kernel) if stride is None else tuple(stride)
+        if func not in ("max", "avg"):
+            raise ValueError(f"pool: unknown function {func!r}")
         t = c_int()
-        _capi.check(_capi.lib().denox_hip_builder_pool(self._h, src.handle, kernel[1], kernel[0], padding[1], padding[0],
-                                                       stride[1], stride[0], byref(t)))
+        entry = _capi.lib().denox_hip_builder_pool if func == "max" else _capi.lib().denox_hip_builder_avg_pool
+        _capi.check(entry(self._h, src.handle, kernel[1], kernel[0], padding[1], padding[0], stride[1], stride[0], byref(t)))
         ow = (src.width + (2 * padding[1] - kernel[1])) // stride[1] + 1
         oh = (src.height + (2 * padding[0] - kernel[0])) // stride[0] + 1
         out = Tensor(self, t.value, self._name("pool"), ow, oh, src.channels)
-        self._ops.append({"op": "pool", "src": src.name, "dst": out.name, "kernel": tuple(kernel)})
+        self._ops.append({"op": "pool", "src": src.name, "dst": out.name, "kernel": tuple(kernel), "func": func})
         return out
 
     def concat(self, a: Tensor, b: Tensor) -> Tensor:

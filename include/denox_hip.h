@@ -108,6 +108,10 @@ int denox_hip_builder_activation(denox_hip_builder *b, int src, int func, float 
 int denox_hip_builder_upsample(denox_hip_builder *b, int src, uint32_t scale, int *out_tensor);            /* nearest */
 int denox_hip_builder_pool(denox_hip_builder *b, int src, uint32_t kx, uint32_t ky, uint32_t pad_x, uint32_t pad_y,
                            uint32_t stride_x, uint32_t stride_y, int *out_tensor);                          /* max */
+/* Model::pool with PoolFunction::Avg (compiler/src/denox/compiler/frontend/model/Model.cpp:150-175,
+ * common/src/denox/common/PoolFunction.hpp:7-10): the window's mean, summed in binary32 and rounded once. */
+int denox_hip_builder_avg_pool(denox_hip_builder *b, int src, uint32_t kx, uint32_t ky, uint32_t pad_x, uint32_t pad_y,
+                               uint32_t stride_x, uint32_t stride_y, int *out_tensor);
 int denox_hip_builder_concat(denox_hip_builder *b, int src0, int src1, int *out_tensor);
 int denox_hip_builder_pad(denox_hip_builder *b, int src, int64_t left_sym, int64_t right_sym, int64_t top_sym, int64_t bottom_sym, int *out_tensor); /* replicate */
 /* mode: 0 replicate the border (PaddingMode::Edge of the reference), 1 zeros (PaddingMode::Zero) */
@@ -119,8 +123,8 @@ int denox_hip_builder_output(denox_hip_builder *b, int src, const char *name);
 /* Fills an empty builder from an ONNX ModelProto held in memory: inputs (NCHW, N = 1; dynamic height / width become
  * named extents after their dim_param), layers and outputs.  Stands for denox::onnx::read
  * (compiler/src/denox/compiler/frontend/onnx/onnx.cpp:70-158), the first step of denox::compile
- * (compiler/src/denox/compiler/compile.cpp:21-61).  Operators: Conv, Relu, LeakyRelu, MaxPool, Resize / Upsample
- * (nearest, integer factor), Concat, Pad (edge), Slice, and the shape arithmetic exporters emit around them;
+ * (compiler/src/denox/compiler/compile.cpp:21-61).  Operators: Conv, Relu, LeakyRelu, MaxPool, AveragePool, Resize / Upsample
+ * (nearest, integer factor), Concat, Pad (edge, or constant 0), Slice, and the shape arithmetic exporters emit around them;
  * anything else reports DENOX_HIP_UNSUPPORTED with the operator's name. */
 int denox_hip_builder_import_onnx(denox_hip_builder *b, const void *onnx_bytes, size_t size);
 /* graph inputs / outputs of a builder, in declaration order */

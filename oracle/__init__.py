@@ -54,6 +54,7 @@ def lib() -> ctypes.CDLL:
         L.dnxo_conv2d_hwc.argtypes = [u16p, i64, i64, i64, u16p, u16p, i64, i64, i64,
                                       i64, i64, i64, i64, ctypes.c_int, f32, ctypes.c_int, u16p]
         L.dnxo_maxpool_hwc_f16.argtypes = [u16p, i64, i64, i64, i64, i64, u16p]
+        L.dnxo_avgpool_hwc_f16.argtypes = [u16p, i64, i64, i64, i64, i64, u16p]
         L.dnxo_upsample_nearest_hwc_f16.argtypes = [u16p, i64, i64, i64, i64, u16p]
         L.dnxo_copy_channels_hwc_f16.argtypes = [u16p, i64, i64, i64, i64, u16p, i64, i64, i64]
         L.dnxo_concat_hwc_f16.argtypes = [u16p, i64, u16p, i64, i64, i64, u16p]
@@ -138,6 +139,14 @@ def maxpool(x: np.ndarray, k: Sequence[int] = (2, 2)) -> np.ndarray:
     H, W, C = xin.shape
     out = np.empty((H // k[0], W // k[1], C), np.float16)
     _check(lib().dnxo_maxpool_hwc_f16(_p(xin), H, W, C, k[0], k[1], _p(out)), "maxpool")
+    return out
+
+
+def avgpool(x: np.ndarray, k: Sequence[int] = (2, 2)) -> np.ndarray:
+    xin = _c(x, np.float16)
+    H, W, C = xin.shape
+    out = np.empty((H // k[0], W // k[1], C), np.float16)
+    _check(lib().dnxo_avgpool_hwc_f16(_p(xin), H, W, C, k[0], k[1], _p(out)), "avgpool")
     return out
 
 
@@ -275,12 +284,14 @@ def run_graph(ops: Sequence[dict], inputs: Dict[str, np.ndarray], mode: str = "f
             elif kind == "pool":
                 x = env[src]
                 k = op.get("kernel", (2, 2))
+                avg = op.get("func", "max") == "avg"
                 if f16:
-                    env[op["dst"]] = maxpool(x, k)
+                    env[op["dst"]] = avgpool(x, k) if avg else maxpool(x, k)
                 else:
                     H, W, C = x.shape
                     Ho, Wo = H // k[0], W // k[1]
-                    env[op["dst"]] = x[:Ho * k[0], :Wo * k[1]].reshape(Ho, k[0], Wo, k[1], C).max(axis=(1, 3))
+                    win = x[:Ho * k[0], :Wo * k[1]].reshape(Ho, k[0], Wo, k[1], C)
+                    env[op["dst"]] = win.mean(axis=(1, 3), dtype=np.float32) if avg else win.max(axis=(1, 3))
             elif kind == "upsample":
                 x = env[src]
                 f = op.get("factor", 2)

@@ -16,6 +16,7 @@
  *   dnxo_f32_to_f16 / dnxo_f16_to_f32      pinned: numpy float16 casts, all 65536 patterns
  *   dnxo_conv2d_hwc                        pinned: F.conv2d fp32, identity tap, all-ones, fp64 brute force
  *   dnxo_maxpool_hwc_f16                   pinned: F.max_pool2d, membership invariant
+ *   dnxo_avgpool_hwc_f16                   pinned: F.avg_pool2d (exact on 2x2 windows, <= 1 ulp otherwise), constant input
  *   dnxo_upsample_nearest_hwc_f16          pinned: F.interpolate(mode="nearest")
  *   dnxo_concat_hwc_f16 / dnxo_copy_channels_hwc_f16   pinned: torch.cat
  *   dnxo_pad_replicate_hwc_f16             pinned: F.pad(mode="replicate")
@@ -271,6 +272,34 @@ static inline int f16_gt(uint16_t a, uint16_t b) { /* a > b for finite/inf value
   if (sa != sb)
     return sb; /* a positive, b negative */
   return sa ? (ma < mb) : (ma > mb);
+}
+
+/* Average pool, kernel == stride, no padding.  The reference carries the
+ * function in its model (common/src/denox/common/PoolFunction.hpp:7-10,
+ * frontend/onnx/details/ops/average_pool.cpp:154) but has no shader for it
+ * (BasicPoolShader.cpp:170), so the arithmetic is this build's own contract:
+ * sum the window in binary32 in row-major order, multiply by the binary32
+ * constant 1/(ky*kx), round once to binary16. */
+DNXO_API int dnxo_avgpool_hwc_f16(const uint16_t *in, int64_t H, int64_t W,
+                                  int64_t C, int64_t ky, int64_t kx,
+                                  uint16_t *out) {
+  if (ky <= 0 || kx <= 0)
+    return -1;
+  const int64_t Ho = H / ky, Wo = W / kx;
+  const float inv = 1.0f / (float)(kx * ky);
+#pragma omp parallel for schedule(static)
+  for (int64_t oh = 0; oh < Ho; ++oh)
+    for (int64_t ow = 0; ow < Wo; ++ow)
+      for (int64_t c = 0; c < C; ++c) {
+        float sum = 0.0f;
+        for (int64_t r = 0; r < ky; ++r)
+          for (int64_t s = 0; s < kx; ++s) {
+            const float v = dnxo_f16_to_f32(in[((oh * ky + r) * W + (ow * kx + s)) * C + c]);
+            sum = (r == 0 && s == 0) ? v : sum + v;
+          }
+        out[(oh * Wo + ow) * C + c] = dnxo_f32_to_f16(sum * inv);
+      }
+  return 0;
 }
 
 DNXO_API int dnxo_maxpool_hwc_f16(const uint16_t *in, int64_t H, int64_t W,

@@ -459,6 +459,34 @@ def test_bandwidth_kernels_store_in_place(oracle, C0, C1):
         assert_bits_equal(g, want[t.name], "in place against the oracle")
 
 
+@pytest.mark.parametrize("C,k", [(3, (2, 2)), (8, (2, 2)), (64, (2, 2)), (16, (3, 3)), (9, (2, 3)), (32, (4, 4))])
+def test_average_pool(oracle, C, k):
+    """Average pool (sum in fp32 in window order, times 1/(ky*kx), one rounding): bit-exact against the oracle routine alone,
+    behind a conv (whose epilogue folds only the maximum, so the pool stays a dispatch) and written in place into a concat."""
+    rng = np.random.default_rng(C + k[0])
+    H, W = 37, 50
+    x = rng.standard_normal((H, W, C)).astype(np.float16)
+    m = dx.Model()
+    inp = m.input("input", "W", "H", C)
+    a = m.pool(inp, k, func="avg")
+    c = m.relu(m.conv2d(inp, he_weights(rng, 16, C), small_bias(rng, 16)))
+    q = m.pool(c, k, func="avg")
+    cat = m.concat(m.pool(inp, k, func="avg"), m.pool(inp, k, func="max"))
+    for t in (a, q, cat):
+        m.output(t)
+    mod = dx.Module.compile(m)
+    names = [d_["name"] for d_ in dx.describe(mod.dnx, H=H, W=W)["dispatches"]]
+    assert "conv3x3+relu" in names and "conv3x3+relu+maxpool" not in names and names.count("avgpool") + names.count("avgpool+concat") == 3
+    got_a, got_q, got_cat = mod.instance(H=H, W=W).infer(x)
+    ops = m.to_ops({"H": H, "W": W})
+    want = oracle.run_graph(ops, {"input": x}, "f16")
+    assert got_a.shape == (H // k[0], W // k[1], C)
+    assert_bits_equal(got_a, want[a.name], "average pool")
+    assert_bits_equal(got_cat, want[cat.name], "average pool into a concat")
+    # behind the conv: the mean of the fp32-evaluated conv outputs, within the conv tolerance
+    assert_conv_close(got_q, oracle.run_graph(ops, {"input": x}, "fp32")[q.name], "average pool behind a conv")
+
+
 @pytest.mark.parametrize("C", [3, 8, 9, 64])
 def test_zero_padding(oracle, C):
     """Pad with zeros (F.pad mode="constant"): a dispatch of its own (the conv loaders fold only the replicate mode), bit-exact

@@ -201,6 +201,23 @@ def test_one_by_one_and_five_by_five_convs_import():
     assert e.value.status == 5
 
 
+def test_average_pool_imports_as_its_own_dispatch():
+    """AveragePool (the reference imports it, frontend/onnx/details/ops/average_pool.cpp:9-156, and then finds no shader):
+    a dispatch of its own -- the conv epilogue folds only the 2x2 maximum -- and the attributes the reference refuses
+    are refused."""
+    ap = lambda *extra: conv_model([node("Relu", ["c"], ["r"]), node("AveragePool", ["r"], ["y"], attr_ints("kernel_shape", [2, 2]), attr_ints("strides", [2, 2]), *extra, name="ap0")],
+                                   "y", (1, 8, "h", "w"))
+    blob = dx.compile_model(dx.Model.from_onnx(ap()))
+    d = dx.describe(blob, H=10, W=21)
+    assert [x["name"] for x in d["dispatches"]] == ["conv3x3+relu", "avgpool"] and "AVG=1" in d["dispatches"][1]["debug_info"]
+    out = d["tensors"][d["outputs"][0]]
+    assert (out["height"], out["width"], out["channels"]) == (5, 10, 8)
+    for extra, word in [(attr_int("count_include_pad", 1), "count_include_pad"), (attr_int("ceil_mode", 1), "ceil_mode")]:
+        with pytest.raises(dx.DenoxHipError) as e:
+            dx.Model.from_onnx(ap(extra))
+        assert e.value.status == 5 and word in str(e.value) and "ap0" in str(e.value)
+
+
 def test_unsupported_and_malformed_models_are_reported():
     with pytest.raises(dx.DenoxHipError) as e:
         dx.Model.from_onnx(conv_model([node("Softmax", ["c"], ["y"], name="sm0")], "y", (1, 8, "h", "w")))

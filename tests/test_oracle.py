@@ -165,6 +165,27 @@ def test_maxpool_vs_torch(oracle, H, W, C):
         assert np.all((win.view(np.uint16) == got.view(np.uint16)[:, None, :, None, :]).any(axis=(1, 3)))
 
 
+@pytest.mark.parametrize("H,W,C,k", [(8, 8, 3, (2, 2)), (9, 7, 16, (2, 2)), (12, 15, 8, (3, 3)), (11, 14, 24, (2, 3)), (1, 5, 8, (2, 2))])
+def test_avgpool_vs_torch(oracle, H, W, C, k):
+    """The mean of a window, one rounding.  Four binary16 values of like magnitude sum exactly in binary32 and 1/4 is a power
+    of two, so a 2x2 window must agree with F.avg_pool2d bit for bit; other windows may differ from it by the summation order
+    and the reciprocal, which a float64 evaluation bounds at one binary16 ulp.  A constant image must come back unchanged."""
+    rng = np.random.default_rng(H * W + C)
+    x = (rng.uniform(0.5, 2.0, (H, W, C)) * rng.choice([-1.0, 1.0], (H, W, C))).astype(np.float16)
+    got = oracle.avgpool(x, k)
+    assert got.shape == (H // k[0], W // k[1], C)
+    if not got.size:
+        return
+    if k == (2, 2):
+        want = nchw_to_hwc(F.avg_pool2d(hwc_to_nchw(x.astype(np.float32)), 2)).astype(np.float16)
+        assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    want64 = nchw_to_hwc(F.avg_pool2d(hwc_to_nchw(x.astype(np.float64)), k))
+    ulp = np.spacing(np.abs(want64).astype(np.float16)).astype(np.float64)
+    assert np.all(np.abs(got.astype(np.float64) - want64) <= ulp)
+    const = np.full((H, W, C), 0.3, np.float16)
+    assert np.array_equal(oracle.avgpool(const, k).view(np.uint16), const[:H // k[0], :W // k[1]].view(np.uint16))
+
+
 @pytest.mark.parametrize("H,W,C,f", [(4, 5, 3, 2), (7, 3, 16, 2), (3, 3, 9, 3), (1, 1, 8, 2)])
 def test_upsample_vs_torch(oracle, H, W, C, f):
     rng = np.random.default_rng(H + W + C)
