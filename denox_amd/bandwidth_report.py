@@ -1,6 +1,6 @@
 """Per-kernel bandwidth of the stand-alone data-movement kernels at benchmark extents.
 
-`python -m denox_amd.bandwidth_report [H W]` builds one-layer models (max pool, upsample, concat, ReLU, pad, slice,
+`python -m denox_amd.bandwidth_report [H W [C ...]]` builds one-layer models (max pool, upsample, concat, ReLU, pad, slice,
 layout conversion), times each dispatch with hipEvents (Instance.bench) and prints achieved GB/s against the
 8 TB/s HBM peak, using the byte counts the dispatches carry (reads + writes of the tensors as stored).
 """
@@ -19,21 +19,21 @@ def cases(C):
     def relu(m, x): return m.relu(x)
     def pad(m, x): return m.pad(x, 0, 0, 0, 8)
     def crop(m, x): return m.slice(x, 0, x.width, 0, x.height - 8)
-    def cat(m, x): return m.concat(x, x)
+    def cat(m, x): return m.concat(x, m.input("other", "W", "H", C))
     return [("maxpool", pool, 1), ("upsample", up, 2), ("relu", relu, 1), ("pad", pad, 1), ("slice", crop, 1), ("concat", cat, 1)]
 
 
-def main(H=1088, W=1920):
+def main(H=1088, W=1920, channels=(64, 32, 8, 9, 3)):
     rng = np.random.default_rng(0)
     print(f"{'kernel':<28}{'C':>4}{'extent':>12}{'ms':>9}{'GB/s':>8}{'of HBM peak':>13}")
     no_fusion = dict(conv_relu_fusion=False, concat_conv_fusion=False, upsample_fusion=False, pool_fusion=False, pad_fusion=False, slice_fusion=False)
-    for C in (64, 32, 9, 3):
+    for C in channels:
         for name, fn, shrink in cases(C):
             h, w = H // shrink, W // shrink
             m = dx.Model()
             m.output(fn(m, m.input("input", "W", "H", C)))
             inst = dx.Module.compile(m, features=no_fusion).instance(H=h, W=w)
-            inst.infer(rng.standard_normal((h, w, C)).astype(np.float16))
+            inst.infer(*[rng.standard_normal((h, w, C)).astype(np.float16) for _ in range(inst.input_count)])
             reps = 5
             acc = {}
             for _ in range(reps):
@@ -55,4 +55,5 @@ def main(H=1088, W=1920):
 
 
 if __name__ == "__main__":
-    main(*(int(a) for a in sys.argv[1:3]))
+    args = [int(a) for a in sys.argv[1:]]
+    main(*args[:2], **({"channels": tuple(args[2:])} if len(args) > 2 else {}))

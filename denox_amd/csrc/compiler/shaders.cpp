@@ -515,6 +515,15 @@ private:
 
 // ------------------------------------------------------------------ bandwidth kernels
 // grid.x: workgroups covering one row of w * vectorsPerPixel vectors; grid.y: the rows
+// threads per pixel of a bandwidth kernel: one per full chunk of 8 channels; with vec == 1 the thread of the last full
+// chunk also moves the partial one behind it (DNX_CHUNKS of the kernels)
+unsigned chunksPerPixel(unsigned channels, unsigned vec) { return vec == 8 || channels >= 8 ? channels / 8 : 1; }
+
+// rows of the iteration space per thread (RPT of the bandwidth kernels): narrow, unaligned pixels need several loads in
+// flight per thread to cover the memory latency
+unsigned rowsPerThread(unsigned vec) { return vec == 8 ? 1 : 4; }
+Sym rowBlocks(SymGraph &sym, Sym rows, unsigned rpt) { return rpt == 1 ? rows : sym.cdiv(rows, rpt); }
+
 Sym rowGrid(SymGraph &sym, Sym w, unsigned vectorsPerPixel) {
   return sym.cdiv(sym.mul(w, static_cast<int64_t>(vectorsPerPixel)), WG_BANDWIDTH);
 }
@@ -591,7 +600,7 @@ public:
     defineOutput(k, place);
     const std::string entry = std::string(avg ? "pool_avg_c" : "pool_max_c") + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, in.channels / vec), out.height, Sym::Const(1), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, chunksPerPixel(in.channels, vec)), out.height, Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     bindOutput(d, sym, model, m, place);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
@@ -611,10 +620,12 @@ public:
     const unsigned vec = place.vec;
     auto k = m_compiler->read("upsample.hip");
     k.define("CH", in.channels); k.define("SCALE", op.scale); k.define("VEC", vec);
+    const unsigned rpt = rowsPerThread(vec);
+    if (rpt > 1) k.define("RPT", rpt);
     defineOutput(k, place);
     const std::string entry = "upsample_c" + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, rowGrid(sym, in.width, in.channels / vec), in.height, Sym::Const(1), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, chunksPerPixel(in.channels, vec)), rowBlocks(sym, in.height, rpt), Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     bindOutput(d, sym, model, m, place);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
@@ -627,7 +638,8 @@ class CopyTransformShader final : public SingleOpShader {
 public:
   explicit CopyTransformShader(const hip::HipCompiler *c) : SingleOpShader(c, OpKind::Concat) {}
   std::string name() const override { return "copy_transform"; }
-  // Explicit concat: one strided channel copy per source (CopyTransformShader.cpp:437-537).
+  // Explicit concat: the reference issues one strided channel copy per source (CopyTransformShader.cpp:437-537); here
+  // both copies are one launch that writes whole pixels, and the one-source copy serves the in-place mixes below.
   // Implicit concat: the reference aliases two channel-block-major (CHWC8) sources behind one another and needs no
   // dispatch (CopyTransformShader.cpp:198-237, OpImpl.cpp:43-65).  Activations here are pixel-major, where the
   // sources interleave per pixel; the same saving comes from the producer side instead: a source whose only
@@ -653,9 +665,28 @@ public:
     const TensorNode &out = model.tensors()[m.output];
     unsigned off = 0;
     impl.edge().config = m.inputVariants.empty() ? "copy" : std::string(m.inputVariants[0] ? "in-place" : "copy") + "/" + (m.inputVariants[1] ? "in-place" : "copy");
+    if (m.inputVariants.empty()) { // both sources are copied: one launch that writes whole pixels
+      const TensorNode &a = model.tensors()[m.inputs[0]], &b = model.tensors()[m.inputs[1]];
+      const unsigned vec = (a.channels % 8 == 0 && b.channels % 8 == 0) ? 8 : 1;
+      auto k = m_compiler->read("copy_transform.hip");
+      k.define("COUNT", a.channels); k.define("COUNT1", b.channels); k.define("VEC", vec);
+      const unsigned rpt = rowsPerThread(vec);
+      if (rpt > 1) k.define("RPT", rpt);
+      const std::string entry = "concat_c" + std::to_string(a.channels) + "_c" + std::to_string(b.channels) + "v" + std::to_string(vec);
+      k.define("KERNEL_NAME", entry);
+      auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, chunksPerPixel(a.channels, vec) + chunksPerPixel(b.channels, vec)),
+                                     rowBlocks(sym, out.height, rpt), Sym::Const(1), WG_BANDWIDTH);
+      d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
+      d.addBinding(dnx::Access::ReadOnly, m.inputs[1]);
+      d.addBinding(dnx::Access::WriteOnly, m.output);
+      d.addPushConstant(out.width); d.addPushConstant(out.height);
+      d.setName("concat-copy"); d.setOperation("concat"); d.setConfig("vec" + std::to_string(vec));
+      d.setMemoryReads(bytesOf(sym, out)); d.setMemoryWrites(bytesOf(sym, out)); d.setFlops(Sym::Const(0));
+      return;
+    }
     for (int s = 0; s < 2; ++s) {
       const TensorNode &in = model.tensors()[m.inputs[s]];
-      if (!m.inputVariants.empty() && m.inputVariants[static_cast<size_t>(s)]) { // already where it belongs
+      if (m.inputVariants[static_cast<size_t>(s)]) { // already where it belongs
         impl.createViewConstrain(m.inputs[s], m.output, static_cast<uint64_t>(off) * 2);
         off += in.channels;
         continue;
@@ -664,9 +695,11 @@ public:
       auto k = m_compiler->read("copy_transform.hip");
       k.define("IN_CH", in.channels); k.define("IN_CH_OFFSET", 0); k.define("OUT_CH", out.channels); k.define("OUT_CH_OFFSET", off);
       k.define("COUNT", in.channels); k.define("VEC", vec);
+      const unsigned rpt = rowsPerThread(vec);
+      if (rpt > 1) k.define("RPT", rpt);
       const std::string entry = "copy_c" + std::to_string(in.channels) + "_to_c" + std::to_string(out.channels) + "o" + std::to_string(off) + "v" + std::to_string(vec);
       k.define("KERNEL_NAME", entry);
-      auto d = impl.registerDispatch(k, entry, rowGrid(sym, in.width, in.channels / vec), in.height, Sym::Const(1), WG_BANDWIDTH);
+      auto d = impl.registerDispatch(k, entry, rowGrid(sym, in.width, chunksPerPixel(in.channels, vec)), rowBlocks(sym, in.height, rpt), Sym::Const(1), WG_BANDWIDTH);
       d.addBinding(dnx::Access::ReadOnly, m.inputs[s]);
       d.addBinding(dnx::Access::WriteOnly, m.output);
       d.addPushConstant(in.width); d.addPushConstant(in.height);
@@ -689,10 +722,12 @@ public:
     auto k = m_compiler->read("activation.hip");
     k.define("CH", in.channels); k.define("VEC", vec); k.define("ACT", op.func == ActivationFunction::ReLU ? 1 : 2);
     if (op.func == ActivationFunction::LeakyReLU) k.define("ALPHA", fmtFloat(op.alpha));
+    const unsigned rpt = rowsPerThread(vec);
+    if (rpt > 1) k.define("RPT", rpt);
     defineOutput(k, place);
     const std::string entry = std::string(op.func == ActivationFunction::ReLU ? "relu_c" : "leaky_relu_c") + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, rowGrid(sym, in.width, in.channels / vec), in.height, Sym::Const(1), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, rowGrid(sym, in.width, chunksPerPixel(in.channels, vec)), rowBlocks(sym, in.height, rpt), Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     bindOutput(d, sym, model, m, place);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
@@ -716,10 +751,12 @@ public:
     k.define("CH", in.channels); k.define("VEC", vec);
     const bool zeros = op.padMode == PaddingMode::Zero;
     if (zeros) k.define("ZERO", 1);
+    const unsigned rpt = rowsPerThread(vec);
+    if (rpt > 1) k.define("RPT", rpt);
     defineOutput(k, place);
     const std::string entry = std::string(zeros ? "memory_pad_zero_c" : "memory_pad_c") + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, in.channels / vec), out.height, Sym::Const(1), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, chunksPerPixel(in.channels, vec)), rowBlocks(sym, out.height, rpt), Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     bindOutput(d, sym, model, m, place);
     d.addPushConstant(out.width); d.addPushConstant(out.height);
@@ -740,10 +777,12 @@ public:
     const unsigned vec = place.vec;
     auto k = m_compiler->read("slice.hip");
     k.define("CH", in.channels); k.define("VEC", vec);
+    const unsigned rpt = rowsPerThread(vec);
+    if (rpt > 1) k.define("RPT", rpt);
     defineOutput(k, place);
     const std::string entry = "memory_slice_c" + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, in.channels / vec), out.height, Sym::Const(1), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, chunksPerPixel(in.channels, vec)), rowBlocks(sym, out.height, rpt), Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     bindOutput(d, sym, model, m, place);
     d.addPushConstant(op.top); d.addPushConstant(op.left);

@@ -20,19 +20,24 @@ __device__ DNX_INLINE _Float16 act1(_Float16 v) {
 }
 extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
     const ushort_t *__restrict__ IN, ushort_t *__restrict__ OUT, PushConstants pc) {
-  constexpr unsigned CV = CH / VEC;
+  constexpr unsigned CV = DNX_CHUNKS(CH);
   const unsigned i = DNX_ROW_INDEX();
   if (i >= pc.W * CV) return;
-  const size_t idx = ((size_t)DNX_BID_Y * pc.W * CV + i) * VEC;
   const unsigned w = i / CV, cv = i - w * CV;
-  const size_t odx = OPITCH == CH ? idx : ((size_t)DNX_BID_Y * pc.W + w) * OPITCH + cv * VEC;
-  const vec_t v = ldv(IN + idx);
-#if VEC == 8
-  half8 a = __builtin_bit_cast(half8, v);
+  const unsigned h0 = DNX_BID_Y * RPT;
+  chunk_t v[RPT];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) a[e] = act1(a[e]);
-  stv(OUT + odx, __builtin_bit_cast(uint4v, a));
-#else
-  stv(OUT + odx, __builtin_bit_cast(ushort_t, act1(__builtin_bit_cast(_Float16, v))));
-#endif
+  for (unsigned u = 0; u < RPT; ++u) {
+    const size_t pix = (size_t)(h0 + u < pc.H ? h0 + u : pc.H - 1) * pc.W + w;
+    v[u] = ld_chunk<CH>(IN + pix * CH, cv);
+  }
+#pragma unroll
+  for (unsigned u = 0; u < RPT; ++u) {
+    if (h0 + u >= pc.H) break;
+    const size_t pix = (size_t)(h0 + u) * pc.W + w;
+    half8 a = __builtin_bit_cast(half8, v[u].a), b = __builtin_bit_cast(half8, v[u].b);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) a[e] = act1(a[e]), b[e] = act1(b[e]);
+    st_chunk<CH>(OUT + pix * OPITCH, cv, chunk_t{__builtin_bit_cast(uint4v, a), __builtin_bit_cast(uint4v, b)});
+  }
 }

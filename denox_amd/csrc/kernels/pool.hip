@@ -23,55 +23,43 @@ __device__ DNX_INLINE float rounded_f32(float x) {
 #endif
 extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
     const ushort_t *__restrict__ IN, ushort_t *__restrict__ OUT, PushConstants pc) {
-  constexpr unsigned CV = CH / VEC;
+  constexpr unsigned CV = DNX_CHUNKS(CH);
   const unsigned W2 = pc.W / KX;
   const unsigned oh = DNX_BID_Y;
   const unsigned i = DNX_ROW_INDEX();
   if (i >= W2 * CV) return;
   const unsigned ow = i / CV, cv = i - ow * CV;
-  const ushort_t *src = IN + ((size_t)(oh * KY) * pc.W + (size_t)ow * KX) * CH + cv * VEC;
+  const ushort_t *src = IN + ((size_t)(oh * KY) * pc.W + (size_t)ow * KX) * CH;
 #ifdef AVG
-  float sum[VEC];
+  float sumA[8], sumB[8];
 #pragma unroll
   for (int r = 0; r < KY; ++r)
 #pragma unroll
     for (int s = 0; s < KX; ++s) {
-      const vec_t v = ldv(src + ((size_t)r * pc.W + s) * CH);
-#if VEC == 8
-      const half8 h = __builtin_bit_cast(half8, v);
+      const chunk_t c = ld_chunk<CH>(src + ((size_t)r * pc.W + s) * CH, cv);
+      const half8 ha = __builtin_bit_cast(half8, c.a), hb = __builtin_bit_cast(half8, c.b);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) sum[e] = (r == 0 && s == 0) ? (float)h[e] : sum[e] + (float)h[e];
-#else
-      const float f = (float)__builtin_bit_cast(_Float16, v);
-      sum[0] = (r == 0 && s == 0) ? f : sum[0] + f;
-#endif
+      for (int e = 0; e < 8; ++e) {
+        sumA[e] = (r == 0 && s == 0) ? (float)ha[e] : sumA[e] + (float)ha[e];
+        sumB[e] = (r == 0 && s == 0) ? (float)hb[e] : sumB[e] + (float)hb[e];
+      }
     }
   constexpr float inv = 1.0f / (float)(KX * KY);
-#if VEC == 8
-  half8 o;
+  half8 oa, ob;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) o[e] = (_Float16)rounded_f32(sum[e] * inv);
-  const vec_t acc = __builtin_bit_cast(uint4v, o);
+  for (int e = 0; e < 8; ++e) oa[e] = (_Float16)rounded_f32(sumA[e] * inv), ob[e] = (_Float16)rounded_f32(sumB[e] * inv);
+  const chunk_t acc = {__builtin_bit_cast(uint4v, oa), __builtin_bit_cast(uint4v, ob)};
 #else
-  const vec_t acc = __builtin_bit_cast(ushort_t, (_Float16)rounded_f32(sum[0] * inv));
-#endif
-#else
-  vec_t acc = ldv(src);
+  chunk_t acc = ld_chunk<CH>(src, cv);
 #pragma unroll
   for (int r = 0; r < KY; ++r)
 #pragma unroll
     for (int s = 0; s < KX; ++s) {
       if (r == 0 && s == 0) continue;
-      const vec_t v = ldv(src + ((size_t)r * pc.W + s) * CH);
-#if VEC == 8
-      half8 a = __builtin_bit_cast(half8, acc), b = __builtin_bit_cast(half8, v);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) a[e] = b[e] > a[e] ? b[e] : a[e];
-      acc = __builtin_bit_cast(uint4v, a);
-#else
-      acc = max_keep_first(acc, v);
-#endif
+      const chunk_t c = ld_chunk<CH>(src + ((size_t)r * pc.W + s) * CH, cv);
+      acc.a = max_keep_first(acc.a, c.a);
+      acc.b = max_keep_first(acc.b, c.b);
     }
 #endif
-  stv(OUT + ((size_t)oh * W2 + ow) * OPITCH + cv * VEC, acc);
+  st_chunk<CH>(OUT + ((size_t)oh * W2 + ow) * OPITCH, cv, acc);
 }

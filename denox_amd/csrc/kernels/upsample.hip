@@ -1,8 +1,11 @@
 // upsample.hip -- nearest-neighbour upsample by SCALE, HWC binary16.
 // Replaces compiler/src/denox/compiler/implement/shaders/upsample/basic_upsample.comp:27-166:
 //   out[h2, w2, c] = in[h2 / SCALE, w2 / SCALE, c].
-// Definitions: CH, SCALE, VEC.  One thread per *input* vector (grid.y = input rows); it writes
-// the SCALE x SCALE replicas, so every input byte is fetched once.
+// Definitions: CH, SCALE, VEC.  One thread per chunk of an *output* row segment, grid.y = input rows: it loads the
+// source chunk (the SCALE threads that share one are neighbours in a wave, so the load is one fetch) and stores it into
+// the SCALE output rows that replicate the input row.  Every store instruction of a wave then covers a contiguous run of
+// an output row; with threads mapped over the input the replicas along x were separate instructions that each wrote
+// every other pixel, which left narrow pixels' cache lines half written.
 #include "common.h"
 #ifndef KERNEL_NAME
 #define KERNEL_NAME upsample_nearest
@@ -10,16 +13,24 @@
 struct PushConstants { unsigned int W, H; }; // input extent
 extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
     const ushort_t *__restrict__ IN, ushort_t *__restrict__ OUT, PushConstants pc) {
-  constexpr unsigned CV = CH / VEC;
-  const unsigned h = DNX_BID_Y;
+  constexpr unsigned CV = DNX_CHUNKS(CH);
+  const unsigned h0 = DNX_BID_Y * RPT;
   const unsigned i = DNX_ROW_INDEX();
-  if (i >= pc.W * CV) return;
-  const unsigned w = i / CV, cv = i - w * CV;
-  const vec_t v = ldv(IN + ((size_t)h * pc.W + w) * CH + cv * VEC);
+  if (i >= pc.W * SCALE * CV) return;
+  const unsigned w2 = i / CV, cv = i - w2 * CV;
+  const unsigned w = w2 / SCALE;
+  chunk_t v[RPT];
+#pragma unroll
+  for (unsigned u = 0; u < RPT; ++u) {
+    const unsigned h = h0 + u < pc.H ? h0 + u : pc.H - 1;
+    v[u] = ld_chunk<CH>(IN + ((size_t)h * pc.W + w) * CH, cv);
+  }
   const size_t W2 = (size_t)pc.W * SCALE;
 #pragma unroll
-  for (int r = 0; r < SCALE; ++r)
+  for (unsigned u = 0; u < RPT; ++u) {
+    const unsigned h = h0 + u;
+    if (h >= pc.H) break;
 #pragma unroll
-    for (int s = 0; s < SCALE; ++s)
-      stv(OUT + (((size_t)h * SCALE + r) * W2 + (size_t)w * SCALE + s) * OPITCH + cv * VEC, v);
+    for (int r = 0; r < SCALE; ++r) st_chunk<CH>(OUT + (((size_t)h * SCALE + r) * W2 + w2) * OPITCH, cv, v[u]);
+  }
 }

@@ -81,8 +81,7 @@ def test_fusion_switches_change_the_schedule():
     m, _ = networks.build("tiny_unet")
     none = dict(conv_relu_fusion=False, concat_conv_fusion=False, upsample_fusion=False, pool_fusion=False)
     names = _dispatch_names(dx.compile_model(m, features=dict(none, implicit_concat=False)), H=64, W=64)
-    assert names == ["conv3x3", "relu", "maxpool", "conv3x3", "relu", "upsample", "concat-copy-src0", "concat-copy-src1",
-                     "conv3x3", "relu", "conv3x3"]
+    assert names == ["conv3x3", "relu", "maxpool", "conv3x3", "relu", "upsample", "concat-copy", "conv3x3", "relu", "conv3x3"]
     # the upsampled tensor is read by the concat only: the upsample stores straight into the concat's tensor; the skip
     # tensor is also read by the pool and keeps its copy
     names = _dispatch_names(dx.compile_model(m, features=none), H=64, W=64)
@@ -154,9 +153,11 @@ def test_concat_sources_are_placed_inside_the_result():
     assert (by_c[16]["offset"], by_c[24]["offset"]) == (0, 32)  # channel 16 of pixel 0
     assert by_c[24]["size"] == out["size"] - 32 and out["size"] == 20 * 30 * 40 * 2
     assert len(d["buffers"]) == 2 + 2  # input, result, two weight blobs: no buffer is left for the sources
-    # switched off: the convs write tensors of their own and two copies follow
+    # switched off: the convs write tensors of their own and one launch copies both into whole pixels
     d = dx.describe(dx.compile_model(m, conv_config="w4r2k16", features={"implicit_concat": False}), H=20, W=30)
-    assert [x_["name"] for x_ in d["dispatches"]] == ["conv3x3", "conv3x3+relu", "concat-copy-src0", "concat-copy-src1"]
+    assert [x_["name"] for x_ in d["dispatches"]] == ["conv3x3", "conv3x3+relu", "concat-copy"]
+    cat = d["dispatches"][2]
+    assert cat["memory_reads"] == cat["memory_writes"] == out["size"] and len(cat["bindings"]) == 3
 
 
 def test_concat_sources_that_cannot_move():
@@ -173,7 +174,7 @@ def test_concat_sources_that_cannot_move():
     blob = dx.compile_model(m, conv_config="w4r2k16")
     assert "in-place" not in dx.last_compile_report()
     d = dx.describe(blob, H=16, W=16)
-    assert sum(x_["name"].startswith("concat-copy") for x_ in d["dispatches"]) == 4
+    assert sum(x_["name"] == "concat-copy" for x_ in d["dispatches"]) == 2
     m = dx.Model()
     x = m.input("input", "W", "H", 8)
     a = m.conv2d(x, _w(rng, 8, 8))
@@ -348,7 +349,9 @@ def test_measured_latencies_drive_the_selection(tmp_path):
         for _ in range(3):
             db.add_sample(i, lat)
     names = _dispatch_names(dx.compile_model(m, assume={"H": 64, "W": 64}, conv_config="w4r2k16", db=db), H=64, W=64)
-    assert "upsample+concat" in names and "concat-copy-src1" in names and not any(n.startswith("concat+") for n in names)
+    # (upsample, then one launch copying both sources) and (upsample stored in place, then a copy of the other source) cost the same here
+    assert ("upsample" in names and "concat-copy" in names) or ("upsample+concat" in names and "concat-copy-src1" in names)
+    assert not any(n.startswith("concat+") for n in names)
     assert "measured" in dx.last_compile_report()
     # without a table the roofline estimate prefers the fused kernel
     names = _dispatch_names(dx.compile_model(m, assume={"H": 64, "W": 64}, conv_config="w4r2k16"), H=64, W=64)
