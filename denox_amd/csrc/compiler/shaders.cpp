@@ -519,8 +519,7 @@ private:
 // chunk also moves the partial one behind it (DNX_CHUNKS of the kernels)
 unsigned chunksPerPixel(unsigned channels, unsigned vec) { return vec == 8 || channels >= 8 ? channels / 8 : 1; }
 
-// rows of the iteration space per thread (RPT of the bandwidth kernels): narrow, unaligned pixels need several loads in
-// flight per thread to cover the memory latency
+// rows per thread of the two-source concat kernel (its RPT): several loads in flight help it on unaligned pixels
 unsigned rowsPerThread(unsigned vec) { return vec == 8 ? 1 : 4; }
 Sym rowBlocks(SymGraph &sym, Sym rows, unsigned rpt) { return rpt == 1 ? rows : sym.cdiv(rows, rpt); }
 
@@ -620,12 +619,10 @@ public:
     const unsigned vec = place.vec;
     auto k = m_compiler->read("upsample.hip");
     k.define("CH", in.channels); k.define("SCALE", op.scale); k.define("VEC", vec);
-    const unsigned rpt = rowsPerThread(vec);
-    if (rpt > 1) k.define("RPT", rpt);
     defineOutput(k, place);
     const std::string entry = "upsample_c" + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, chunksPerPixel(in.channels, vec)), rowBlocks(sym, in.height, rpt), Sym::Const(1), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, chunksPerPixel(in.channels, vec)), in.height, Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     bindOutput(d, sym, model, m, place);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
@@ -695,11 +692,9 @@ public:
       auto k = m_compiler->read("copy_transform.hip");
       k.define("IN_CH", in.channels); k.define("IN_CH_OFFSET", 0); k.define("OUT_CH", out.channels); k.define("OUT_CH_OFFSET", off);
       k.define("COUNT", in.channels); k.define("VEC", vec);
-      const unsigned rpt = rowsPerThread(vec);
-      if (rpt > 1) k.define("RPT", rpt);
       const std::string entry = "copy_c" + std::to_string(in.channels) + "_to_c" + std::to_string(out.channels) + "o" + std::to_string(off) + "v" + std::to_string(vec);
       k.define("KERNEL_NAME", entry);
-      auto d = impl.registerDispatch(k, entry, rowGrid(sym, in.width, chunksPerPixel(in.channels, vec)), rowBlocks(sym, in.height, rpt), Sym::Const(1), WG_BANDWIDTH);
+      auto d = impl.registerDispatch(k, entry, rowGrid(sym, in.width, chunksPerPixel(in.channels, vec)), in.height, Sym::Const(1), WG_BANDWIDTH);
       d.addBinding(dnx::Access::ReadOnly, m.inputs[s]);
       d.addBinding(dnx::Access::WriteOnly, m.output);
       d.addPushConstant(in.width); d.addPushConstant(in.height);
@@ -722,12 +717,10 @@ public:
     auto k = m_compiler->read("activation.hip");
     k.define("CH", in.channels); k.define("VEC", vec); k.define("ACT", op.func == ActivationFunction::ReLU ? 1 : 2);
     if (op.func == ActivationFunction::LeakyReLU) k.define("ALPHA", fmtFloat(op.alpha));
-    const unsigned rpt = rowsPerThread(vec);
-    if (rpt > 1) k.define("RPT", rpt);
     defineOutput(k, place);
     const std::string entry = std::string(op.func == ActivationFunction::ReLU ? "relu_c" : "leaky_relu_c") + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, rowGrid(sym, in.width, chunksPerPixel(in.channels, vec)), rowBlocks(sym, in.height, rpt), Sym::Const(1), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, rowGrid(sym, in.width, chunksPerPixel(in.channels, vec)), in.height, Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     bindOutput(d, sym, model, m, place);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
@@ -751,12 +744,10 @@ public:
     k.define("CH", in.channels); k.define("VEC", vec);
     const bool zeros = op.padMode == PaddingMode::Zero;
     if (zeros) k.define("ZERO", 1);
-    const unsigned rpt = rowsPerThread(vec);
-    if (rpt > 1) k.define("RPT", rpt);
     defineOutput(k, place);
     const std::string entry = std::string(zeros ? "memory_pad_zero_c" : "memory_pad_c") + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, chunksPerPixel(in.channels, vec)), rowBlocks(sym, out.height, rpt), Sym::Const(1), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, chunksPerPixel(in.channels, vec)), out.height, Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     bindOutput(d, sym, model, m, place);
     d.addPushConstant(out.width); d.addPushConstant(out.height);
@@ -777,12 +768,10 @@ public:
     const unsigned vec = place.vec;
     auto k = m_compiler->read("slice.hip");
     k.define("CH", in.channels); k.define("VEC", vec);
-    const unsigned rpt = rowsPerThread(vec);
-    if (rpt > 1) k.define("RPT", rpt);
     defineOutput(k, place);
     const std::string entry = "memory_slice_c" + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, chunksPerPixel(in.channels, vec)), rowBlocks(sym, out.height, rpt), Sym::Const(1), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, chunksPerPixel(in.channels, vec)), out.height, Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     bindOutput(d, sym, model, m, place);
     d.addPushConstant(op.top); d.addPushConstant(op.left);

@@ -24,20 +24,10 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
   const unsigned i = DNX_ROW_INDEX();
   if (i >= pc.W * CV) return;
   const unsigned w = i / CV, cv = i - w * CV;
-  const unsigned h0 = DNX_BID_Y * RPT;
-  chunk_t v[RPT];
+  const size_t pix = (size_t)DNX_BID_Y * pc.W + w;
+  const chunk_t v = ld_chunk<CH>(IN + pix * CH, cv);
+  half8 a = __builtin_bit_cast(half8, v.a), b = __builtin_bit_cast(half8, v.b);
 #pragma unroll
-  for (unsigned u = 0; u < RPT; ++u) {
-    const size_t pix = (size_t)(h0 + u < pc.H ? h0 + u : pc.H - 1) * pc.W + w;
-    v[u] = ld_chunk<CH>(IN + pix * CH, cv);
-  }
-#pragma unroll
-  for (unsigned u = 0; u < RPT; ++u) {
-    if (h0 + u >= pc.H) break;
-    const size_t pix = (size_t)(h0 + u) * pc.W + w;
-    half8 a = __builtin_bit_cast(half8, v[u].a), b = __builtin_bit_cast(half8, v[u].b);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) a[e] = act1(a[e]), b[e] = act1(b[e]);
-    st_chunk<CH>(OUT + pix * OPITCH, cv, chunk_t{__builtin_bit_cast(uint4v, a), __builtin_bit_cast(uint4v, b)});
-  }
+  for (int e = 0; e < 8; ++e) a[e] = act1(a[e]), b[e] = act1(b[e]);
+  st_chunk<CH>(OUT + pix * OPITCH, cv, chunk_t{__builtin_bit_cast(uint4v, a), __builtin_bit_cast(uint4v, b)});
 }

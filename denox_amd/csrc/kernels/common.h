@@ -33,14 +33,6 @@ typedef uint4v uint4u __attribute__((aligned(2)));
 typedef uint2v uint2u __attribute__((aligned(2)));
 typedef unsigned int uint1u __attribute__((aligned(2)));
 
-// Rows of the iteration space per thread.  A thread with one 16-byte load outstanding keeps too few bytes in flight to
-// cover the memory latency when pixels are narrow (a wave of a 9-channel kernel has 0.6 KB in flight against the 1 KB of
-// an aligned one, and far fewer waves fit a small image); with RPT > 1 it loads the same chunk of RPT consecutive rows
-// before it stores any of them.  grid.y = ceil(rows / RPT); rows past the end are loaded from the last row and not stored.
-#ifndef RPT
-#define RPT 1
-#endif
-
 // What one thread moves: a chunk of 8 channels and, when VEC = 1 and it is the pixel's last full chunk, the partial chunk
 // behind it too (so a 9-channel pixel is one thread's 16 + 2 bytes, not a full thread and a nearly idle one).
 struct chunk_t { vec_t a, b; };

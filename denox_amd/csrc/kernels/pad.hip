@@ -14,35 +14,22 @@ struct PushConstants { unsigned int OUT_W, OUT_H, PAD_L, PAD_R, PAD_T, PAD_B; };
 extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
     const ushort_t *__restrict__ IN, ushort_t *__restrict__ OUT, PushConstants pc) {
   constexpr unsigned CV = DNX_CHUNKS(CH);
-  const unsigned h0 = DNX_BID_Y * RPT;
+  const int ho = (int)DNX_BID_Y;
   const unsigned i = DNX_ROW_INDEX();
   if (i >= pc.OUT_W * CV) return;
   const unsigned wo = i / CV, cv = i - wo * CV;
   const int IN_W = (int)(pc.OUT_W - pc.PAD_L - pc.PAD_R);
   const int IN_H = (int)(pc.OUT_H - pc.PAD_T - pc.PAD_B);
-  int wi = (int)wo - (int)pc.PAD_L;
+  int hi = ho - (int)pc.PAD_T, wi = (int)wo - (int)pc.PAD_L;
 #if ZERO
-  const bool insideX = wi >= 0 && wi < IN_W;
+  const bool inside = hi >= 0 && hi < IN_H && wi >= 0 && wi < IN_W;
 #endif
+  hi = hi < 0 ? 0 : (hi > IN_H - 1 ? IN_H - 1 : hi);
   wi = wi < 0 ? 0 : (wi > IN_W - 1 ? IN_W - 1 : wi);
-  chunk_t v[RPT];
-#pragma unroll
-  for (unsigned u = 0; u < RPT; ++u) {
-    int hi = (int)(h0 + u) - (int)pc.PAD_T;
+  chunk_t v = ld_chunk<CH>(IN + ((size_t)hi * IN_W + wi) * CH, cv); // the clamped read is in range in both modes
 #if ZERO
-    const bool inside = insideX && hi >= 0 && hi < IN_H;
+  const chunk_t zero = {};
+  v = inside ? v : zero;
 #endif
-    hi = hi < 0 ? 0 : (hi > IN_H - 1 ? IN_H - 1 : hi);
-    v[u] = ld_chunk<CH>(IN + ((size_t)hi * IN_W + wi) * CH, cv); // the clamped read is in range in both modes
-#if ZERO
-    const chunk_t zero = {};
-    v[u] = inside ? v[u] : zero;
-#endif
-  }
-#pragma unroll
-  for (unsigned u = 0; u < RPT; ++u) {
-    const unsigned ho = h0 + u;
-    if (ho >= pc.OUT_H) break;
-    st_chunk<CH>(OUT + ((size_t)ho * pc.OUT_W + wo) * OPITCH, cv, v[u]);
-  }
+  st_chunk<CH>(OUT + ((size_t)ho * pc.OUT_W + wo) * OPITCH, cv, v);
 }

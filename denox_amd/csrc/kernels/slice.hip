@@ -10,20 +10,10 @@ struct PushConstants { unsigned int IN_TOP, IN_LEFT, IN_W, IN_H, OUT_W, OUT_H; }
 extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
     const ushort_t *__restrict__ IN, ushort_t *__restrict__ OUT, PushConstants pc) {
   constexpr unsigned CV = DNX_CHUNKS(CH);
-  const unsigned h0 = DNX_BID_Y * RPT;
+  const unsigned h = DNX_BID_Y;
   const unsigned i = DNX_ROW_INDEX();
   if (i >= pc.OUT_W * CV) return;
   const unsigned w = i / CV, cv = i - w * CV;
-  chunk_t v[RPT];
-#pragma unroll
-  for (unsigned u = 0; u < RPT; ++u) {
-    const unsigned h = h0 + u < pc.OUT_H ? h0 + u : pc.OUT_H - 1;
-    v[u] = ld_chunk<CH>(IN + ((size_t)(h + pc.IN_TOP) * pc.IN_W + (w + pc.IN_LEFT)) * CH, cv);
-  }
-#pragma unroll
-  for (unsigned u = 0; u < RPT; ++u) {
-    const unsigned h = h0 + u;
-    if (h >= pc.OUT_H) break;
-    st_chunk<CH>(OUT + ((size_t)h * pc.OUT_W + w) * OPITCH, cv, v[u]);
-  }
+  st_chunk<CH>(OUT + ((size_t)h * pc.OUT_W + w) * OPITCH, cv,
+               ld_chunk<CH>(IN + ((size_t)(h + pc.IN_TOP) * pc.IN_W + (w + pc.IN_LEFT)) * CH, cv));
 }

@@ -14,23 +14,13 @@ struct PushConstants { unsigned int W, H; }; // input extent
 extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
     const ushort_t *__restrict__ IN, ushort_t *__restrict__ OUT, PushConstants pc) {
   constexpr unsigned CV = DNX_CHUNKS(CH);
-  const unsigned h0 = DNX_BID_Y * RPT;
+  const unsigned h = DNX_BID_Y;
   const unsigned i = DNX_ROW_INDEX();
   if (i >= pc.W * SCALE * CV) return;
   const unsigned w2 = i / CV, cv = i - w2 * CV;
   const unsigned w = w2 / SCALE;
-  chunk_t v[RPT];
-#pragma unroll
-  for (unsigned u = 0; u < RPT; ++u) {
-    const unsigned h = h0 + u < pc.H ? h0 + u : pc.H - 1;
-    v[u] = ld_chunk<CH>(IN + ((size_t)h * pc.W + w) * CH, cv);
-  }
+  const chunk_t v = ld_chunk<CH>(IN + ((size_t)h * pc.W + w) * CH, cv);
   const size_t W2 = (size_t)pc.W * SCALE;
 #pragma unroll
-  for (unsigned u = 0; u < RPT; ++u) {
-    const unsigned h = h0 + u;
-    if (h >= pc.H) break;
-#pragma unroll
-    for (int r = 0; r < SCALE; ++r) st_chunk<CH>(OUT + (((size_t)h * SCALE + r) * W2 + w2) * OPITCH, cv, v[u]);
-  }
+  for (int r = 0; r < SCALE; ++r) st_chunk<CH>(OUT + (((size_t)h * SCALE + r) * W2 + w2) * OPITCH, cv, v);
 }
