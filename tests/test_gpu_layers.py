@@ -459,6 +459,32 @@ def test_bandwidth_kernels_store_in_place(oracle, C0, C1):
         assert_bits_equal(g, want[t.name], "in place against the oracle")
 
 
+@pytest.mark.parametrize("C", [1, 2, 4, 5, 6, 7, 10, 11, 13, 14, 15, 23, 31, 41])
+def test_every_channel_remainder(oracle, C):
+    """Channel counts with every remainder modulo 8, below and above 8: the bandwidth kernels move a pixel's full chunks of 8
+    channels as 16-byte accesses and the remainder as 8 + 4 + 2 bytes.  Each op alone and stored in place into a concat whose
+    other half is written by another dispatch -- a store one element too wide would damage the neighbour's channels."""
+    rng = np.random.default_rng(C)
+    H, W = 10, 27
+    x = rng.standard_normal((H, W, C)).astype(np.float16)
+    m = dx.Model()
+    inp = m.input("input", "W", "H", C)
+    singles = [m.relu(inp), m.activation(inp, "leaky_relu", 0.125), m.pool(inp), m.pool(inp, func="avg"), m.upsample(inp),
+               m.pad(inp, 1, 2, 3, 0), m.pad(inp, 2, 1, 0, 3, mode="zero"), m.slice(inp, 1, m.sym("W") - 2, 2, m.sym("H") - 1)]
+    pairs = [m.concat(m.relu(inp), m.activation(inp, "leaky_relu", 0.5)),
+             m.concat(m.pad(m.pool(inp), 0, m.sym("W") - m.sym("W") // 2, 0, m.sym("H") - m.sym("H") // 2), m.relu(inp)),
+             m.concat(m.upsample(inp), m.pad(inp, 0, m.sym("W"), m.sym("H"), 0))]
+    for t in singles + pairs:
+        m.output(t)
+    mod = dx.Module.compile(m)
+    names = [d_["name"] for d_ in dx.describe(mod.dnx, H=H, W=W)["dispatches"]]
+    assert sum(n.endswith("+concat") for n in names) >= 5, names
+    got = mod.instance(H=H, W=W).infer(x)
+    want = oracle.run_graph(m.to_ops({"H": H, "W": W}), {"input": x}, "f16")
+    for t, g in zip(singles + pairs, got):
+        assert_bits_equal(g, want[t.name], f"C={C} {t.name}")
+
+
 @pytest.mark.parametrize("CA,CB", [(3, 3), (9, 64), (64, 9), (8, 8), (12, 20), (73, 7), (16, 24), (1, 1), (5, 17)])
 def test_concat_copy_of_two_sources(oracle, CA, CB):
     """Both sources copied by one launch that writes whole pixels (model inputs cannot be written in place, so neither source
