@@ -120,7 +120,9 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     const int i = tid + it * NT;
     const int pix = i / VA, v = i - pix * VA;
     const int hy = pix / AW, hx = pix - hy * AW;
-    aLds[it] = (i < AH * AW * VA && v * 8 < CA) ? pix * APITCH + v * 8 : -1;
+    // every vector of the CAP staged channels gets a slot: those past CA are stored as zeros (their weights are zero, but
+    // what LDS held before is not, and 0 * NaN is NaN)
+    aLds[it] = i < AH * AW * VA ? pix * APITCH + v * 8 : -1;
     aYX[it] = (hy << 16) | hx;
     aRel[it] = ((hy * WL + hx) * CA + v * 8) * 2;
   }
@@ -132,7 +134,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
 #pragma unroll
     for (int it = 0; it < NVA; ++it) {
       const int yl = yb + (aYX[it] >> 16), xl = xb + (aYX[it] & 0xFFFF);
-      const bool ok = live && aLds[it] >= 0 && yl >= 0 && yl < HL && xl >= 0 && xl < WL;
+      const bool ok = live && aLds[it] >= 0 && aLds[it] % APITCH < CA && yl >= 0 && yl < HL && xl >= 0 && xl < WL;
       ga[it] = __builtin_amdgcn_raw_buffer_load_b128(ra, ok ? (unsigned)(base + aRel[it]) : NO_LOAD, 0, 0);
     }
   };
@@ -153,7 +155,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     const int cc = v * 8;
     const int chan = (CB % 8 == 0 || cc + 8 <= CB) ? cc : CB - 8; // the partial last vector ends at the last channel
     // columns de-interleaved by parity: even columns first (33 of them), then the odd ones
-    bLds[it] = (i < BH * BW * VB && cc < CB) ? (hy * BW + (hx & 1) * 33 + (hx >> 1)) * BPITCH + cc : -1;
+    bLds[it] = i < BH * BW * VB ? (hy * BW + (hx & 1) * 33 + (hx >> 1)) * BPITCH + cc : -1; // vectors past CB: stored as zeros
     bYX[it] = (hy << 16) | hx;
 #if PADB
     bRel[it] = chan * 2;
@@ -171,7 +173,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
 #pragma unroll
     for (int it = 0; it < NVB; ++it) {
       const int gy = yb + (bYX[it] >> 16), gx = xb + (bYX[it] & 0xFFFF);
-      const bool ok = live && bLds[it] >= 0 && gy >= 0 && gy < (int)pc.IN_H && gx >= 0 && gx < (int)pc.IN_W;
+      const bool ok = live && bLds[it] >= 0 && bLds[it] % BPITCH < CB && gy >= 0 && gy < (int)pc.IN_H && gx >= 0 && gx < (int)pc.IN_W;
 #if PADB
       const int sy = clampi(gy - (int)pc.PAD_T, 0, (int)pc.SRC_H - 1), sx = clampi(gx - (int)pc.PAD_L, 0, (int)pc.SRC_W - 1);
       const unsigned off = (unsigned)((sy * (int)pc.SRC_W + sx) * CB * 2 + bRel[it]);

@@ -133,6 +133,9 @@ private:
   ModelHandle m_model;
   std::vector<int64_t> m_sym;
   std::vector<void *> m_buffers;
+  std::vector<char> m_ownBuffer; // 1: an allocation of its own, 0: a range of m_arena
+  void *m_arena = nullptr;       // memory shared by the intermediate buffers
+  void freeBuffers();
   std::vector<uint64_t> m_bufferSizes;
   std::vector<Launch> m_launches;
   std::vector<void *> m_boundInputs, m_boundOutputs; // external overrides currently patched in

@@ -127,3 +127,35 @@ def one_geometry_case(oracle, seed):
 def test_random_conv_geometry(oracle, block):
     for seed in range(block * 25, block * 25 + 25):
         one_geometry_case(oracle, seed)
+
+
+@pytest.mark.parametrize("CA,CB", [(8, 33), (24, 0), (40, 17), (32, 33)])
+def test_stale_lds_contents_do_not_reach_the_result(oracle, CA, CB):
+    """The upsample-folding kernel stages its sources padded to 16 channels and multiplies the padding with zero weights:
+    the padding must be stored as zeros, not left as whatever the previous kernel had in LDS (0 * NaN is NaN).  A conv over
+    an all-NaN image runs first so that LDS is full of NaNs, then layers whose channel counts leave 8 padded channels."""
+    rng = np.random.default_rng(CA + CB)
+    p = dx.Model()
+    p.output(p.relu(p.conv2d(p.input("x", "W", "H", 64), he_weights(rng, 64, 64))))
+    poison = dx.Module.compile(p).instance(H=256, W=256)
+    H, W = 36, 44
+    m = dx.Model()
+    a = m.input("a", m.sym("W") // 2, m.sym("H") // 2, CA)
+    feeds = {"a": rng.standard_normal((H // 2, W // 2, CA)).astype(np.float16)}
+    t = m.upsample(a)
+    if CB:
+        t = m.concat(t, m.input("b", "W", "H", CB))
+        feeds["b"] = rng.standard_normal((H, W, CB)).astype(np.float16)
+    t = m.conv2d(t, he_weights(rng, 16, CA + CB), small_bias(rng, 16))
+    m.output(t)
+    want = oracle.run_graph(m.to_ops({"H": H, "W": W}), feeds, "fp32")[t.name]
+    for config in ("f4r1", "f8r1", "f4r2"):
+        try:
+            inst = dx.Module.compile(m, conv_config=config).instance(H=H, W=W)
+        except dx.DenoxHipError as e:
+            assert e.status == 5, str(e)
+            continue
+        for _ in range(3):
+            poison.infer(np.full((256, 256, 64), np.nan, np.float16))
+            got = inst.infer(*[feeds[k] for k in ("a", "b") if k in feeds])[0]
+            assert_conv_close(got, want, f"{config} after a kernel that left NaNs in LDS")

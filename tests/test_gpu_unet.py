@@ -100,6 +100,28 @@ def test_device_pointer_path_matches_host_path():
     inst.synchronize()
 
 
+@pytest.mark.parametrize("net,features", [("oidn_unet", None), ("oidn_unet", dict(conv_relu_fusion=False, concat_conv_fusion=False, upsample_fusion=False, pool_fusion=False, pad_fusion=False, slice_fusion=False)),
+                                          ("tiny_unet", dict(implicit_concat=False, concat_conv_fusion=False))])
+def test_intermediate_buffers_share_memory(monkeypatch, net, features):
+    """Intermediate buffers with disjoint lifetimes share one arena: fewer device bytes than one allocation per buffer
+    (DENOX_HIP_NO_ALIAS=1 switches the sharing off for this comparison), the same bits out, also on a second inference
+    into the now dirty arena and for a schedule with many small dispatches."""
+    H, W = 72, 104
+    m, _ = networks.build(net, seed=11)
+    x = networks.synthetic_input(net, H, W, seed=11)
+    mod = dx.Module.compile(m, features=features) if features else dx.Module.compile(m)
+    shared = dx.Instance(mod.runtime_model, H=H, W=W)
+    monkeypatch.setenv("DENOX_HIP_NO_ALIAS", "1")
+    separate = dx.Instance(mod.runtime_model, H=H, W=W)
+    monkeypatch.delenv("DENOX_HIP_NO_ALIAS")
+    assert shared.device_bytes < separate.device_bytes
+    want = separate.infer(x)[0]
+    assert_bits_equal(shared.infer(x)[0], want, "shared arena")
+    assert_bits_equal(shared.infer(x)[0], want, "shared arena, second inference")
+    x2 = networks.synthetic_input(net, H, W, seed=12)
+    assert_bits_equal(shared.infer(x2)[0], separate.infer(x2)[0], "shared arena, other input")
+
+
 # ----------------------------------------------------------------------------- full size
 FULL_H, FULL_W = 1080, 1920
 

@@ -356,3 +356,49 @@ def test_measured_latencies_drive_the_selection(tmp_path):
     # without a table the roofline estimate prefers the fused kernel
     names = _dispatch_names(dx.compile_model(m, assume={"H": 64, "W": 64}, conv_config="w4r2k16"), H=64, W=64)
     assert "concat+upsample+conv3x3+relu" in names
+
+
+# ----------------------------------------------------------------------------- arena planner (runtime/arena_plan.hpp)
+@pytest.fixture(scope="module")
+def arena_probe(tmp_path_factory):
+    import ctypes
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = tmp_path_factory.mktemp("arena") / "libarena_probe.so"
+    subprocess.run(["g++", "-O1", "-g", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-Werror", os.path.join(root, "tests", "arena_probe.cpp"), "-o", str(out)],
+                   check=True)
+    lib = ctypes.CDLL(str(out))
+
+    def plan(items):
+        n = len(items)
+        U, I = ctypes.c_ulonglong * n, ctypes.c_int * n
+        offs, arena = U(), ctypes.c_ulonglong()
+        lib.arena_probe_plan(n, U(*[b for b, _, _ in items]), I(*[f for _, f, _ in items]), I(*[l for _, _, l in items]), offs, ctypes.byref(arena))
+        return list(offs), arena.value
+    return plan
+
+
+def test_arena_plan_never_overlaps_live_buffers(arena_probe):
+    """Buffers alive at the same dispatch never share a byte; the arena is never larger than the sum of the buffers nor
+    smaller than the largest set alive at one dispatch; a chain of equally sized buffers ping-pongs between two slots."""
+    rng = np.random.default_rng(0)
+    for trial in range(300):
+        n = int(rng.integers(1, 24))
+        T = int(rng.integers(1, 20))
+        items = []
+        for _ in range(n):
+            f = int(rng.integers(0, T))
+            items.append((int(rng.integers(1, 40)) * 256, f, int(rng.integers(f, T))))
+        offs, arena = arena_probe(items)
+        for i in range(n):
+            assert offs[i] + items[i][0] <= arena
+            for j in range(i):
+                alive_together = items[i][1] <= items[j][2] and items[j][1] <= items[i][2]
+                apart = offs[i] + items[i][0] <= offs[j] or offs[j] + items[j][0] <= offs[i]
+                assert apart or not alive_together, (trial, i, j)
+        peak = max(sum(b for b, f, l in items if f <= t <= l) for t in range(T))
+        assert peak <= arena <= sum(b for b, _, _ in items)
+    chain = [(1024, t, t + 1) for t in range(10)]  # each buffer written at t, read at t + 1
+    offs, arena = arena_probe(chain)
+    assert arena == 2048 and all(offs[t] != offs[t + 1] for t in range(9))
+    assert arena_probe([]) == ([], 0)
