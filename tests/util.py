@@ -32,3 +32,21 @@ def assert_bits_equal(got, want, what=""):
     assert g.shape == w.shape, (g.shape, w.shape)
     bad = np.argwhere(g != w)
     assert bad.size == 0, f"{what}: {len(bad)} differing elements, first at {tuple(bad[0])}: got {g[tuple(bad[0])]:#06x} want {w[tuple(bad[0])]:#06x}"
+
+
+_poison = None
+
+
+def fill_lds_with_nans():
+    """Runs a conv whose image, weights and bias are all NaN on every compute unit, in the configuration that keeps the
+    most LDS (resident weights + halo).  What a kernel leaves in LDS is what the next one finds there: a kernel that
+    multiplies a staged value it never wrote with a zero weight then produces NaN.  Called in front of fuzzed layers so
+    that such a read shows up whatever ran before."""
+    global _poison
+    import denox_amd as dx
+    if _poison is None:
+        m = dx.Model()
+        nan = np.float16(np.nan)
+        m.output(m.conv2d(m.input("x", "W", "H", 64), np.full((64, 64, 3, 3), nan, np.float16), np.full(64, nan, np.float16)))
+        _poison = (dx.Module.compile(m, conv_config="s8r2k16").instance(H=256, W=512), np.full((256, 512, 64), nan, np.float16))
+    _poison[0].infer(_poison[1])
