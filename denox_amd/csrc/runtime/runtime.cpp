@@ -166,6 +166,12 @@ Instance::Instance(ModelHandle model, const std::vector<ValueSpec> &specs) : m_m
     }
     // parameters (instance.cpp:65-113 of the reference)
     hipStream_t s = m_model->context()->stream();
+    if (std::getenv("DENOX_HIP_POISON")) { // debugging: every activation byte starts as 0xFF (binary16 NaN), so a kernel that
+                                           // lets memory nobody wrote reach its result shows up in the output
+      if (m_arena) hipCheck(hipMemsetAsync(m_arena, 0xFF, arenaBytes, s), "hipMemsetAsync(poison)");
+      for (size_t i = 0; i < m.buffers.size(); ++i)
+        if (m_ownBuffer[i]) hipCheck(hipMemsetAsync(m_buffers[i], 0xFF, padded(i), s), "hipMemsetAsync(poison)");
+    }
     for (const auto &init : m.initializers) {
       const auto &t = m.tensors[init.tensor];
       const uint64_t sz = static_cast<uint64_t>(t.size.eval(m_sym));

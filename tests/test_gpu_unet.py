@@ -120,6 +120,16 @@ def test_intermediate_buffers_share_memory(monkeypatch, net, features):
     assert_bits_equal(shared.infer(x)[0], want, "shared arena, second inference")
     x2 = networks.synthetic_input(net, H, W, seed=12)
     assert_bits_equal(shared.infer(x2)[0], separate.infer(x2)[0], "shared arena, other input")
+    # every activation byte NaN before the first inference (DENOX_HIP_POISON=1): no dispatch may let memory that nobody
+    # wrote reach the result, with or without sharing
+    monkeypatch.setenv("DENOX_HIP_POISON", "1")
+    poisoned = dx.Instance(mod.runtime_model, H=H, W=W)
+    monkeypatch.setenv("DENOX_HIP_NO_ALIAS", "1")
+    poisoned_separate = dx.Instance(mod.runtime_model, H=H, W=W)
+    monkeypatch.delenv("DENOX_HIP_NO_ALIAS")
+    monkeypatch.delenv("DENOX_HIP_POISON")
+    assert_bits_equal(poisoned.infer(x)[0], want, "arena filled with NaNs")
+    assert_bits_equal(poisoned_separate.infer(x)[0], want, "buffers filled with NaNs")
 
 
 # ----------------------------------------------------------------------------- full size
