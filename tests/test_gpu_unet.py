@@ -132,6 +132,48 @@ def test_intermediate_buffers_share_memory(monkeypatch, net, features):
     assert_bits_equal(poisoned_separate.infer(x)[0], want, "buffers filled with NaNs")
 
 
+def test_threads_with_their_own_handles_run_at_once():
+    """One handle, one thread at a time is the contract; threads that each own a context, a compiled model and an instance may
+    compile and infer at the same time (the kernel cache, the last-error string and the compile report are the shared or
+    thread-local state).  Each thread's results must equal the ones computed alone."""
+    import threading
+    nets = [("oidn_unet", 40, 56), ("tiny_unet", 64, 96), ("oidn_unet", 33, 47), ("tiny_unet", 37, 61)]
+    alone = []
+    for i, (net, H, W) in enumerate(nets):
+        m, _ = networks.build(net, seed=i)
+        alone.append(dx.Module.compile(m).instance(H=H, W=W).infer(networks.synthetic_input(net, H, W, seed=i))[0])
+    results, errors = [None] * len(nets), []
+    start = threading.Barrier(len(nets))
+
+    def work(i):
+        try:
+            net, H, W = nets[i]
+            m, _ = networks.build(net, seed=i)
+            x = networks.synthetic_input(net, H, W, seed=i)
+            start.wait()
+            ctx = dx.Context()
+            mod = dx.Module.compile(m, ctx=ctx)
+            inst = mod.instance(H=H, W=W)
+            outs = [inst.infer(x)[0] for _ in range(25)]
+            with pytest.raises(dx.DenoxHipError) as e:  # an error on this thread leaves the others' last-error strings alone
+                dx.Instance(mod.runtime_model, H=H)
+            assert "'W'" in str(e.value)
+            results[i] = outs
+        except BaseException as exc:  # noqa: BLE001 -- reported below, in the main thread
+            errors.append((i, repr(exc)))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(len(nets))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not errors, errors
+    assert all(not t.is_alive() for t in threads)
+    for i, outs in enumerate(results):
+        for o in outs:
+            assert_bits_equal(o, alone[i], f"thread {i}")
+
+
 # ----------------------------------------------------------------------------- full size
 FULL_H, FULL_W = 1080, 1920
 
