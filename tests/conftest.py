@@ -25,3 +25,12 @@ def oracle():
     import oracle as _oracle
     _oracle.build()
     return _oracle
+
+
+@pytest.fixture(autouse=True)
+def activations_start_as_nans(request, monkeypatch):
+    """GPU tests create their instances with every activation byte 0xFF (binary16 NaN, DENOX_HIP_POISON=1): a dispatch
+    that lets memory nobody wrote reach its result then fails its comparison instead of passing on whatever the
+    allocation happened to hold."""
+    if request.node.get_closest_marker("gpu") is not None:
+        monkeypatch.setenv("DENOX_HIP_POISON", "1")
