@@ -1,6 +1,7 @@
 #include "runtime.hpp"
 #include "arena_plan.hpp"
 #include <algorithm>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 
@@ -147,11 +148,11 @@ Instance::Instance(ModelHandle model, const std::vector<ValueSpec> &specs) : m_m
     for (size_t i = 0; i < m.buffers.size(); ++i)
       if (!own[i] && last[i] >= 0 && !std::getenv("DENOX_HIP_NO_ALIAS")) shared.push_back(i);
     // (placing in order of first use with a preference for ranges that died just before was measured too: 16 % more
-    // memory and 1 % slower than the plain largest-first placement of plan_arena)
+    // memory and 1 % slower than the largest-first placement of plan_arena)
     std::vector<ArenaItem> items;
     for (size_t i : shared) items.push_back(ArenaItem{padded(i), first[i], last[i]});
     uint64_t arenaBytes = 0;
-    const std::vector<uint64_t> at = plan_arena(items, arenaBytes);
+    const std::vector<uint64_t> at = plan_arena(items, arenaBytes, static_cast<int>(m_model->dispatches().size()));
     if (arenaBytes) {
       hipCheck(hipMalloc(&m_arena, arenaBytes), "hipMalloc(arena)");
       m_deviceBytes += arenaBytes;

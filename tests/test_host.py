@@ -369,11 +369,11 @@ def arena_probe(tmp_path_factory):
                    check=True)
     lib = ctypes.CDLL(str(out))
 
-    def plan(items):
+    def plan(items, period=0):
         n = len(items)
         U, I = ctypes.c_ulonglong * n, ctypes.c_int * n
         offs, arena = U(), ctypes.c_ulonglong()
-        lib.arena_probe_plan(n, U(*[b for b, _, _ in items]), I(*[f for _, f, _ in items]), I(*[l for _, _, l in items]), offs, ctypes.byref(arena))
+        lib.arena_probe_plan(n, U(*[b for b, _, _ in items]), I(*[f for _, f, _ in items]), I(*[l for _, _, l in items]), period, offs, ctypes.byref(arena))
         return list(offs), arena.value
     return plan
 
@@ -402,3 +402,9 @@ def test_arena_plan_never_overlaps_live_buffers(arena_probe):
     offs, arena = arena_probe(chain)
     assert arena == 2048 and all(offs[t] != offs[t + 1] for t in range(9))
     assert arena_probe([]) == ([], 0)
+    # an inference's first dispatch follows the previous inference's last: the buffer written first goes where the buffer
+    # read last was, not to the lowest free offset (which holds a buffer that died one dispatch earlier)
+    items = [(512, 0, 1), (1024, 13, 14), (512, 14, 15)]
+    offs, arena = arena_probe(items, 16)
+    assert arena == 1536 and offs == [1024, 0, 1024]
+    assert arena_probe(items, -1)[0] == [0, 0, 1024]  # the preference switched off
