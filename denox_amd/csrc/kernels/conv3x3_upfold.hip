@@ -135,7 +135,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     for (int it = 0; it < NVA; ++it) {
       const int yl = yb + (aYX[it] >> 16), xl = xb + (aYX[it] & 0xFFFF);
       const bool ok = live && aLds[it] >= 0 && aLds[it] % APITCH < CA && yl >= 0 && yl < HL && xl >= 0 && xl < WL;
-      ga[it] = __builtin_amdgcn_raw_buffer_load_b128(ra, ok ? (unsigned)(base + aRel[it]) : NO_LOAD, 0, 0);
+      ga[it] = __builtin_amdgcn_raw_buffer_load_b128(ra, ok ? (unsigned)(base + aRel[it]) : NO_LOAD, 0, LOAD_AUX);
     }
   };
   auto commitA = [&]() {
@@ -180,7 +180,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
 #else
       const unsigned off = (unsigned)(base + bRel[it]);
 #endif
-      gb[it] = __builtin_amdgcn_raw_buffer_load_b128(rb, ok ? off : NO_LOAD, 0, 0);
+      gb[it] = __builtin_amdgcn_raw_buffer_load_b128(rb, ok ? off : NO_LOAD, 0, LOAD_AUX);
     }
   };
   auto commitB = [&]() {

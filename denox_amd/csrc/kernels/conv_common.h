@@ -100,6 +100,9 @@ typedef unsigned short ushort_t;
 #define HALO_PIX (HALO_W * HALO_H)
 #define CKP (CK + 8)
 #define KB (KT / MF)
+#ifndef LOAD_AUX
+#define LOAD_AUX 0 // cache policy bits of the halo loads through buffer resources (bit 1: non-temporal)
+#endif
 #ifndef STORE_AUX
 #define STORE_AUX 0 // cache policy bits of the output stores (bit 1: non-temporal)
 #endif
@@ -382,7 +385,7 @@ struct Halo {
 #ifdef DBG_SKIP_FETCH
       off = NO_LOAD;
 #endif
-      st.v[it] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0);
+      st.v[it] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, LOAD_AUX);
     }
 #else
     const _Float16 *__restrict__ A = src.A;
