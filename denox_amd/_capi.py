@@ -128,6 +128,7 @@ SIGNATURES = {
     "denox_hip_instance_input_device_ptr": (c_int, [c_void_p, c_uint32, POINTER(c_void_p)]),
     "denox_hip_instance_output_device_ptr": (c_int, [c_void_p, c_uint32, POINTER(c_void_p)]),
     "denox_hip_instance_bench": (c_int, [c_void_p, c_uint32, POINTER(Timing), c_uint32, POINTER(c_uint32)]),
+    "denox_hip_instance_bench_in_frame": (c_int, [c_void_p, c_uint32, c_uint32, c_uint32, POINTER(c_float)]),
     "denox_hip_instance_device_bytes": (c_int, [c_void_p, POINTER(c_uint64)]),
 }
 

@@ -531,6 +531,12 @@ int denox_hip_instance_bench(denox_hip_instance *inst, uint32_t warmup, denox_hi
     }
   });
 }
+int denox_hip_instance_bench_in_frame(denox_hip_instance *inst, uint32_t dispatch, uint32_t frames, uint32_t warmup, float *out_ms) {
+  return guarded([&] {
+    need(inst, "instance"); need(out_ms, "out_ms");
+    *out_ms = inst->inst->benchInFrame(dispatch, static_cast<int>(frames), static_cast<int>(warmup));
+  });
+}
 int denox_hip_instance_device_bytes(const denox_hip_instance *inst, uint64_t *out) {
   return guarded([&] { need(inst, "instance"); need(out, "out"); *out = inst->inst->deviceBytes(); });
 }

@@ -485,6 +485,43 @@ void Instance::infer(const void *const *inputs, void *const *outputs) {
   hipCheck(hipStreamSynchronize(s), "hipStreamSynchronize");
 }
 
+// One dispatch timed where it runs: `frames` whole inferences as plain launches on the instance's stream, with an event
+// in front of and behind dispatch `index` only, so that the kernel finds the caches, clocks and memory traffic of the
+// frame around it (launched several times back to back, as bench() does, a matrix-bound kernel runs 4 % slower than
+// after a lighter neighbour).  The interval holds one launch gap; returns the mean over the frames in milliseconds.
+float Instance::benchInFrame(uint32_t index, int frames, int warmup) {
+  if (index >= m_launches.size()) fail(Status::InvalidArgument, "dispatch index out of range");
+  if (frames < 1) fail(Status::InvalidArgument, "frames must be at least 1");
+  m_model->context()->makeCurrent();
+  rebind(nullptr, nullptr);
+  hipStream_t s = m_model->context()->stream();
+  for (int i = 0; i < warmup; ++i) launchAll(s);
+  hipCheck(hipStreamSynchronize(s), "hipStreamSynchronize");
+  std::vector<hipEvent_t> ev(2 * static_cast<size_t>(frames), nullptr);
+  double sum = 0.0;
+  try {
+    for (auto &e : ev) hipCheck(hipEventCreate(&e), "hipEventCreate");
+    for (int f = 0; f < frames; ++f)
+      for (size_t i = 0; i < m_launches.size(); ++i) {
+        auto &l = m_launches[i];
+        if (i == index) hipCheck(hipEventRecord(ev[2 * static_cast<size_t>(f)], s), "hipEventRecord");
+        launchOne(l.fn, l.grid, l.block, l.args, s);
+        if (i == index) hipCheck(hipEventRecord(ev[2 * static_cast<size_t>(f) + 1], s), "hipEventRecord");
+      }
+    hipCheck(hipStreamSynchronize(s), "hipStreamSynchronize");
+    for (int f = 0; f < frames; ++f) {
+      float ms = 0.0f;
+      hipCheck(hipEventElapsedTime(&ms, ev[2 * static_cast<size_t>(f)], ev[2 * static_cast<size_t>(f) + 1]), "hipEventElapsedTime");
+      sum += ms;
+    }
+  } catch (...) {
+    for (auto e : ev) if (e) (void)hipEventDestroy(e);
+    throw;
+  }
+  for (auto e : ev) if (e) (void)hipEventDestroy(e);
+  return static_cast<float>(sum / frames);
+}
+
 std::vector<DispatchTiming> Instance::bench(int warmup) {
   const dnx::Model &m = m_model->dnx();
   m_model->context()->makeCurrent();

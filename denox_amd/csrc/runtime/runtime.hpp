@@ -104,6 +104,7 @@ public:
   void synchronize();
   // Per-dispatch timings with hipEvents after warm-up passes (instance.cpp:432-654).
   std::vector<DispatchTiming> bench(int warmup);
+  float benchInFrame(uint32_t index, int frames, int warmup);
 
   size_t inputCount() const { return m_model->dnx().inputs.size(); }
   size_t outputCount() const { return m_model->dnx().outputs.size(); }

@@ -348,6 +348,13 @@ class Instance:
                         "TFLOPs": t.flops / ms * 1e-9 if ms > 0 else 0.0})
         return out
 
+    def bench_in_frame(self, dispatch: int, frames: int = 50, warmup: int = 5) -> float:
+        """Milliseconds of dispatch `dispatch` (an index into bench()'s list) inside whole inferences: events around that
+        dispatch only, mean over `frames` frames."""
+        ms = ctypes.c_float()
+        _capi.check(_capi.lib().denox_hip_instance_bench_in_frame(self._h, dispatch, frames, warmup, byref(ms)))
+        return float(ms.value)
+
 
 class _PinnedBlock:
     """Owner of one hipHostMalloc allocation; the arrays made from it keep it alive through their `base` chain."""

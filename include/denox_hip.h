@@ -268,6 +268,11 @@ int denox_hip_instance_input_device_ptr(const denox_hip_instance *inst, uint32_t
 int denox_hip_instance_output_device_ptr(const denox_hip_instance *inst, uint32_t i, void **out);
 /* per-dispatch timings after `warmup` untimed passes; writes min(count, capacity) entries */
 int denox_hip_instance_bench(denox_hip_instance *inst, uint32_t warmup, denox_hip_timing *out, uint32_t capacity, uint32_t *out_count);
+/* Dispatch `dispatch` (an index into the timings above) timed inside `frames` whole inferences, after `warmup` untimed ones:
+ * hipEvents in front of and behind that dispatch only, so that it runs with the caches, clocks and memory traffic of the
+ * frame around it.  No counterpart in the reference, whose Instance::bench (runtime/src/denox/runtime/instance.cpp) times
+ * every dispatch of a pass with timestamp queries; here that per-dispatch pass repeats each kernel back to back. */
+int denox_hip_instance_bench_in_frame(denox_hip_instance *inst, uint32_t dispatch, uint32_t frames, uint32_t warmup, float *out_ms);
 int denox_hip_instance_device_bytes(const denox_hip_instance *inst, uint64_t *out);
 
 #ifdef __cplusplus

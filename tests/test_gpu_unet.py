@@ -132,6 +132,24 @@ def test_intermediate_buffers_share_memory(monkeypatch, net, features):
     assert_bits_equal(poisoned_separate.infer(x)[0], want, "buffers filled with NaNs")
 
 
+def test_dispatch_timed_inside_the_frame():
+    """bench_in_frame times one dispatch with the rest of the inference running around it: a positive figure of the same
+    order as the per-dispatch pass reports, an index past the last dispatch is refused, and the outputs are untouched."""
+    H, W = 96, 160
+    m, _ = networks.build("oidn_unet", seed=2)
+    x = networks.synthetic_input("oidn_unet", H, W, seed=2)
+    inst = dx.Module.compile(m).instance(H=H, W=W)
+    want = inst.infer(x)[0]
+    alone = inst.bench(warmup=2)
+    for i in (0, len(alone) // 2, len(alone) - 1):
+        ms = inst.bench_in_frame(i, frames=20, warmup=2)
+        assert 0.0 < ms < 1.0 and ms < 20 * alone[i]["latency_ms"] + 0.05
+    with pytest.raises(dx.DenoxHipError) as e:
+        inst.bench_in_frame(len(alone), frames=5)
+    assert e.value.status == 1
+    assert_bits_equal(inst.infer(x)[0], want, "after timing")
+
+
 def test_threads_with_their_own_handles_run_at_once():
     """One handle, one thread at a time is the contract; threads that each own a context, a compiled model and an instance may
     compile and infer at the same time (the kernel cache, the last-error string and the compile report are the shared or
