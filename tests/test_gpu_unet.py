@@ -132,6 +132,25 @@ def test_intermediate_buffers_share_memory(monkeypatch, net, features):
     assert_bits_equal(poisoned_separate.infer(x)[0], want, "buffers filled with NaNs")
 
 
+def test_plain_launches_without_a_graph(monkeypatch):
+    """DENOX_HIP_NO_GRAPH=1: the instance launches its dispatches one by one instead of replaying a captured hipGraph; the
+    same bits from the blocking call, from a sequence of frames and after the graph-less instance has been timed."""
+    H, W = 40, 56
+    m, _ = networks.build("oidn_unet", seed=4)
+    xs = [networks.synthetic_input("oidn_unet", H, W, seed=s) for s in (4, 5, 6)]
+    mod = dx.Module.compile(m)
+    want = [dx.Instance(mod.runtime_model, H=H, W=W).infer(x)[0] for x in xs]
+    monkeypatch.setenv("DENOX_HIP_NO_GRAPH", "1")
+    plain = dx.Instance(mod.runtime_model, H=H, W=W)
+    monkeypatch.delenv("DENOX_HIP_NO_GRAPH")
+    for x, w in zip(xs, want):
+        assert_bits_equal(plain.infer(x)[0], w, "plain launches")
+    for got, w in zip(plain.infer_many([[x] for x in xs]), want):
+        assert_bits_equal(got[0], w, "plain launches, frame sequence")
+    assert len(plain.bench(warmup=1)) == mod.runtime_model.dispatch_count
+    assert_bits_equal(plain.infer(xs[0])[0], want[0], "plain launches after timing")
+
+
 def test_dispatch_timed_inside_the_frame():
     """bench_in_frame times one dispatch with the rest of the inference running around it: a positive figure of the same
     order as the per-dispatch pass reports, an index past the last dispatch is refused, and the outputs are untouched."""
