@@ -199,20 +199,30 @@ Instance::Instance(ModelHandle model, const std::vector<ValueSpec> &specs) : m_m
       const size_t pcOff = (ptrBytes + pcAlign - 1) / pcAlign * pcAlign;
       l.args.assign(pcOff + d.push_constant.size, 0);
       for (size_t i = 0; i < md.tensors.size(); ++i) {
-        void *p = tensorPtr(md.tensors[i].first);
+        const uint32_t tensor = md.tensors[i].first;
+        void *p = tensorPtr(tensor);
         std::memcpy(l.args.data() + i * sizeof(void *), &p, sizeof(void *));
-        l.ptrSlots.emplace_back(i * sizeof(void *), md.tensors[i].first);
+        Launch::Slot slot{i * sizeof(void *), tensor, -1, false, 0};
+        // Everything in an interface tensor's buffer moves with the address the caller binds: the tensor itself and
+        // the tensors placed inside it (concat sources that their producers write in place, compile.cpp view constrains).
+        const uint32_t buffer = m.tensors[tensor].buffer;
+        const int64_t off = m.tensors[tensor].offset.eval(m_sym);
+        for (size_t k = 0; k < m.inputs.size() && slot.iface < 0; ++k)
+          if (m.tensors[m.inputs[k]].buffer == buffer) slot = Launch::Slot{slot.offset, tensor, static_cast<int>(k), true, off - m.tensors[m.inputs[k]].offset.eval(m_sym)};
+        for (size_t k = 0; k < m.outputs.size() && slot.iface < 0; ++k)
+          if (m.tensors[m.outputs[k]].buffer == buffer) slot = Launch::Slot{slot.offset, tensor, static_cast<int>(k), false, off - m.tensors[m.outputs[k]].offset.eval(m_sym)};
+        l.ptrSlots.push_back(slot);
       }
       for (const auto &f : d.push_constant.fields) putScalar(l.args, pcOff + f.offset, f.dtype, f.source.eval(m_sym));
       m_launches.push_back(std::move(l));
     }
     m_boundInputs.assign(m.inputs.size(), nullptr);
     m_boundOutputs.assign(m.outputs.size(), nullptr);
-    if (!std::getenv("DENOX_HIP_NO_GRAPH")) buildGraph();
+    m_useGraph = !std::getenv("DENOX_HIP_NO_GRAPH");
+    if (m_useGraph) selectGraph();
   } catch (...) {
     freeBuffers();
-    if (m_graphExec) (void)hipGraphExecDestroy(m_graphExec);
-    if (m_graph) (void)hipGraphDestroy(m_graph);
+    destroyGraphs();
     throw;
   }
 }
@@ -223,9 +233,24 @@ Instance::~Instance() {
     (void)hipStreamSynchronize(m_model->context()->stream());
   }
   destroyPipeline();
-  if (m_graphExec) (void)hipGraphExecDestroy(m_graphExec);
-  if (m_graph) (void)hipGraphDestroy(m_graph);
+  destroyGraphs();
   freeBuffers();
+}
+
+void Instance::destroyGraphs() {
+  bool current = false;
+  for (auto &c : m_graphCache) {
+    current |= c.exec == m_graphExec;
+    if (c.exec) (void)hipGraphExecDestroy(c.exec);
+    if (c.graph) (void)hipGraphDestroy(c.graph);
+  }
+  m_graphCache.clear();
+  if (!current) { // captured but not filed yet (a failure in between)
+    if (m_graphExec) (void)hipGraphExecDestroy(m_graphExec);
+    if (m_graph) (void)hipGraphDestroy(m_graph);
+  }
+  m_graphExec = nullptr;
+  m_graph = nullptr;
 }
 
 void Instance::freeBuffers() {
@@ -296,48 +321,74 @@ void Instance::buildGraph() {
     throw;
   }
   hipCheck(hipStreamEndCapture(s, &m_graph), "hipStreamEndCapture");
-  hipCheck(hipGraphInstantiate(&m_graphExec, m_graph, nullptr, nullptr, 0), "hipGraphInstantiate");
+  const hipError_t e = hipGraphInstantiate(&m_graphExec, m_graph, nullptr, nullptr, 0);
+  if (e != hipSuccess) {
+    (void)hipGraphDestroy(m_graph);
+    m_graph = nullptr;
+    m_graphExec = nullptr;
+    hipCheck(e, "hipGraphInstantiate");
+  }
 }
 
 void Instance::rebind(const void *const *inputs, void *const *outputs) {
-  // Patch external input/output addresses into the argument buffers.  The graph
-  // is rebuilt only when an address differs from the last call's.
+  // Patch external input/output addresses into the argument buffers.  A graph is captured only for a set of addresses
+  // not seen before (the last few are kept).
   const dnx::Model &m = m_model->dnx();
   bool changed = false;
-  std::vector<std::pair<uint32_t, void *>> over; // tensor -> address
+  std::vector<void *> in(m.inputs.size()), out(m.outputs.size());
   for (size_t i = 0; i < m.inputs.size(); ++i) {
     void *p = inputs ? const_cast<void *>(inputs[i]) : nullptr;
     if (p != m_boundInputs[i]) { changed = true; m_boundInputs[i] = p; }
-    over.emplace_back(m.inputs[i], p ? p : tensorPtr(m.inputs[i]));
+    in[i] = p ? p : tensorPtr(m.inputs[i]);
   }
   for (size_t i = 0; i < m.outputs.size(); ++i) {
     void *p = outputs ? outputs[i] : nullptr;
     if (p != m_boundOutputs[i]) { changed = true; m_boundOutputs[i] = p; }
-    over.emplace_back(m.outputs[i], p ? p : tensorPtr(m.outputs[i]));
+    out[i] = p ? p : tensorPtr(m.outputs[i]);
   }
   if (!changed) return;
-  for (auto &l : m_launches)
-    for (const auto &[off, tensor] : l.ptrSlots)
-      for (const auto &[t, p] : over)
-        if (t == tensor) std::memcpy(l.args.data() + off, &p, sizeof(void *));
-  if (m_graphExec) {
-    (void)hipGraphExecDestroy(m_graphExec);
-    (void)hipGraphDestroy(m_graph);
-    m_graphExec = nullptr;
-    m_graph = nullptr;
-    buildGraph();
-  }
+  patchInterface(in, out);
+  if (!m_useGraph) return; // plain launches read the argument buffers at launch time
+  selectGraph();
 }
 
-// Writes the given interface addresses into the argument buffers (no graph is touched).
+// Makes m_graph / m_graphExec the captured dispatch list for the interface addresses bound now (m_boundInputs /
+// m_boundOutputs, which the argument buffers already hold): from the cache, or captured and filed there.
+void Instance::selectGraph() {
+  std::vector<void *> key = m_boundInputs;
+  key.insert(key.end(), m_boundOutputs.begin(), m_boundOutputs.end());
+  for (auto &c : m_graphCache)
+    if (c.key == key) {
+      m_graph = c.graph;
+      m_graphExec = c.exec;
+      c.lastUse = ++m_graphUse;
+      return;
+    }
+  constexpr size_t kCachedGraphs = 4;
+  if (m_graphCache.size() >= kCachedGraphs) {
+    // The one used longest ago goes.  An earlier launch of it may still be running (inferDevice does not wait), and
+    // an executable graph must not be destroyed under a running launch.
+    hipCheck(hipStreamSynchronize(m_model->context()->stream()), "hipStreamSynchronize");
+    auto victim = std::min_element(m_graphCache.begin(), m_graphCache.end(), [](const CachedGraph &a, const CachedGraph &b) { return a.lastUse < b.lastUse; });
+    (void)hipGraphExecDestroy(victim->exec);
+    (void)hipGraphDestroy(victim->graph);
+    m_graphCache.erase(victim);
+  }
+  m_graph = nullptr;
+  m_graphExec = nullptr; // until the capture below succeeds, inferDevice would fall back to plain launches
+  buildGraph();
+  m_graphCache.push_back(CachedGraph{std::move(key), m_graph, m_graphExec, ++m_graphUse});
+}
+
+// Writes the given interface addresses into the argument buffers (no graph is touched): every bound tensor that lives
+// in an interface tensor's buffer follows that tensor's address.
 void Instance::patchInterface(const std::vector<void *> &inputs, const std::vector<void *> &outputs) {
-  const dnx::Model &m = m_model->dnx();
   for (auto &l : m_launches)
-    for (const auto &[off, tensor] : l.ptrSlots) {
-      for (size_t i = 0; i < m.inputs.size(); ++i)
-        if (m.inputs[i] == tensor) std::memcpy(l.args.data() + off, &inputs[i], sizeof(void *));
-      for (size_t i = 0; i < m.outputs.size(); ++i)
-        if (m.outputs[i] == tensor) std::memcpy(l.args.data() + off, &outputs[i], sizeof(void *));
+    for (const auto &slot : l.ptrSlots) {
+      if (slot.iface < 0) continue;
+      void *base = slot.isInput ? inputs[static_cast<size_t>(slot.iface)] : outputs[static_cast<size_t>(slot.iface)];
+      void *p = static_cast<uint8_t *>(base) + slot.delta;
+      std::memcpy(l.args.data() + slot.offset, &p, sizeof(void *));
     }
 }
 

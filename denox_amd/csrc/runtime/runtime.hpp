@@ -38,6 +38,7 @@ private:
   hipStream_t m_stream = nullptr;
   hipDeviceProp_t m_props;
 };
+
 using ContextHandle = std::shared_ptr<Context>;
 
 struct ModelDispatch {
@@ -113,15 +114,18 @@ public:
   void *inputDevicePtr(size_t i) const { return tensorPtr(m_model->dnx().inputs.at(i)); }
   void *outputDevicePtr(size_t i) const { return tensorPtr(m_model->dnx().outputs.at(i)); }
   uint64_t deviceBytes() const { return m_deviceBytes; }
-  bool usesGraph() const { return m_graphExec != nullptr; }
+  bool usesGraph() const { return m_useGraph; }
 
 private:
   struct Launch {
     hipFunction_t fn;
     unsigned grid[3], block[3];
     std::vector<uint8_t> args;              // pointers then push constants
-    std::vector<std::pair<size_t, uint32_t>> ptrSlots; // (byte offset in args, tensor id)
-    hipGraphNode_t node = nullptr;
+    // One per bound tensor.  A tensor that lives in the buffer of an interface tensor (that tensor itself, or a channel
+    // range of it written in place) follows the interface address: iface = index into inputs (isInput) / outputs,
+    // delta = byte distance from the interface tensor's start; iface < 0 otherwise.
+    struct Slot { size_t offset; uint32_t tensor; int iface; bool isInput; int64_t delta; };
+    std::vector<Slot> ptrSlots;
   };
   TensorDesc describe(uint32_t tensor) const;
   void *tensorPtr(uint32_t tensor) const;
@@ -140,8 +144,16 @@ private:
   std::vector<uint64_t> m_bufferSizes;
   std::vector<Launch> m_launches;
   std::vector<void *> m_boundInputs, m_boundOutputs; // external overrides currently patched in
-  hipGraph_t m_graph = nullptr;
+  hipGraph_t m_graph = nullptr;       // the captured dispatch list for the interface addresses bound now
   hipGraphExec_t m_graphExec = nullptr;
+  // Captured graphs of interface addresses used before (a caller that alternates between a few sets of buffers
+  // finds its graph again instead of paying a capture per frame); m_graph / m_graphExec are one of these.
+  struct CachedGraph { std::vector<void *> key; hipGraph_t graph; hipGraphExec_t exec; uint64_t lastUse; };
+  std::vector<CachedGraph> m_graphCache;
+  uint64_t m_graphUse = 0;
+  bool m_useGraph = false;
+  void selectGraph();
+  void destroyGraphs();
   uint64_t m_deviceBytes = 0;
   // inferMany: the second set of interface tensors with its own captured graph, copy streams, per-set events
   struct Pipeline {

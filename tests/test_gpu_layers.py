@@ -10,6 +10,7 @@ import numpy as np
 import pytest
 
 import denox_amd as dx
+from denox_amd import networks
 from util import assert_bits_equal, assert_conv_close, he_weights, small_bias
 
 pytestmark = pytest.mark.gpu
@@ -326,6 +327,58 @@ def test_concat_sources_written_in_place(oracle, config, C, K0, K1, tail):
     assert_bits_equal(got, ref.instance(H=H, W=W).infer(x)[0], "in place against copied")
     want = oracle.run_graph(m.to_ops({"H": H, "W": W}), {"input": x}, "fp32")[out.name]
     assert_conv_close(got, want, f"in-place concat {config}")
+
+
+def test_concat_output_written_in_place_follows_external_pointers(oracle):
+    """A model output that is a concat whose sources are written in place by their producers: no dispatch binds the
+    output tensor itself, only channel ranges inside its buffer.  Caller-supplied output addresses (infer_device) and
+    the second set of interface tensors of a frame sequence (infer_many) must reach those dispatches as well."""
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(5)
+    H, W, C, K0, K1 = 37, 70, 16, 16, 24
+    m = dx.Model()
+    t = m.input("input", "W", "H", C)
+    c = m.concat(m.relu(m.conv2d(t, he_weights(rng, K0, C), small_bias(rng, K0))), m.relu(m.conv2d(t, he_weights(rng, K1, C), small_bias(rng, K1))))
+    m.output(c)
+    mod = dx.Module.compile(m)
+    assert mod.runtime_model.dispatch_count == 2  # both convs store straight into the output
+    xs = [rng.standard_normal((H, W, C)).astype(np.float16) for _ in range(4)]
+    inst = mod.instance(H=H, W=W)
+    wants = [inst.infer(x)[0] for x in xs]
+    for x, want in zip(xs, wants):
+        assert_conv_close(want, oracle.run_graph(m.to_ops({"H": H, "W": W}), {"input": x}, "fp32")[c.name], "concat output")
+    outs = [torch.full((H, W, K0 + K1), float("nan"), dtype=torch.float16, device="cuda") for _ in range(2)]
+    d_in = [torch.from_numpy(x).cuda() for x in xs]
+    torch.cuda.synchronize()
+    for i in range(4):  # alternating output buffers, as a double-buffering caller would
+        inst.infer_device([d_in[i].data_ptr()], [outs[i & 1].data_ptr()])
+        inst.synchronize()
+        assert_bits_equal(outs[i & 1].cpu().numpy(), wants[i], f"external output, frame {i}")
+    many = inst.infer_many([[x] for x in xs])
+    for i, want in enumerate(wants):
+        assert_bits_equal(many[i][0], want, f"frame sequence, frame {i}")
+    assert_bits_equal(inst.infer(xs[0])[0], wants[0], "own buffers afterwards")
+
+
+def test_graphs_of_recent_interface_addresses_are_kept():
+    """More distinct interface address sets than the instance keeps captured graphs for: every one still gives the same bits."""
+    torch = pytest.importorskip("torch")
+    H, W = 24, 40
+    m, _ = networks.build("tiny_unet", seed=8)
+    x = networks.synthetic_input("tiny_unet", H, W, seed=8)
+    inst = dx.Module.compile(m).instance(H=H, W=W)
+    want = inst.infer(x)[0]
+    d_in = torch.from_numpy(x).cuda()
+    outs = [torch.zeros((H, W, 3), dtype=torch.float16, device="cuda") for _ in range(7)]
+    torch.cuda.synchronize()
+    for rnd in range(2):
+        for o in outs:
+            inst.infer_device([d_in.data_ptr()], [o.data_ptr()])  # not synchronised: the eviction has to wait by itself
+        inst.synchronize()
+        for i, o in enumerate(outs):
+            assert_bits_equal(o.cpu().numpy(), want, f"round {rnd}, buffer {i}")
+            o.zero_()
+        torch.cuda.synchronize()
 
 
 def test_concat_with_one_source_in_place(oracle):
