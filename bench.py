@@ -7,8 +7,10 @@ C ABI (denox_hip_instance_infer_device) as one hipGraph on the library's stream.
 
 Prints ONE JSON line: Mpix/s (= 1920*1080 / time per frame) with ms/frame in
 `ms_per_step`, a `roofline` object for the dominant kernel (per-dispatch
-hipEvent timing on the launch stream) and a `cpu_baseline` object (the CPU
-oracle timed on a bounded crop of the same workload).
+hipEvent timing on the launch stream), a `cpu_baseline` object (the CPU oracle
+timed on one frame of the same workload) and a `parity` object: the output of
+the schedule that was just timed against that oracle frame (exit status 1 when
+it misses the bar).
 """
 import argparse
 import json
@@ -45,22 +47,34 @@ def lavapipe_probe() -> str:
     return "unavailable (denox itself cannot be built here: needs glslang, SPIRV-Tools, FlatBuffers)"
 
 
-def cpu_baseline(net: str, kw: dict, seed: int, budget_h: int, budget_w: int) -> dict:
-    """CPU oracle (fp32 accumulation, OpenMP over rows) on one frame of the workload (capped at 1080p), same network and weights."""
+def cpu_baseline(net: str, kw: dict, seed: int, H: int, W: int, gpu_out_hwc) -> dict:
+    """CPU oracle (fp32 evaluation, OpenMP over rows) on one frame of the workload, same network, weights and input
+    (the top-left 1920 x 1080 window of larger frames, 16-aligned), timed as the CPU baseline -- and, since it is the fp32
+    evaluation the parity bar is defined against, compared with what the GPU schedule just timed has produced."""
     import numpy as np
     import oracle
     from denox_amd import networks
     oracle.build()
-    budget_h, budget_w = min(budget_h, 1080), min(budget_w, 1920)
+    budget_h, budget_w = (H if H <= 1088 else 1072), (W if W <= 1920 else 1920)
     model, _ = networks.build(net, seed=seed, **kw)
-    x = networks.synthetic_input(net, budget_h, budget_w, seed=seed)
+    x = np.ascontiguousarray(networks.synthetic_input(net, H, W, seed=seed)[:budget_h, :budget_w])
     ops = model.to_ops({"H": budget_h, "W": budget_w})
     t0 = time.perf_counter()
-    oracle.run_graph(ops, {"input": x}, "f16")
+    want = oracle.run_graph(ops, {"input": x}, "fp32")[model.outputs[0].name]
     dt = time.perf_counter() - t0
+    # A window cut out of a larger frame equals the frame's result only away from the cut: the deepest network here sees
+    # less than 96 pixels in each direction.
+    ys = slice(0, budget_h if budget_h == H else budget_h - 96)
+    xs = slice(0, budget_w if budget_w == W else budget_w - 96)
+    got = np.asarray(gpu_out_hwc[:budget_h, :budget_w][ys, xs], np.float32)
+    err = np.abs(got - np.asarray(want, np.float32)[ys, xs])
+    scale = max(1.0, float(np.abs(want).max()))
+    parity = {"max_abs": float(err.max()), "mean_abs": float(err.mean()), "bar_max_abs": 2e-2 * scale, "bar_mean_abs": 2e-3 * scale,
+              "pixels_compared": int(got.shape[0] * got.shape[1]), "against": "CPU oracle, fp32 evaluation of the same frame",
+              "ok": bool(np.isfinite(got).all() and err.max() <= 2e-2 * scale and err.mean() <= 2e-3 * scale)}
     out = {"value": budget_h * budget_w / dt * 1e-6, "unit": "Mpix/s", "cores": oracle.num_threads(), "kind": "port",
-           "sample": f"one {budget_w}x{budget_h} frame of the same network, fp32 accumulation, {dt:.1f} s wall",
-           "lavapipe_baseline": lavapipe_probe()}
+           "sample": f"one {budget_w}x{budget_h} frame of the same network, fp32 evaluation, {dt:.1f} s wall",
+           "lavapipe_baseline": lavapipe_probe(), "parity": parity}
     try:
         out.update(torch_cpu_baseline(ops, x, budget_h, budget_w))
     except Exception as e:  # context only: never fail the benchmark over it
@@ -123,6 +137,7 @@ def main() -> int:
     ap.add_argument("--conv-config", default=None)
     ap.add_argument("--db", default=None, help="timing table to select the schedule with (default: measure one now)")
     ap.add_argument("--no-tune", action="store_true", help="skip the timing table; select by roofline estimates")
+    ap.add_argument("--no-unfused-pass", action="store_true", help="skip the second, unfused schedule that times the stand-alone bandwidth kernels")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on exactly one GPU (independent frames shard trivially across GPUs; "
@@ -189,10 +204,12 @@ def main() -> int:
         inst.synchronize()
         singles.append((time.perf_counter() - t1) * 1e3)
     singles.sort()
-    out_host = d_out.cpu().numpy()
+    out_host = d_out.cpu().numpy()  # what the timed schedule wrote in its last step
     if not np.isfinite(out_host).all():
         print("bench.py: non-finite output", file=sys.stderr)
         return 1
+    od = inst.output_desc()
+    out_hwc = out_host.reshape(od["channels"], od["height"], od["width"]).transpose(1, 2, 0) if layout == "CHW" else out_host.reshape(od["height"], od["width"], od["channels"])
 
     # the reference's own entry point (host pointers in and out, blocking): PCIe-inclusive, reported beside, never as `value`
     t0 = time.perf_counter()
@@ -250,18 +267,53 @@ def main() -> int:
                 "non_conv_frac_of_hbm": other_bytes / other_ms * 1e-6 / PEAK_HBM_GBPS if other_ms else None,
                 "sum_dispatch_ms": sum(a["latency_ms"] for a in acc)}
 
-    # HBM traffic of the dominant kernel from the committed rocprofv3 --pmc summary, when it covers this kernel:
-    # the summary lists every configuration of that layer; the compile report says which one this schedule uses
+    # Which configuration each dispatch of the schedule runs, and the SHA-256 of its code object.
+    desc = dx.describe(blob, H=H, W=W)["dispatches"]
+    chosen = [f'{d["name"]}: {d["debug_info"].split(" | ")[0]}' for d in desc]
+    dom_desc = desc[acc.index(dom)]
+    roofline["kernel_entry_point"] = dom_desc["entry_point"]
+    roofline["kernel_code_sha256"] = dom_desc["code_sha256"]
+    # HBM traffic of the dominant kernel is not measured in this run: it comes from the committed rocprofv3 --pmc
+    # summary, and only if that summary was taken from this very code object (same SHA-256), else null.
+    roofline["traffic_source"] = "profiles/dominant_conv_traffic.json (committed rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by a copy kernel of known size); not measured in this run"
     try:
         with open(os.path.join(ROOT, "profiles", "dominant_conv_traffic.json")) as f:
             tr = json.load(f)
-        if tr["dispatch_name"] == dom["name"] and (H, W) == (tr["height"], tr["width"]):
-            cfg = next(l.split()[1] for l in report.splitlines() if l.startswith("conv3x3_mfma ") and l.split()[2] == dom["name"])
-            roofline["kernel_config"] = cfg
-            roofline["traffic"] = tr["configs"][cfg]["fetch_bytes"] + tr["configs"][cfg]["write_bytes"]
-            roofline["traffic_unit"] = "bytes per launch (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel)"
-    except (OSError, KeyError, ValueError, StopIteration):
+        entry = tr["kernels"].get(dom_desc["code_sha256"])
+        if entry is not None and (H, W) == (tr["height"], tr["width"]):
+            roofline["traffic"] = entry["fetch_bytes"] + entry["write_bytes"]
+            roofline["traffic_unit"] = "bytes per launch"
+    except (OSError, KeyError, ValueError):
         pass
+
+    # The headline schedule folds every pool, upsample, concat, pad and crop into a convolution, so it has no
+    # bandwidth-only dispatch to report.  The stand-alone bandwidth kernels are timed here in a second, unfused
+    # schedule of the same network (not part of `value`): hipEvent pairs per dispatch, bytes as each dispatch declares them.
+    non_conv = None
+    if net == "oidn_unet" and not args.no_unfused_pass:
+        ublob = dx.compile_model(model, assume={"H": H, "W": W}, features=networks.UNFUSED_FEATURES, input_layout=lay, output_layout=lay)
+        uinst = dx.Module.load(ublob).instance(H=H, W=W)
+        uinst.infer_device(ins, None)
+        uinst.synchronize()
+        uacc = None
+        for _ in range(passes):
+            t = uinst.bench(warmup=2)
+            if uacc is None:
+                uacc = t
+            else:
+                for a2, b2 in zip(uacc, t):
+                    a2["latency_ms"] += b2["latency_ms"]
+        bw = [a2 for a2 in uacc if not (a2["flops"] > 0 and "conv" in a2["name"])]
+        bw_ms = sum(a2["latency_ms"] for a2 in bw) / passes
+        bw_bytes = sum(a2["memory_reads"] + a2["memory_writes"] for a2 in bw)
+        non_conv = {"dispatches": len(bw), "bytes": bw_bytes, "ms": bw_ms, "GBps": bw_bytes / bw_ms * 1e-6, "frac_of_hbm": bw_bytes / bw_ms * 1e-6 / PEAK_HBM_GBPS,
+                    "per_dispatch": [{"name": a2["name"], "in": a2["input"], "out": a2["output"], "GBps": round((a2["memory_reads"] + a2["memory_writes"]) / (a2["latency_ms"] / passes) * 1e-6, 1)} for a2 in bw],
+                    "note": "pool / upsample / concat / pad / slice dispatches of the same network compiled with those fusions switched off"}
+        del uinst
+        if other_ms == 0:
+            roofline["non_conv_GBps"] = non_conv["GBps"]
+            roofline["non_conv_frac_of_hbm"] = non_conv["frac_of_hbm"]
+            roofline["non_conv_source"] = "unfused second schedule (the timed schedule has no bandwidth-only dispatch)"
 
     line = {
         "metric": "oidn_unet_fp16_hwc_1080p_throughput" if args.workload == "oidn_1080p" else f"{args.workload}_throughput", "value": H * W / (ms * 1e-3) * 1e-6, "unit": "Mpix/s",
@@ -270,13 +322,21 @@ def main() -> int:
         "config": {"workload": f"{description}; {mod.runtime_model.dispatch_count} dispatches in one hipGraph", "device_bytes": inst.device_bytes,
                    "schedule": "min-cost over measured dispatch latencies" if db is not None else "min-cost over roofline estimates",
                    "tuning_seconds": round(tune_s, 2), "host_pointer_path_ms_per_frame": round(host_ms, 3), "host_pointer_pipelined_ms_per_frame": round(pipelined_ms, 3),
-                   "single_replay_ms_median": round(singles[len(singles) // 2], 4), "single_replay_ms_p95": round(singles[int(len(singles) * 0.95)], 4)},
+                   "single_replay_ms_median": round(singles[len(singles) // 2], 4), "single_replay_ms_p95": round(singles[int(len(singles) * 0.95)], 4),
+                   "schedule_configs": chosen},
         "roofline": roofline,
     }
+    if non_conv is not None:
+        line["non_conv_kernels"] = non_conv
+    rc = 0
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(net, net_kw, args.seed, H, W)
+        line["cpu_baseline"] = cpu_baseline(net, net_kw, args.seed, H, W, out_hwc)
+        line["parity"] = line["cpu_baseline"]["parity"]
+        if not line["parity"]["ok"]:
+            print(f"bench.py: the timed schedule's output misses the parity bar: {line['parity']}", file=sys.stderr)
+            rc = 1
     print(json.dumps(line))
-    return 0
+    return rc
 
 
 if __name__ == "__main__":

@@ -2,6 +2,7 @@
 #pragma GCC visibility push(default)
 #include "../../include/denox_hip.h"
 #pragma GCC visibility pop
+#include "common/sha256.hpp"
 #include "compiler/compile.hpp"
 #include "database/db.hpp"
 #include "device_info/device_info.hpp"
@@ -357,12 +358,20 @@ int denox_hip_dnx_describe(const void *dnxbuf, size_t size, const char *const *n
       o << "}";
     }
     o << "],\"binaries\":" << m.shader_binaries.size() << ",\"dispatches\":[";
+    // SHA-256 of each code object: what ties a profile or a measurement to the exact kernel a dispatch runs
+    std::vector<std::string> codeSha(m.shader_binaries.size());
+    for (size_t i = 0; i < m.shader_binaries.size(); ++i) {
+      Sha256 h;
+      h.update(m.shader_binaries[i].code_object.data(), m.shader_binaries[i].code_object.size());
+      codeSha[i] = Sha256::hex(h.digest());
+    }
     for (size_t i = 0; i < m.dispatches.size(); ++i) {
       const auto &d = m.dispatches[i];
       o << (i ? "," : "") << "{\"name\":"; jsonEscape(o, d.info.name);
       o << ",\"entry_point\":"; jsonEscape(o, d.entry_point);
       o << ",\"src_path\":"; jsonEscape(o, d.info.src_path);
       o << ",\"debug_info\":"; jsonEscape(o, d.info.debug_info);
+      o << ",\"code_sha256\":"; jsonEscape(o, d.binary_id < codeSha.size() ? codeSha[d.binary_id] : std::string());
       o << ",\"binary_id\":" << d.binary_id << ",\"workgroup_count\":[" << d.workgroup_count_x.eval(dp) << ',' << d.workgroup_count_y.eval(dp) << ',' << d.workgroup_count_z.eval(dp)
         << "],\"workgroup_size\":[" << d.workgroup_size[0] << ',' << d.workgroup_size[1] << ',' << d.workgroup_size[2] << "],\"bindings\":[";
       bool first = true;

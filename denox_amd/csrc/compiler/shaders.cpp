@@ -424,7 +424,7 @@ public:
     if (padB) k.define("PADB", 1);
     if (crop) k.define("CROP", 1);
     k.define("WAVES", cfg.waves); k.define("RPW", cfg.rpw); k.define("CK", cfg.fold ? 16u : stepChannels(cfg, g.CPAD));
-    if (cfg.resident) k.define("SLOTS", g.slots);
+    if (cfg.resident) { k.define("SLOTS", g.slots); k.define("NXCD", opt.deviceInfo.xcdCount); } // the grid below is xcdCount * nkt * slots workgroups
     if (cfg.pw) k.define("PW", cfg.pw);
     if (cfg.pp) k.define("PP", 1);
     if (conv.R != 3 || conv.S != 3) { k.define("KR", conv.R); k.define("KS", conv.S); }

@@ -57,9 +57,24 @@ HipCompiler::HipCompiler(std::string kernelDir, std::string cacheDir, std::strin
   } else {
     fail(Status::IoError, "kernel directory not found: " + m_kernelDir);
   }
-  std::sort(headers.begin(), headers.end());
-  for (const auto &h : headers) m_headerDigest += "//" + h + "\n" + readFile(m_kernelDir + "/" + h);
+  for (const auto &h : headers) m_headerText[h] = readFile(m_kernelDir + "/" + h);
   if (!m_cacheDir.empty()) mkdir(m_cacheDir.c_str(), 0755);
+}
+
+// Names of the headers of the kernel directory that `text` includes with #include "name".
+static std::vector<std::string> includedHeaders(const std::string &text) {
+  std::vector<std::string> out;
+  size_t pos = 0;
+  while ((pos = text.find("#include", pos)) != std::string::npos) {
+    pos += 8;
+    const size_t eol = text.find('\n', pos);
+    const size_t q0 = text.find('"', pos);
+    if (q0 == std::string::npos || (eol != std::string::npos && q0 > eol)) continue;
+    const size_t q1 = text.find('"', q0 + 1);
+    if (q1 == std::string::npos || (eol != std::string::npos && q1 > eol)) continue;
+    out.push_back(text.substr(q0 + 1, q1 - q0 - 1));
+  }
+  return out;
 }
 
 HipCompilerInstance HipCompiler::read(const std::string &relPath) const {
@@ -67,6 +82,21 @@ HipCompilerInstance HipCompiler::read(const std::string &relPath) const {
   inst.m_compiler = this;
   inst.m_path = relPath;
   inst.m_source = readFile(m_kernelDir + "/" + relPath);
+  // A kernel's identity covers the headers it can see, not every header of the directory: a change to the
+  // convolution headers leaves the cached code objects of the bandwidth kernels valid.
+  {
+    std::vector<std::string> seen, todo = includedHeaders(inst.m_source);
+    while (!todo.empty()) {
+      const std::string h = todo.back();
+      todo.pop_back();
+      auto it = m_headerText.find(h);
+      if (it == m_headerText.end() || std::find(seen.begin(), seen.end(), h) != seen.end()) continue;
+      seen.push_back(h);
+      for (const auto &n : includedHeaders(it->second)) todo.push_back(n);
+    }
+    std::sort(seen.begin(), seen.end());
+    for (const auto &h : seen) inst.m_headers += "//" + h + "\n" + m_headerText.at(h);
+  }
   // Experiment hook: extra "NAME=value NAME=value" definitions for every kernel (they take
   // part in the hash, so such code objects never mix with regular ones).
   if (const char *extra = std::getenv("DENOX_HIP_EXTRA_DEFINES")) {
@@ -93,7 +123,7 @@ std::string HipCompilerInstance::sha256() const {
   Sha256 h;
   h.update(m_source);
   h.update(std::string("\n//headers\n"));
-  h.update(m_compiler->m_headerDigest);
+  h.update(m_headers);
   h.update(std::string("\n//defines\n"));
   h.update(defineString());
   h.update(std::string("\n//flags\n"));

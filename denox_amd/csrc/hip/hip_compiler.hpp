@@ -37,6 +37,7 @@ private:
   const HipCompiler *m_compiler = nullptr;
   std::string m_path;   // path of the kernel source, relative to the kernel directory
   std::string m_source; // its text
+  std::string m_headers; // names and text of the kernel-directory headers it includes, directly or through them
   std::map<std::string, std::string> m_defines;
 };
 
@@ -55,7 +56,7 @@ public:
 private:
   friend class HipCompilerInstance;
   std::string m_kernelDir, m_cacheDir, m_arch;
-  std::string m_headerDigest; // text of every *.h in the kernel directory
+  std::map<std::string, std::string> m_headerText; // every *.h in the kernel directory
   mutable std::atomic<uint64_t> m_compiled{0}, m_cacheHits{0};
 };
 

@@ -25,7 +25,9 @@
 
 #define NKT (KOUTP / KT)
 #define CPADP (CPAD + 8)
-#define NXCD 8
+#ifndef NXCD
+#define NXCD 8 // accelerator dies, each with an L2 of its own; the host sizes the grid with the same number
+#endif
 #define NSTAGE ((PW > 0 ? PW : WAVES) * 64) // threads that stage halos
 
 extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(

@@ -25,7 +25,9 @@ static_assert(UPA == 1 && MF == 32 && !POOL && !CROP && !PADA && KR == 3 && KS =
 static_assert(CA % 8 == 0 && (CB == 0 || CB >= 8), "whole 8-channel vectors of A; at least one whole vector of B");
 
 #define NKT (KOUTP / KT)
-#define NXCD 8
+#ifndef NXCD
+#define NXCD 8 // accelerator dies, each with an L2 of its own; the host sizes the grid with the same number
+#endif
 #define CAP ((CA + 15) / 16 * 16)
 #define CBP ((CB + 15) / 16 * 16)
 #define APITCH (CAP + 8)

@@ -19,7 +19,7 @@ import numpy as np
 import pytest
 
 import denox_amd as dx
-from util import assert_bits_equal, assert_conv_close, he_weights, small_bias
+from util import assert_bits_equal, assert_conv_close, assert_reference_allclose, he_weights, small_bias
 
 pytestmark = pytest.mark.gpu
 
@@ -55,6 +55,8 @@ def run_case(oracle, build, C, in_layout=HWC, out_layout=HWC, H=100, W=100, exac
         assert_bits_equal(got, want)
     else:
         assert_conv_close(got, want)
+        # the reference's own bar, against the layers evaluated with binary16 tensors between them
+        assert_reference_allclose(got, oracle.run_graph(m.to_ops({"H": H, "W": W}), {"input": x}, "f16")[t.name])
 
 
 CONV_SHAPES = [(3, 3), (3, 32), (32, 3), (8, 16), (16, 8), (16, 32), (32, 16), (32, 32), (64, 64), (24, 24), (32, 48), (48, 48),

@@ -289,6 +289,77 @@ def test_full_size_oidn_unet_centre_of_crop(oracle):
         assert_conv_close(got[y0:y0 + h, x0:x0 + S][ys, xs], want[ys, xs], f"crop at {(y0, x0)}")
 
 
+def check_crops(oracle, m, x_hwc, got_hwc, H, W, spots, what, S=272, Mg=96):
+    """`got_hwc` (the full frame) against the oracle on 16-aligned S x S crops of the input: the U-Net's receptive field is
+    below Mg pixels, so a crop evaluation equals the full-frame result Mg pixels inside every cut edge (true image edges
+    keep their own padding and are compared up to the border)."""
+    for y0, x0 in spots:
+        y0 -= y0 % 16
+        x0 -= x0 % 16
+        h, w = min(S, H - y0), min(S, W - x0)
+        crop = np.ascontiguousarray(x_hwc[y0:y0 + h, x0:x0 + w])
+        want = oracle_net(oracle, m, crop, h, w)
+        ys = slice(0 if y0 == 0 else Mg, h if y0 + h >= H else h - Mg)
+        xs = slice(0 if x0 == 0 else Mg, w if x0 + w >= W else w - Mg)
+        assert_conv_close(got_hwc[y0:y0 + h, x0:x0 + w][ys, xs], want[ys, xs], f"{what}: crop at {(y0, x0)}")
+
+
+def test_full_size_4k_oidn_unet_centre_of_crop(oracle):
+    """The same network at 3840 x 2160 (no padding needed: 2160 = 16 x 135), the largest activation footprint."""
+    H, W = 2160, 3840
+    m, _ = networks.build("oidn_unet", seed=0)
+    x = networks.synthetic_input("oidn_unet", H, W, seed=3)
+    inst = dx.Module.compile(m, assume={"H": H, "W": W}).instance(H=H, W=W)
+    got = inst.infer(x)[0]
+    assert got.shape == (H, W, 3) and np.isfinite(got).all()
+    check_crops(oracle, m, x, got, H, W, [(0, 0), (1000, 2000), (H - 272, W - 272), (0, W - 272), (H - 272, 1600)], "4K")
+    assert_bits_equal(inst.infer(x)[0], got, "4K replay")
+
+
+def test_full_size_4k_bandwidth_kernels_bit_exact():
+    rng = np.random.default_rng(7)
+    H, W, C = 2160, 3840, 9
+    x = rng.standard_normal((H, W, C)).astype(np.float16)
+    m = dx.Model()
+    i = m.input("input", "W", "H", C)
+    m.output(m.concat(m.upsample(m.pool(i)), i))
+    got = dx.Module.compile(m).instance(H=H, W=W).infer(x)[0]
+    pooled = x.reshape(H // 2, 2, W // 2, 2, C).max(axis=(1, 3))
+    up = np.repeat(np.repeat(pooled, 2, axis=0), 2, axis=1)
+    assert_bits_equal(got, np.concatenate([up, x], axis=2), "pool/upsample/concat at 4K, 9 channels")
+
+
+def test_full_size_double_width_unet_chw_1077x1917(oracle):
+    """Every channel width doubled, CHW in and out, 1917 x 1077 (replicate-padded to 1920 x 1088 inside the network):
+    edge tiles, doubled widths and the layout conversion at the real extent."""
+    H, W = 1077, 1917
+    m, _ = networks.build("oidn_unet", seed=4, width_mult=2)
+    x = networks.synthetic_input("oidn_unet", H, W, seed=4)
+    mod = dx.Module.compile(m, input_layout=dx.Layout.CHW, output_layout=dx.Layout.CHW, assume={"H": H, "W": W})
+    got = mod.instance(H=H, W=W).infer(np.ascontiguousarray(x.transpose(2, 0, 1)))[0]
+    assert got.shape == (3, H, W) and np.isfinite(got).all()
+    got = got.transpose(1, 2, 0)
+    # the last two crops reach the replicate-padded bottom rows and right columns
+    check_crops(oracle, m, x, got, H, W, [(0, 0), (400, 800), (H - 272 + 16, W - 272 + 16), (H - 272 + 16, 0)], "2x width CHW")
+
+
+def test_full_size_schedule_selected_from_a_timing_table(oracle, tmp_path):
+    """What the benchmark times: populate -> bench on this GPU -> compile against the measured latencies, at 1920 x 1080.
+    Every selected dispatch must have been measured, and that schedule's output is checked on oracle crops."""
+    m, _ = networks.build("oidn_unet", seed=0)
+    x = networks.synthetic_input("oidn_unet", FULL_H, FULL_W, seed=0)
+    db = dx.Db(str(tmp_path / "gpu.db"))
+    db.populate(m, assume={"H": FULL_H, "W": FULL_W})
+    db.bench(min_samples=5, max_relative_error=0.05, max_samples=20)
+    blob = dx.compile_model(m, assume={"H": FULL_H, "W": FULL_W}, db=db)
+    report = dx.last_compile_report()
+    chosen = [l for l in report.splitlines()[1:] if l.strip()]
+    assert chosen and all(l.endswith(" measured") for l in chosen), report
+    got = dx.Module.load(blob).instance(H=FULL_H, W=FULL_W).infer(x)[0]
+    assert got.shape == (FULL_H, FULL_W, 3) and np.isfinite(got).all()
+    check_crops(oracle, m, x, got, FULL_H, FULL_W, [(0, 0), (400, 800), (FULL_H - 272 + 8, FULL_W - 272), (600, 0)], "tuned schedule")
+
+
 def test_model_file_round_trip_and_a_model_compiled_for_vulkan(tmp_path):
     # the bytes on disk are the whole model: save, load in a fresh Module, same bits out
     m, _ = networks.build("tiny_unet", seed=5)

@@ -26,6 +26,16 @@ def assert_conv_close(got_f16, want_f32, what=""):
     assert err.mean() <= CONV_MEAN_ABS * scale, f"{what}: mean abs err {err.mean():.4g}"
 
 
+def assert_reference_allclose(got_f16, want_f16, what="", rtol=1e-3, atol=1e-2):
+    """The reference's own acceptance: torch.allclose(output, expected, rtol=1e-3, atol=1e-2) against a binary16
+    evaluation of the same layers (test/__init__.py:45-49,97 of the reference)."""
+    got = np.asarray(got_f16, np.float32)
+    want = np.asarray(want_f16, np.float32)
+    assert got.shape == want.shape, (got.shape, want.shape)
+    excess = np.abs(got - want) - (atol + rtol * np.abs(want))
+    assert (excess <= 0).all(), f"{what}: |got - want| exceeds atol + rtol |want| by {excess.max():.4g} at {np.unravel_index(excess.argmax(), excess.shape)}"
+
+
 def assert_bits_equal(got, want, what=""):
     g = np.ascontiguousarray(got, np.float16).view(np.uint16)
     w = np.ascontiguousarray(want, np.float16).view(np.uint16)
