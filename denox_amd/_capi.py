@@ -124,6 +124,7 @@ SIGNATURES = {
     "denox_hip_instance_infer_many": (c_int, [c_void_p, c_uint32, POINTER(c_void_p), POINTER(c_void_p)]),
     "denox_hip_host_alloc": (c_int, [c_size_t, POINTER(c_void_p)]),
     "denox_hip_host_free": (None, [c_void_p]),
+    "denox_hip_instance_infer_device_static": (c_int, [c_void_p, POINTER(c_void_p), POINTER(c_void_p)]),
     "denox_hip_instance_synchronize": (c_int, [c_void_p]),
     "denox_hip_instance_input_device_ptr": (c_int, [c_void_p, c_uint32, POINTER(c_void_p)]),
     "denox_hip_instance_output_device_ptr": (c_int, [c_void_p, c_uint32, POINTER(c_void_p)]),

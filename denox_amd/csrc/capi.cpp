@@ -516,6 +516,10 @@ void denox_hip_host_free(void *p) { if (p) (void)hipHostFree(p); }
 int denox_hip_instance_infer_device(denox_hip_instance *inst, const void *const *in, void *const *out) {
   return guarded([&] { need(inst, "instance"); inst->inst->inferDevice(in, out); });
 }
+static_assert(DENOX_HIP_STATIC_SCRATCH_BYTES == runtime::kStaticScratchBytes, "header and library disagree on the static scratch size");
+int denox_hip_instance_infer_device_static(denox_hip_instance *inst, const void *const *in, void *const *out) {
+  return guarded([&] { need(inst, "instance"); inst->inst->inferDeviceStatic(in, out); });
+}
 int denox_hip_instance_synchronize(denox_hip_instance *inst) {
   return guarded([&] { need(inst, "instance"); inst->inst->synchronize(); });
 }

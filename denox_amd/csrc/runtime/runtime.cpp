@@ -20,6 +20,12 @@ Context::Context(int device) : m_device(device) {
   hipCheck(hipGetDeviceProperties(&m_props, device), "hipGetDeviceProperties");
   // default priority, non-blocking with respect to the null stream
   hipCheck(hipStreamCreateWithFlags(&m_stream, hipStreamNonBlocking), "hipStreamCreateWithFlags");
+  try {
+    m_staticScratch = staticScratchAddress(device); // set-up time: the allocation-free entry point must not have to ask
+  } catch (...) {
+    (void)hipStreamDestroy(m_stream);
+    throw;
+  }
 }
 
 Context::~Context() {
@@ -153,6 +159,7 @@ Instance::Instance(ModelHandle model, const std::vector<ValueSpec> &specs) : m_m
     for (size_t i : shared) items.push_back(ArenaItem{padded(i), first[i], last[i]});
     uint64_t arenaBytes = 0;
     const std::vector<uint64_t> at = plan_arena(items, arenaBytes, static_cast<int>(m_model->dispatches().size()));
+    m_arenaBytes = arenaBytes;
     if (arenaBytes) {
       hipCheck(hipMalloc(&m_arena, arenaBytes), "hipMalloc(arena)");
       m_deviceBytes += arenaBytes;
@@ -214,6 +221,16 @@ Instance::Instance(ModelHandle model, const std::vector<ValueSpec> &specs) : m_m
         l.ptrSlots.push_back(slot);
       }
       for (const auto &f : d.push_constant.fields) putScalar(l.args, pcOff + f.offset, f.dtype, f.source.eval(m_sym));
+      // the argument buffer of the allocation-free path: arena addresses become static-scratch addresses
+      l.staticArgs = l.args;
+      if (m_arena && m_arenaBytes <= kStaticScratchBytes && m_model->context()->staticScratch())
+        for (const auto &slot : l.ptrSlots) {
+          uint8_t *p = static_cast<uint8_t *>(tensorPtr(slot.tensor));
+          uint8_t *a = static_cast<uint8_t *>(m_arena);
+          if (p < a || p >= a + m_arenaBytes) continue;
+          void *q = static_cast<uint8_t *>(m_model->context()->staticScratch()) + (p - a);
+          std::memcpy(l.staticArgs.data() + slot.offset, &q, sizeof(void *));
+        }
       m_launches.push_back(std::move(l));
     }
     m_boundInputs.assign(m.inputs.size(), nullptr);
@@ -382,13 +399,13 @@ void Instance::selectGraph() {
 
 // Writes the given interface addresses into the argument buffers (no graph is touched): every bound tensor that lives
 // in an interface tensor's buffer follows that tensor's address.
-void Instance::patchInterface(const std::vector<void *> &inputs, const std::vector<void *> &outputs) {
+void Instance::patchInterface(const std::vector<void *> &inputs, const std::vector<void *> &outputs, bool staticArgs) {
   for (auto &l : m_launches)
     for (const auto &slot : l.ptrSlots) {
       if (slot.iface < 0) continue;
       void *base = slot.isInput ? inputs[static_cast<size_t>(slot.iface)] : outputs[static_cast<size_t>(slot.iface)];
       void *p = static_cast<uint8_t *>(base) + slot.delta;
-      std::memcpy(l.args.data() + slot.offset, &p, sizeof(void *));
+      std::memcpy((staticArgs ? l.staticArgs : l.args).data() + slot.offset, &p, sizeof(void *));
     }
 }
 
@@ -510,6 +527,28 @@ void Instance::inferDevice(const void *const *inputs, void *const *outputs) {
     hipCheck(hipGraphLaunch(m_graphExec, s), "hipGraphLaunch");
   else
     launchAll(s);
+}
+
+void Instance::inferDeviceStatic(const void *const *inputs, void *const *outputs) {
+  // No allocation on this path: no graph is captured or instantiated, nothing is malloc'ed on the device; the
+  // argument buffers exist since the instance was made and are only overwritten in place.
+  const dnx::Model &m = m_model->dnx();
+  if (m_arenaBytes > kStaticScratchBytes)
+    fail(Status::Unsupported, "this instance needs " + std::to_string(m_arenaBytes) + " bytes for its intermediate tensors; the static scratch array holds " +
+                                  std::to_string(kStaticScratchBytes));
+  if (m_arenaBytes && !m_arena) fail(Status::Unsupported, "the allocation-free path needs the intermediate buffers in one arena (DENOX_HIP_NO_ALIAS is set)");
+  if (!m_model->context()->staticScratch()) fail(Status::HipError, "the static scratch array has no device address");
+  m_model->context()->makeCurrent();
+  for (auto &l : m_launches)
+    for (const auto &slot : l.ptrSlots) {
+      if (slot.iface < 0) continue;
+      void *ext = slot.isInput ? (inputs ? const_cast<void *>(inputs[slot.iface]) : nullptr) : (outputs ? outputs[slot.iface] : nullptr);
+      void *base = ext ? ext : tensorPtr(slot.isInput ? m.inputs[static_cast<size_t>(slot.iface)] : m.outputs[static_cast<size_t>(slot.iface)]);
+      void *p = static_cast<uint8_t *>(base) + slot.delta;
+      std::memcpy(l.staticArgs.data() + slot.offset, &p, sizeof(void *));
+    }
+  hipStream_t s = m_model->context()->stream();
+  for (auto &l : m_launches) launchOne(l.fn, l.grid, l.block, l.staticArgs, s);
 }
 
 void Instance::synchronize() {

@@ -32,13 +32,20 @@ public:
   hipStream_t stream() const { return m_stream; }
   void makeCurrent() const;
   const hipDeviceProp_t &props() const { return m_props; }
+  // this device's copy of the library's static scratch array (static_scratch.hip); resolved when the context is made
+  void *staticScratch() const { return m_staticScratch; }
 
 private:
   int m_device;
   hipStream_t m_stream = nullptr;
   hipDeviceProp_t m_props;
+  void *m_staticScratch = nullptr;
 };
 
+// The library's allocation-free path keeps intermediate results in a file-scope device array of this many bytes per GPU.
+constexpr uint64_t kStaticScratchBytes = 64ull << 20;
+// Device address of that array on `device`, which must be current (hipGetSymbolAddress once per device, then cached).
+void *staticScratchAddress(int device);
 using ContextHandle = std::shared_ptr<Context>;
 
 struct ModelDispatch {
@@ -95,6 +102,11 @@ public:
   // stream and returns without synchronising.  A null entry means "use the
   // instance's own buffer for that tensor" (see inputDevicePtr/outputDevicePtr).
   void inferDevice(const void *const *inputs, void *const *outputs);
+  // inferDevice without any allocation: plain launches (no graph is built or instantiated) with the intermediate
+  // buffers placed in the library's static scratch array instead of this instance's arena.  Fails when the arena
+  // would not fit.  Every instance on one GPU shares that array: calls that overlap in time race.
+  void inferDeviceStatic(const void *const *inputs, void *const *outputs);
+  uint64_t arenaBytes() const { return m_arenaBytes; }
   // A sequence of frames from host memory, arrays frame-major (inputs[f * inputCount() + i]); blocking.
   // Upload of frame f+1, the dispatches of frame f and the download of frame f-1 run at the same time on three
   // streams: the interface tensors exist twice, everything in between once (the dispatches of consecutive frames
@@ -121,6 +133,7 @@ private:
     hipFunction_t fn;
     unsigned grid[3], block[3];
     std::vector<uint8_t> args;              // pointers then push constants
+    std::vector<uint8_t> staticArgs;        // the same with arena addresses replaced by static-scratch addresses
     // One per bound tensor.  A tensor that lives in the buffer of an interface tensor (that tensor itself, or a channel
     // range of it written in place) follows the interface address: iface = index into inputs (isInput) / outputs,
     // delta = byte distance from the interface tensor's start; iface < 0 otherwise.
@@ -132,7 +145,7 @@ private:
   void launchAll(hipStream_t s);
   void buildGraph();
   void rebind(const void *const *inputs, void *const *outputs);
-  void patchInterface(const std::vector<void *> &inputs, const std::vector<void *> &outputs);
+  void patchInterface(const std::vector<void *> &inputs, const std::vector<void *> &outputs, bool staticArgs = false);
   void preparePipeline();
 
   ModelHandle m_model;
@@ -140,6 +153,7 @@ private:
   std::vector<void *> m_buffers;
   std::vector<char> m_ownBuffer; // 1: an allocation of its own, 0: a range of m_arena
   void *m_arena = nullptr;       // memory shared by the intermediate buffers
+  uint64_t m_arenaBytes = 0;
   void freeBuffers();
   std::vector<uint64_t> m_bufferSizes;
   std::vector<Launch> m_launches;

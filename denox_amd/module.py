@@ -314,6 +314,12 @@ class Instance:
         pout = (c_void_p * self.output_count)(*outputs) if outputs is not None else None
         _capi.check(_capi.lib().denox_hip_instance_infer_device(self._h, pin, pout))
 
+    def infer_device_static(self, inputs: Optional[Sequence[int]] = None, outputs: Optional[Sequence[int]] = None) -> None:
+        """`infer_device` without any device allocation: plain launches, intermediates in the library's static scratch array."""
+        pin = (c_void_p * self.input_count)(*inputs) if inputs is not None else None
+        pout = (c_void_p * self.output_count)(*outputs) if outputs is not None else None
+        _capi.check(_capi.lib().denox_hip_instance_infer_device_static(self._h, pin, pout))
+
     def synchronize(self) -> None:
         _capi.check(_capi.lib().denox_hip_instance_synchronize(self._h))
 

@@ -263,6 +263,16 @@ void denox_hip_host_free(void *p);
 /* asynchronous on the context's stream; device arrays, entries (or the arrays
  * themselves) may be NULL to use the instance's own tensors */
 int denox_hip_instance_infer_device(denox_hip_instance *inst, const void *const *dev_inputs, void *const *dev_outputs);
+/* denox_hip_instance_infer_device for callers that cannot allocate (code under HIP graph capture, serving loops and
+ * harnesses that forbid hipMalloc): same arguments, same results bit for bit, and no allocation of any kind on the
+ * device -- plain kernel launches on the context's stream (no graph is captured or instantiated), with the instance's
+ * intermediate tensors kept in a static device array that the library holds on every GPU it runs on
+ * (DENOX_HIP_STATIC_SCRATCH_BYTES, resolved when the context is created).  It has no counterpart in the reference,
+ * whose Instance allocates every buffer it uses (runtime/src/denox/runtime/instance.cpp:65-113).
+ * Returns DENOX_HIP_UNSUPPORTED, with the size needed in the error text, when the instance's intermediate tensors need more than that.  All instances on one GPU share the array and each call
+ * overwrites it: calls that overlap in time on one GPU race, and nothing in it survives from one call to the next. */
+#define DENOX_HIP_STATIC_SCRATCH_BYTES (64ull << 20)
+int denox_hip_instance_infer_device_static(denox_hip_instance *inst, const void *const *dev_inputs, void *const *dev_outputs);
 int denox_hip_instance_synchronize(denox_hip_instance *inst);
 int denox_hip_instance_input_device_ptr(const denox_hip_instance *inst, uint32_t i, void **out);
 int denox_hip_instance_output_device_ptr(const denox_hip_instance *inst, uint32_t i, void **out);
