@@ -40,7 +40,8 @@ class CompileOptions(Structure):
                 ("enable_slice_fusion", c_int32), ("enable_alternating_traversal", c_int32), ("enable_upsample_fold", c_int32), ("enable_implicit_concat", c_int32), ("input_format", c_int32),
                 ("output_format", c_int32), ("assumption_count", c_uint32), ("assumption_names", POINTER(c_char_p)),
                 ("assumption_values", POINTER(c_int64)), ("force_conv_config", c_char_p), ("device", c_int32),
-                ("populate_compile_kernels", c_int32), ("kernel_shard_index", c_uint32), ("kernel_shard_count", c_uint32)]
+                ("populate_compile_kernels", c_int32), ("kernel_shard_index", c_uint32), ("kernel_shard_count", c_uint32),
+                ("enable_conv_conv_fusion", c_int32)]
 
 
 class DbBenchOptions(Structure):

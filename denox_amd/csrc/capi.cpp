@@ -83,6 +83,7 @@ compiler::CompileOptions toOptions(const denox_hip_compile_options *o) {
   opt.features.enableAlternatingTraversal = o->enable_alternating_traversal != 0;
   opt.features.enableUpsampleFold = o->enable_upsample_fold != 0;
   opt.features.enableImplicitConcat = o->enable_implicit_concat != 0;
+  opt.features.enableConvConvFusion = o->enable_conv_conv_fusion != 0;
   auto fmt = [](int f) {
     switch (f) {
     case 0: case DENOX_HIP_FORMAT_HWC: return dnx::TensorFormat::SSBO_HWC;
@@ -249,6 +250,7 @@ void denox_hip_compile_options_default(denox_hip_compile_options *o) {
   o->enable_alternating_traversal = 1;
   o->enable_upsample_fold = 1;
   o->enable_implicit_concat = 1;
+  o->enable_conv_conv_fusion = 1;
   o->device = -1;
   o->populate_compile_kernels = 1;
   o->kernel_shard_index = 0;

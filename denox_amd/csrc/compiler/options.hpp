@@ -20,6 +20,7 @@ struct Features {
   bool enableUpsampleFold = true;     // candidates that fold a fused 2x upsample into the conv weights (2x2 taps per output parity)
   bool enableAlternatingTraversal = true; // consecutive conv dispatches walk their tiles in opposite directions
   bool enableImplicitConcat = true;   // memory-aliasing concat where layouts allow it
+  bool enableConvConvFusion = true;   // two consecutive 3x3 convolutions in one dispatch, the tensor between them kept in LDS
 };
 
 struct InterfaceTensorDescriptor {

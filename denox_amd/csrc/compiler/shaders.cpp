@@ -85,7 +85,7 @@ const ConvConfig kConvConfigs[] = {
 };
 constexpr unsigned kNumConvConfigs = sizeof(kConvConfigs) / sizeof(kConvConfigs[0]);
 
-enum ConvPatternBits : unsigned { PAT_CONCAT = 1, PAT_UPSAMPLE = 2, PAT_ACT = 4, PAT_POOL = 8, PAT_PADA = 16, PAT_PADB = 32, PAT_CROP = 64 };
+enum ConvPatternBits : unsigned { PAT_CONCAT = 1, PAT_UPSAMPLE = 2, PAT_ACT = 4, PAT_POOL = 8, PAT_PADA = 16, PAT_PADB = 32, PAT_CROP = 64, PAT_ACT_FIRST = 128 };
 
 struct ConvGeometry {
   unsigned CA, CB, C, CPAD, K, KOUTP, KT, slots;
@@ -256,6 +256,8 @@ std::vector<uint8_t> packFoldWeights(const Op &conv, const FoldGeometry &g) {
   return bytes;
 }
 
+bool isPairConfigName(const std::string &name); // a configuration of the conv -> conv shader below
+
 class ConvMfmaShader final : public IShader {
 public:
   explicit ConvMfmaShader(const hip::HipCompiler *c) : m_compiler(c) {}
@@ -276,52 +278,66 @@ public:
     return out;
   }
 
+  // What can be folded in front of a convolution (sources seen through an upsample, a replicate pad, a concat) and
+  // behind it (activation, then a 2x2 max pool or a crop).  A fused-away tensor may have other consumers: whoever needs
+  // it materialised gets it from another edge, and the selection weighs both.
+  struct Pro { unsigned bits; std::vector<int> ops; std::vector<int> inputs; };
+  struct Epi { unsigned bits; std::vector<int> ops; int output; };
+  static bool convSupported(const Op &conv) {
+    // filters up to 7 x 7, zero padding up to 15, strides up to 4, no dilation (the reference's conv shaders take
+    // kernel size, STRIDE_* and PADDING_* as parameters as well and have no dilation either)
+    return conv.kind == OpKind::Conv && !(conv.R < 1 || conv.S < 1 || conv.R > 7 || conv.S > 7 || conv.strideX < 1 || conv.strideY < 1 || conv.strideX > 4 ||
+                                          conv.strideY > 4 || conv.padX > 15 || conv.padY > 15 || conv.dilX != 1 || conv.dilY != 1);
+  }
+  static std::vector<Pro> prologuesOf(const Model &model, const Op &conv, const CompileOptions &opt) {
+    const auto &ops = model.ops();
+    std::vector<Pro> pros;
+    const TensorHandle in = conv.inputs[0];
+    for (const Source &s : sourcesOf(model, in, true, PAT_PADA, opt)) pros.push_back(Pro{s.bits, s.ops, {s.tensor}});
+    const int prod = model.tensors()[in].producer;
+    if (prod >= 0 && ops[prod].kind == OpKind::Concat && opt.features.enableConcatConvFusion) {
+      const Op &cat = ops[prod];
+      for (const Source &a : sourcesOf(model, cat.inputs[0], true, PAT_PADA, opt))
+        for (const Source &b : sourcesOf(model, cat.inputs[1], false, PAT_PADB, opt)) {
+          if ((a.bits & PAT_PADA) && (b.bits & PAT_PADB)) continue; // one padded source per dispatch
+          Pro p{PAT_CONCAT | a.bits | b.bits, a.ops, {a.tensor, b.tensor}};
+          p.ops.insert(p.ops.end(), b.ops.begin(), b.ops.end());
+          p.ops.push_back(prod);
+          pros.push_back(std::move(p));
+        }
+    }
+    return pros;
+  }
+  static std::vector<Epi> epiloguesOf(const Model &model, const Op &conv, const CompileOptions &opt) {
+    const auto &ops = model.ops();
+    std::vector<Epi> epis;
+    epis.push_back(Epi{0, {}, conv.output});
+    auto poolOk = [](const Op &q) { return q.kind == OpKind::Pool && q.poolFunc == PoolFunction::Max && q.kernelX == 2 && q.kernelY == 2 && q.poolStrideX == 2 && q.poolStrideY == 2 && q.poolPadX == 0 && q.poolPadY == 0; };
+    auto tails = [&](TensorHandle t, unsigned bits, std::vector<int> chain) {
+      if (!singleUse(model, t)) return;
+      const int c = model.tensors()[t].consumers[0];
+      if (poolOk(ops[c]) && opt.features.enablePoolFusion) { auto ch = chain; ch.push_back(c); epis.push_back(Epi{bits | PAT_POOL, ch, ops[c].output}); }
+      if (ops[c].kind == OpKind::Slice && opt.features.enableSliceFusion) { auto ch = chain; ch.push_back(c); epis.push_back(Epi{bits | PAT_CROP, ch, ops[c].output}); }
+    };
+    tails(conv.output, 0, {});
+    if (singleUse(model, conv.output)) {
+      const int c1 = model.tensors()[conv.output].consumers[0];
+      if (ops[c1].kind == OpKind::Activation && opt.features.enableConvReluFusion) {
+        epis.push_back(Epi{PAT_ACT, {c1}, ops[c1].output});
+        tails(ops[c1].output, PAT_ACT, {c1});
+      }
+    }
+    return epis;
+  }
+
   std::vector<Match> matchAll(const Model &model, const CompileOptions &opt) const override {
     std::vector<Match> out;
     const auto &ops = model.ops();
     for (size_t i = 0; i < ops.size(); ++i) {
       const Op &conv = ops[i];
-      if (conv.kind != OpKind::Conv) continue;
-      // filters up to 7 x 7, zero padding up to 15, strides up to 4, no dilation (the reference's conv shaders take
-      // kernel size, STRIDE_* and PADDING_* as parameters as well and have no dilation either)
-      if (conv.R < 1 || conv.S < 1 || conv.R > 7 || conv.S > 7 || conv.strideX < 1 || conv.strideY < 1 || conv.strideX > 4 || conv.strideY > 4 ||
-          conv.padX > 15 || conv.padY > 15 || conv.dilX != 1 || conv.dilY != 1) continue;
-      // A fused-away tensor may have other consumers: whoever needs it materialised gets it
-      // from another edge, and the selection weighs both.
-      struct Pro { unsigned bits; std::vector<int> ops; std::vector<int> inputs; };
-      std::vector<Pro> pros;
-      const TensorHandle in = conv.inputs[0];
-      for (const Source &s : sourcesOf(model, in, true, PAT_PADA, opt)) pros.push_back(Pro{s.bits, s.ops, {s.tensor}});
-      const int prod = model.tensors()[in].producer;
-      if (prod >= 0 && ops[prod].kind == OpKind::Concat && opt.features.enableConcatConvFusion) {
-        const Op &cat = ops[prod];
-        for (const Source &a : sourcesOf(model, cat.inputs[0], true, PAT_PADA, opt))
-          for (const Source &b : sourcesOf(model, cat.inputs[1], false, PAT_PADB, opt)) {
-            if ((a.bits & PAT_PADA) && (b.bits & PAT_PADB)) continue; // one padded source per dispatch
-            Pro p{PAT_CONCAT | a.bits | b.bits, a.ops, {a.tensor, b.tensor}};
-            p.ops.insert(p.ops.end(), b.ops.begin(), b.ops.end());
-            p.ops.push_back(prod);
-            pros.push_back(std::move(p));
-          }
-      }
-      struct Epi { unsigned bits; std::vector<int> ops; int output; };
-      std::vector<Epi> epis;
-      epis.push_back(Epi{0, {}, conv.output});
-      auto poolOk = [](const Op &q) { return q.kind == OpKind::Pool && q.poolFunc == PoolFunction::Max && q.kernelX == 2 && q.kernelY == 2 && q.poolStrideX == 2 && q.poolStrideY == 2 && q.poolPadX == 0 && q.poolPadY == 0; };
-      auto tails = [&](TensorHandle t, unsigned bits, std::vector<int> chain) {
-        if (!singleUse(model, t)) return;
-        const int c = model.tensors()[t].consumers[0];
-        if (poolOk(ops[c]) && opt.features.enablePoolFusion) { auto ch = chain; ch.push_back(c); epis.push_back(Epi{bits | PAT_POOL, ch, ops[c].output}); }
-        if (ops[c].kind == OpKind::Slice && opt.features.enableSliceFusion) { auto ch = chain; ch.push_back(c); epis.push_back(Epi{bits | PAT_CROP, ch, ops[c].output}); }
-      };
-      tails(conv.output, 0, {});
-      if (singleUse(model, conv.output)) {
-        const int c1 = model.tensors()[conv.output].consumers[0];
-        if (ops[c1].kind == OpKind::Activation && opt.features.enableConvReluFusion) {
-          epis.push_back(Epi{PAT_ACT, {c1}, ops[c1].output});
-          tails(ops[c1].output, PAT_ACT, {c1});
-        }
-      }
+      if (!convSupported(conv)) continue;
+      const std::vector<Pro> pros = prologuesOf(model, conv, opt);
+      const std::vector<Epi> epis = epiloguesOf(model, conv, opt);
       for (const auto &p : pros)
         for (const auto &e : epis) {
           Match m;
@@ -353,11 +369,13 @@ public:
     const unsigned CA = model.tensors()[m.inputs[0]].channels;
     const unsigned CB = m.inputs.size() > 1 ? model.tensors()[m.inputs[1]].channels : 0;
     std::vector<unsigned> out;
+    // a forced configuration of the conv -> conv shader restricts that shader only: single convolutions keep their choice
+    const std::string forced = isPairConfigName(opt.forceConvConfig) ? std::string() : opt.forceConvConfig;
     for (unsigned c = 0; c < kNumConvConfigs; ++c) {
       const ConvConfig &cfg = kConvConfigs[c];
       const unsigned kstep = cfg.mf == 32 ? 16 : 32;
       const unsigned cpad = (CA + CB + kstep - 1) / kstep * kstep;
-      if (!opt.forceConvConfig.empty() && opt.forceConvConfig != cfg.name) continue;
+      if (!forced.empty() && forced != cfg.name) continue;
       if (cfg.fold) {
         const unsigned others = PAT_POOL | PAT_CROP | PAT_PADA;
         FoldGeometry fg;
@@ -377,9 +395,9 @@ public:
       out.push_back(c);
     }
     bool forcedFold = false; // a forced upsample-folding configuration leaves matches without an upsample to nobody: not an error
-    for (unsigned c = 0; c < kNumConvConfigs; ++c) forcedFold |= kConvConfigs[c].fold && opt.forceConvConfig == kConvConfigs[c].name;
-    if (out.empty() && !opt.forceConvConfig.empty() && !(forcedFold && !(m.pattern & PAT_UPSAMPLE)))
-      fail(Status::Unsupported, "conv configuration '" + opt.forceConvConfig + "' is not valid for this layer");
+    for (unsigned c = 0; c < kNumConvConfigs; ++c) forcedFold |= kConvConfigs[c].fold && forced == kConvConfigs[c].name;
+    if (out.empty() && !forced.empty() && !(forcedFold && !(m.pattern & PAT_UPSAMPLE)))
+      fail(Status::Unsupported, "conv configuration '" + forced + "' is not valid for this layer");
     return out;
   }
 
@@ -507,6 +525,240 @@ public:
     d.setMemoryReads(reads);
     d.setMemoryWrites(bytesOf(sym, model.tensors()[m.output]));
     d.setFlops(sym.mul(sym.mul(OW, OH), static_cast<int64_t>(2) * conv.R * conv.S * conv.C * conv.K));
+  }
+
+private:
+  const hip::HipCompiler *m_compiler;
+};
+
+// ------------------------------------------------------------------ conv -> conv
+// Two consecutive 3x3 convolutions (stride 1, extent-preserving) whose intermediate tensor has at most 32 channels and no
+// other consumer, in one dispatch (conv3x3_pair.hip): the intermediate tensor stays in LDS.  Everything the
+// single-convolution shader folds in front of a convolution is available in front of the first one, everything it folds
+// behind a convolution behind the second one.  The reference fuses for the same purpose -- to keep a tensor from
+// crossing memory -- in ConcatConvCMShader (conv/ConcatConvCMShader.cpp:760-965); a conv -> conv fusion it does not have.
+struct PairConfig { unsigned waves, rpw, ck; const char *name; }; // ck: input channels of the first convolution per LDS stage
+const PairConfig kPairConfigs[] = {{8, 2, 16, "x8r2k16"}, {4, 2, 32, "x4r2k32"}, {4, 4, 16, "x4r4k16"}, {4, 2, 16, "x4r2k16"}};
+constexpr unsigned kNumPairConfigs = sizeof(kPairConfigs) / sizeof(kPairConfigs[0]);
+
+bool isPairConfigName(const std::string &name) {
+  for (const PairConfig &c : kPairConfigs) if (name == c.name) return true;
+  return false;
+}
+
+struct PairGeometry { unsigned CA, CB, C, CPAD, K1, K2, ck, slots; bool tapm; size_t ldsBytes; };
+
+bool choosePair(const PairConfig &cfg, unsigned CA, unsigned CB, unsigned K1, unsigned K2, bool pool, const DeviceInfo &dev, PairGeometry &g) {
+  g.CA = CA; g.CB = CB; g.C = CA + CB; g.CPAD = (g.C + 15) / 16 * 16; g.K1 = K1; g.K2 = K2;
+  if (K1 > 32 || K2 > 32 || cfg.ck % 16 || cfg.ck > 64) return false;
+  if (cfg.ck > g.CPAD && cfg.ck != 16) return false; // a larger stage than the whole reduction adds nothing
+  g.ck = std::min(cfg.ck, g.CPAD);
+  const unsigned ih = cfg.waves * cfg.rpw, haloPix = (ih + 2) * 34, ckp = g.ck + 8, threads = cfg.waves * 64;
+  if ((haloPix * (g.ck / 8) + threads - 1) / threads > 64) return false;
+  const unsigned regBudget = std::min(256u, 512u / ((cfg.waves + 3) / 4));
+  // A second convolution with at most 5 output channels carries its three filter columns in the matrix rows (TAPM in
+  // conv3x3_pair.hip): a third of the matrix instructions, weights of 3 instead of 9 taps in registers.
+  g.tapm = 3 * K2 <= 15 && !pool;
+  // the second convolution's weights (taps x 2 fragments of 4 registers), one accumulator set, fragments, the converted tile, halo registers
+  if ((g.tapm ? 24 : 72) + cfg.rpw * 16 + 96 > regBudget) return false;
+  const unsigned nchunk = (g.CPAD + g.ck - 1) / g.ck;
+  const unsigned ringRows = nchunk == 1 ? 2 * ih + 2 : ih + 2; // see conv3x3_pair.hip
+  g.ldsBytes = static_cast<size_t>(9 * 32) * (g.CPAD + 8) * 2 + 2 * static_cast<size_t>(haloPix) * ckp * 2 + (static_cast<size_t>(ringRows) * 32 + 2) * 40 * 2 + 2 * 32 * 4;
+  if (g.ldsBytes > dev.maxComputeSharedMemory) return false;
+  g.slots = std::max(1u, dev.computeUnits / dev.xcdCount);
+  return true;
+}
+
+// [tap][32 rows][cpad] with the rows permuted as the kernels' epilogue expects (rowChannel), zero beyond K and C
+std::vector<uint8_t> packPairWeights(const Op &conv, unsigned cpad) {
+  ConvGeometry g{};
+  g.C = conv.C; g.CPAD = cpad; g.K = conv.K; g.KOUTP = 32; g.KT = 32;
+  return packConvWeights(conv, g, cpad, 32);
+}
+
+// Second convolution with its filter columns in the matrix rows: [r][32 rows][32 channels]; the row that the epilogue
+// reads as channel s * K + k holds W[k][c][r][s] (zero elsewhere).
+std::vector<uint8_t> packPairWeightsTapM(const Op &conv) {
+  std::vector<uint16_t> out(static_cast<size_t>(3) * 32 * 32, 0);
+  for (unsigned r = 0; r < 3; ++r)
+    for (unsigned row = 0; row < 32; ++row) {
+      const unsigned lam = rowChannel(32, 32, row);
+      if (lam >= 3 * conv.K) continue;
+      const unsigned s = lam / conv.K, k = lam % conv.K;
+      for (unsigned c = 0; c < conv.C; ++c) out[(static_cast<size_t>(r) * 32 + row) * 32 + c] = conv.weights[((static_cast<size_t>(k) * conv.C + c) * 3 + r) * 3 + s];
+    }
+  std::vector<uint8_t> bytes(out.size() * 2);
+  std::memcpy(bytes.data(), out.data(), bytes.size());
+  return bytes;
+}
+
+class ConvPairShader final : public IShader {
+public:
+  explicit ConvPairShader(const hip::HipCompiler *c) : m_compiler(c) {}
+  std::string name() const override { return "conv3x3_pair"; }
+
+  static bool plain3x3(const Op &c) {
+    return ConvMfmaShader::convSupported(c) && c.R == 3 && c.S == 3 && c.strideX == 1 && c.strideY == 1 && c.padX == 1 && c.padY == 1 && c.K <= 32;
+  }
+
+  std::vector<Match> matchAll(const Model &model, const CompileOptions &opt) const override {
+    std::vector<Match> out;
+    if (!opt.features.enableConvConvFusion) return out;
+    const auto &ops = model.ops();
+    for (size_t i = 0; i < ops.size(); ++i) {
+      const Op &first = ops[i];
+      if (!plain3x3(first) || !singleUse(model, first.output)) continue;
+      std::vector<int> mid{static_cast<int>(i)};
+      unsigned midBits = 0;
+      int next = model.tensors()[first.output].consumers[0];
+      if (ops[next].kind == OpKind::Activation && opt.features.enableConvReluFusion && singleUse(model, ops[next].output)) {
+        mid.push_back(next);
+        midBits = PAT_ACT_FIRST;
+        next = model.tensors()[ops[next].output].consumers[0];
+      }
+      const Op &second = ops[next];
+      if (!plain3x3(second) || second.C != first.K) continue;
+      mid.push_back(next);
+      for (const auto &p : ConvMfmaShader::prologuesOf(model, first, opt))
+        for (const auto &e : ConvMfmaShader::epiloguesOf(model, second, opt)) {
+          Match m;
+          m.pattern = p.bits | e.bits | midBits;
+          m.ops = p.ops;
+          m.ops.insert(m.ops.end(), mid.begin(), mid.end());
+          m.ops.insert(m.ops.end(), e.ops.begin(), e.ops.end());
+          m.inputs = p.inputs;
+          m.output = e.output;
+          out.push_back(std::move(m));
+        }
+    }
+    return out;
+  }
+
+  // the two convolutions of a match, in order
+  static std::pair<const Op *, const Op *> convsOf(const Model &model, const Match &m) {
+    const Op *a = nullptr, *b = nullptr;
+    for (int o : m.ops)
+      if (model.ops()[o].kind == OpKind::Conv) (a ? b : a) = &model.ops()[o];
+    if (!a || !b) fail(Status::Internal, "conv pair match lacks a convolution");
+    return {a, b};
+  }
+
+  std::vector<unsigned> acceptMatch(const Model &model, const Match &m, const CompileOptions &opt) const override {
+    const auto [first, second] = convsOf(model, m);
+    const unsigned CA = model.tensors()[m.inputs[0]].channels;
+    const unsigned CB = m.inputs.size() > 1 ? model.tensors()[m.inputs[1]].channels : 0;
+    std::vector<unsigned> out;
+    for (unsigned c = 0; c < kNumPairConfigs; ++c) {
+      const PairConfig &cfg = kPairConfigs[c];
+      if (isPairConfigName(opt.forceConvConfig) && opt.forceConvConfig != cfg.name) continue;
+      if ((m.pattern & PAT_POOL) && (cfg.rpw % 2)) continue;
+      if (cfg.waves * 64 > opt.deviceInfo.maxComputeWorkGroupInvocations) continue;
+      PairGeometry g;
+      if (choosePair(cfg, CA, CB, first->K, second->K, (m.pattern & PAT_POOL) != 0, opt.deviceInfo, g)) out.push_back(c);
+    }
+    return out;
+  }
+
+  size_t parameterMemorySize(const Model &model, const Match &m) const override {
+    const auto [first, second] = convsOf(model, m);
+    return static_cast<size_t>(9 * 32) * ((first->C + 15) / 16 * 16 + 32) * 2 + 4 * 32;
+    (void)second;
+  }
+
+  void implement(OpImpl &impl, const Model &model, const Match &m, unsigned config, SymGraph &sym, const CompileOptions &opt) const override {
+    const PairConfig &cfg = kPairConfigs[config];
+    const auto [firstP, secondP] = convsOf(model, m);
+    const Op &first = *firstP, &second = *secondP;
+    const TensorNode &convIn = model.tensors()[first.inputs[0]];
+    const TensorNode &tA = model.tensors()[m.inputs[0]];
+    const unsigned CA = tA.channels, CB = m.inputs.size() > 1 ? model.tensors()[m.inputs[1]].channels : 0;
+    PairGeometry g;
+    if (!choosePair(cfg, CA, CB, first.K, second.K, (m.pattern & PAT_POOL) != 0, opt.deviceInfo, g)) fail(Status::Internal, "conv pair config rejected at implement time");
+    // activations: the one between the convolutions is the first Activation op of the match when PAT_ACT_FIRST is set
+    int act1 = 0, act2 = 0;
+    float alpha1 = 0.0f, alpha2 = 0.0f;
+    {
+      bool seenSecond = false;
+      for (int o : m.ops) {
+        const Op &op = model.ops()[o];
+        if (&op == &second) seenSecond = true;
+        if (op.kind != OpKind::Activation) continue;
+        const int a = op.func == ActivationFunction::ReLU ? 1 : 2;
+        if (!seenSecond) { act1 = a; alpha1 = op.alpha; } else { act2 = a; alpha2 = op.alpha; }
+      }
+    }
+    const bool pool = (m.pattern & PAT_POOL) != 0, up = (m.pattern & PAT_UPSAMPLE) != 0, crop = (m.pattern & PAT_CROP) != 0;
+    const bool padA = (m.pattern & PAT_PADA) != 0, padB = (m.pattern & PAT_PADB) != 0;
+
+    hip::HipCompilerInstance k = m_compiler->read("conv3x3_pair.hip");
+    k.define("CA", CA); k.define("CB", CB); k.define("UPA", up ? 1 : 0);
+    k.define("K1", first.K); k.define("ACT1", act1); k.define("HAS_BIAS1", first.hasBias ? 1 : 0);
+    if (act1 == 2) k.define("ALPHA1", fmtFloat(alpha1));
+    k.define("KOUT", second.K); k.define("KT", 32); k.define("ACT", act2); k.define("HAS_BIAS", second.hasBias ? 1 : 0);
+    if (act2 == 2) k.define("ALPHA", fmtFloat(alpha2));
+    k.define("POOL", pool ? 1 : 0);
+    if (padA) k.define("PADA", 1);
+    if (padB) k.define("PADB", 1);
+    if (crop) k.define("CROP", 1);
+    k.define("WAVES", cfg.waves); k.define("RPW", cfg.rpw); k.define("CK", g.ck);
+    k.define("SLOTS", g.slots); k.define("NXCD", opt.deviceInfo.xcdCount);
+    if (g.tapm) k.define("TAPM", 1);
+    auto actName = [](int a) { return a == 1 ? "_relu" : a == 2 ? "_lrelu" : ""; };
+    const std::string entry = "convpair_c" + std::to_string(CA) + (up ? "u" : "") + (padA ? "e" : "") + (CB ? "p" + std::to_string(CB) + (padB ? "e" : "") : "") + "_k" +
+                              std::to_string(first.K) + actName(act1) + "_k" + std::to_string(second.K) + actName(act2) + (pool ? "_pool" : "") + (crop ? "_crop" : "") + "_" + cfg.name;
+    k.define("KERNEL_NAME", entry);
+    auto d = impl.registerDispatch(k, entry, Sym::Const(opt.deviceInfo.xcdCount * g.slots), Sym::Const(1), Sym::Const(1), cfg.waves * 64);
+    d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
+    if (CB) d.addBinding(dnx::Access::ReadOnly, m.inputs[1]);
+    d.addBinding(dnx::Access::WriteOnly, m.output);
+    const Op firstCopy = first, secondCopy = second; // the lazy packers outlive the model reference
+    auto biasOf = [](const Op &conv) {
+      std::vector<uint8_t> b(32 * 2, 0);
+      std::memcpy(b.data(), conv.bias.data(), conv.bias.size() * 2);
+      return b;
+    };
+    d.addParamBinding(impl.createParameter(static_cast<size_t>(9 * 32) * g.CPAD * 2, dnx::ScalarType::F16, [firstCopy, cpad = g.CPAD]() { return packPairWeights(firstCopy, cpad); }));
+    if (first.hasBias) d.addParamBinding(impl.createParameter(32 * 2, dnx::ScalarType::F16, [firstCopy, biasOf]() { return biasOf(firstCopy); }));
+    if (g.tapm) d.addParamBinding(impl.createParameter(static_cast<size_t>(3 * 32) * 32 * 2, dnx::ScalarType::F16, [secondCopy]() { return packPairWeightsTapM(secondCopy); }));
+    else d.addParamBinding(impl.createParameter(static_cast<size_t>(9 * 32) * 32 * 2, dnx::ScalarType::F16, [secondCopy]() { return packPairWeights(secondCopy, 32); }));
+    if (second.hasBias) d.addParamBinding(impl.createParameter(32 * 2, dnx::ScalarType::F16, [secondCopy, biasOf]() { return biasOf(secondCopy); }));
+    d.addPushConstant(convIn.width, dnx::ScalarType::U32);
+    d.addPushConstant(convIn.height, dnx::ScalarType::U32);
+    if (padA || padB) {
+      const Op *pad = nullptr;
+      for (int o : m.ops) if (model.ops()[o].kind == OpKind::Pad) pad = &model.ops()[o];
+      if (!pad) fail(Status::Internal, "conv pair match lacks its pad");
+      const TensorNode &src = model.tensors()[pad->inputs[0]];
+      d.addPushConstant(src.width); d.addPushConstant(src.height); d.addPushConstant(pad->left); d.addPushConstant(pad->top);
+    }
+    if (crop) {
+      const Op *sl = nullptr;
+      for (int o : m.ops) if (model.ops()[o].kind == OpKind::Slice) sl = &model.ops()[o];
+      if (!sl) fail(Status::Internal, "conv pair match lacks its slice");
+      const TensorNode &o = model.tensors()[m.output];
+      d.addPushConstant(o.width); d.addPushConstant(o.height); d.addPushConstant(sl->left); d.addPushConstant(sl->top);
+    }
+    d.addTraversalFlag();
+
+    std::string nm = "conv3x3";
+    if (up) nm = "upsample+" + nm;
+    if (padA || padB) nm = "pad+" + nm;
+    if (m.pattern & PAT_CONCAT) nm = "concat+" + nm;
+    if (act1 == 1) nm += "+relu"; else if (act1 == 2) nm += "+leaky_relu";
+    nm += "+conv3x3";
+    if (act2 == 1) nm += "+relu"; else if (act2 == 2) nm += "+leaky_relu";
+    if (pool) nm += "+maxpool";
+    if (crop) nm += "+slice";
+    d.setName(nm);
+    d.setOperation(nm);
+    d.setConfig(cfg.name);
+    impl.edge().config = cfg.name;
+    Sym reads = bytesOf(sym, tA);
+    if (CB) reads = sym.add(reads, bytesOf(sym, model.tensors()[m.inputs[1]]));
+    reads = sym.add(reads, static_cast<int64_t>(first.K) * first.C * 9 * 2 + (first.hasBias ? first.K * 2 : 0) + static_cast<int64_t>(second.K) * second.C * 9 * 2 + (second.hasBias ? second.K * 2 : 0));
+    d.setMemoryReads(reads);
+    d.setMemoryWrites(bytesOf(sym, model.tensors()[m.output]));
+    d.setFlops(sym.mul(sym.mul(convIn.width, convIn.height), static_cast<int64_t>(2) * 9 * (static_cast<int64_t>(first.C) * first.K + static_cast<int64_t>(second.C) * second.K)));
   }
 
 private:
@@ -787,6 +1039,7 @@ public:
 std::vector<std::unique_ptr<IShader>> get_all_shaders(const hip::HipCompiler *c) {
   std::vector<std::unique_ptr<IShader>> s;
   s.push_back(std::make_unique<ConvMfmaShader>(c));
+  s.push_back(std::make_unique<ConvPairShader>(c));
   s.push_back(std::make_unique<BasicPoolShader>(c));
   s.push_back(std::make_unique<BasicUpsampleShader>(c));
   s.push_back(std::make_unique<CopyTransformShader>(c));

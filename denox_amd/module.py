@@ -84,6 +84,7 @@ def _options(features: Optional[dict], input_layout, output_layout, assume: Opti
     o.enable_alternating_traversal = int(f.get("alternating_traversal", True))
     o.enable_upsample_fold = int(f.get("upsample_fold", True))
     o.enable_implicit_concat = int(f.get("implicit_concat", True))
+    o.enable_conv_conv_fusion = int(f.get("conv_conv_fusion", True))
     o.input_format = int(input_layout)
     o.output_format = int(output_layout)
     keep = []

@@ -120,7 +120,7 @@ def synthetic_input(name: str, H: int, W: int, seed: int = 0, C: int | None = No
 # Compile features that keep every pool, upsample, concat, pad and slice a dispatch of its own (conv + activation stay
 # fused): the schedule in which the stand-alone bandwidth kernels can be timed on a whole network.
 UNFUSED_FEATURES = dict(conv_relu_fusion=True, concat_conv_fusion=False, upsample_fusion=False, pool_fusion=False, pad_fusion=False,
-                        slice_fusion=False, implicit_concat=False)
+                        slice_fusion=False, implicit_concat=False, conv_conv_fusion=False)
 
 # networks whose code objects __graft_entry__.build() compiles ahead of time
 CACHE_WARM_CONFIGS = [

@@ -162,6 +162,8 @@ typedef struct denox_hip_compile_options {
   int32_t populate_compile_kernels;
   uint32_t kernel_shard_index;
   uint32_t kernel_shard_count;
+  int32_t enable_conv_conv_fusion;   /* two consecutive 3x3 convolutions with at most 32 channels between them in one dispatch,
+                                        the tensor between them kept on chip (no counterpart in the reference) */
 } denox_hip_compile_options;
 void denox_hip_compile_options_default(denox_hip_compile_options *opt);
 /* db may be NULL (roofline estimates drive the selection).  The blob is

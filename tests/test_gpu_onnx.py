@@ -100,6 +100,7 @@ def test_oidn_unet_exported_by_torch_at_test_time():
         want = net(torch.from_numpy(x.astype(np.float32))).numpy()[0]
     m = dx.Model.from_onnx(buf.getvalue())
     blob = dx.compile_model(m, input_layout=dx.Layout.CHW, output_layout=dx.Layout.CHW)
-    assert dx.last_compile_report().count("conv3x3_mfma") == 16  # everything else folded into the 16 convs
+    rep = dx.last_compile_report()  # everything else folded into the 16 convs, the thin full-resolution pairs at either end joined
+    assert rep.count("conv3x3_mfma") == 12 and rep.count("conv3x3_pair") == 2
     got = dx.Module.load(blob).instance(H=70, W=100).infer(x[0])[0]
     assert_conv_close(got, want, "onnx oidn unet")

@@ -58,7 +58,9 @@ def _dispatch_names(blob, **ext):
 
 def test_tiny_unet_schedule_and_geometry():
     m, _ = networks.build("tiny_unet")
-    d = dx.describe(dx.compile_model(m), H=128, W=128)
+    # by default the last two convolutions (16 channels between them, read by nobody else) are one dispatch
+    assert _dispatch_names(dx.compile_model(m), H=128, W=128) == ["conv3x3+relu", "maxpool", "conv3x3+relu", "concat+upsample+conv3x3+relu+conv3x3"]
+    d = dx.describe(dx.compile_model(m, features=dict(conv_conv_fusion=False)), H=128, W=128)
     names = [x["name"] for x in d["dispatches"]]
     # e0 feeds both the pool and the skip, so the pool stays its own dispatch; upsample+concat fold into the conv
     assert names == ["conv3x3+relu", "maxpool", "conv3x3+relu", "concat+upsample+conv3x3+relu", "conv3x3"]
@@ -79,27 +81,36 @@ def test_tiny_unet_schedule_and_geometry():
 
 def test_fusion_switches_change_the_schedule():
     m, _ = networks.build("tiny_unet")
-    none = dict(conv_relu_fusion=False, concat_conv_fusion=False, upsample_fusion=False, pool_fusion=False)
+    none = dict(conv_relu_fusion=False, concat_conv_fusion=False, upsample_fusion=False, pool_fusion=False, conv_conv_fusion=False)
     names = _dispatch_names(dx.compile_model(m, features=dict(none, implicit_concat=False)), H=64, W=64)
     assert names == ["conv3x3", "relu", "maxpool", "conv3x3", "relu", "upsample", "concat-copy", "conv3x3", "relu", "conv3x3"]
     # the upsampled tensor is read by the concat only: the upsample stores straight into the concat's tensor; the skip
     # tensor is also read by the pool and keeps its copy
     names = _dispatch_names(dx.compile_model(m, features=none), H=64, W=64)
     assert names == ["conv3x3", "relu", "maxpool", "conv3x3", "relu", "upsample+concat", "concat-copy-src1", "conv3x3", "relu", "conv3x3"]
-    names = _dispatch_names(dx.compile_model(m, features=dict(upsample_fusion=False)), H=64, W=64)
+    names = _dispatch_names(dx.compile_model(m, features=dict(upsample_fusion=False, conv_conv_fusion=False)), H=64, W=64)
     assert names == ["conv3x3+relu", "maxpool", "conv3x3+relu", "upsample", "concat+conv3x3+relu", "conv3x3"]
+    names = _dispatch_names(dx.compile_model(m, features=dict(upsample_fusion=False)), H=64, W=64)
+    assert names == ["conv3x3+relu", "maxpool", "conv3x3+relu", "upsample", "concat+conv3x3+relu+conv3x3"]
 
 
 def test_oidn_unet_schedule_dispatch_geometry_covers_every_pixel():
     m, _ = networks.build("oidn_unet")
     for H, W in [(1080, 1920), (1077, 1917), (16, 16), (17, 33)]:
-        d = dx.describe(dx.compile_model(m, assume={"H": H, "W": W}), H=H, W=W)
         Hp, Wp = (H + 15) // 16 * 16, (W + 15) // 16 * 16
+        # the default schedule joins the two thin full-resolution layer pairs at either end of the network
+        f = dx.describe(dx.compile_model(m, assume={"H": H, "W": W}), H=H, W=W)
+        assert f["dispatches"][0]["name"] == "pad+conv3x3+relu+conv3x3+relu+maxpool" and f["dispatches"][-1]["name"] == "conv3x3+relu+conv3x3+slice"
+        assert len(f["dispatches"]) == 14 and all("conv3x3" in x["name"] for x in f["dispatches"])
+        assert sum(x["flops"] for x in f["dispatches"]) == pytest.approx(523.9e9 * (Hp * Wp) / (1088 * 1920), rel=2e-3)
+        for x in (f["dispatches"][0], f["dispatches"][-1]):  # persistent launches of one workgroup per compute unit
+            assert x["workgroup_count"] == [256, 1, 1] and x["push_constants"][:2] == [Wp, Hp]
+        d = dx.describe(dx.compile_model(m, assume={"H": H, "W": W}, features=dict(conv_conv_fusion=False)), H=H, W=W)
         # pad and crop fold into the first / last conv: IN extent, then source extent + offsets or crop window
         assert d["dispatches"][0]["name"] == "pad+conv3x3+relu" and d["dispatches"][-1]["name"] == "conv3x3+slice"
         assert d["dispatches"][0]["push_constants"] == [Wp, Hp, W, H, 0, 0, 0]
         assert d["dispatches"][-1]["push_constants"] == [Wp, Hp, W, H, 0, 0, 1]
-        u = dx.describe(dx.compile_model(m, assume={"H": H, "W": W}, features=dict(pad_fusion=False, slice_fusion=False)), H=H, W=W)
+        u = dx.describe(dx.compile_model(m, assume={"H": H, "W": W}, features=dict(pad_fusion=False, slice_fusion=False, conv_conv_fusion=False)), H=H, W=W)
         assert u["dispatches"][0]["name"] == "pad" and u["dispatches"][-1]["name"] == "slice"
         assert u["dispatches"][0]["push_constants"] == [Wp, Hp, 0, Wp - W, 0, Hp - H]
         assert u["dispatches"][-1]["push_constants"] == [0, 0, Wp, Hp, W, H]
@@ -341,20 +352,21 @@ def test_measured_latencies_drive_the_selection(tmp_path):
     # make the unfused upsample + concat + conv look cheaper than the fused kernel: the compiler must follow the table
     m, _ = networks.build("tiny_unet")
     db = dx.Db(str(tmp_path / "t.db"))
-    db.populate(m, assume={"H": 64, "W": 64}, conv_config="w4r2k16")
+    single = dict(conv_conv_fusion=False)  # this test is about one layer's alternatives
+    db.populate(m, assume={"H": 64, "W": 64}, conv_config="w4r2k16", features=single)
     rows = db.dump_csv().splitlines()[1:]
     for i, r in enumerate(rows):
         op = r.split('","')[0].strip('"')
         lat = 900_000.0 if ("concat+" in op or "upsample+" in op) else 1_000.0
         for _ in range(3):
             db.add_sample(i, lat)
-    names = _dispatch_names(dx.compile_model(m, assume={"H": 64, "W": 64}, conv_config="w4r2k16", db=db), H=64, W=64)
+    names = _dispatch_names(dx.compile_model(m, assume={"H": 64, "W": 64}, conv_config="w4r2k16", db=db, features=single), H=64, W=64)
     # (upsample, then one launch copying both sources) and (upsample stored in place, then a copy of the other source) cost the same here
     assert ("upsample" in names and "concat-copy" in names) or ("upsample+concat" in names and "concat-copy-src1" in names)
     assert not any(n.startswith("concat+") for n in names)
     assert "measured" in dx.last_compile_report()
     # without a table the roofline estimate prefers the fused kernel
-    names = _dispatch_names(dx.compile_model(m, assume={"H": 64, "W": 64}, conv_config="w4r2k16"), H=64, W=64)
+    names = _dispatch_names(dx.compile_model(m, assume={"H": 64, "W": 64}, conv_config="w4r2k16", features=single), H=64, W=64)
     assert "concat+upsample+conv3x3+relu" in names
 
 

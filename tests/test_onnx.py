@@ -87,8 +87,10 @@ def test_torch_exported_unet_imports_and_fuses():
     m = dx.Model.from_onnx(os.path.join(GOLD, "onnx_unet_dynamic.onnx"))
     assert [(t.name, t.channels) for t in m.inputs] == [("input", 3)] and [(t.name, t.channels) for t in m.outputs] == [("output", 3)]
     blob = dx.compile_model(m)
-    # pad folds into the first conv, upsample + concat into the third, the two crops (one Slice node per axis) into the last
-    assert dispatch_names(blob, H=33, W=47) == ["pad+conv3x3+relu", "maxpool", "conv3x3+relu", "concat+upsample+conv3x3+relu", "conv3x3+slice"]
+    # pad folds into the first conv, upsample + concat into the third, which runs in one dispatch with the last, and the two
+    # crops (one Slice node per axis) fold into that
+    assert dispatch_names(blob, H=33, W=47) == ["pad+conv3x3+relu", "maxpool", "conv3x3+relu", "concat+upsample+conv3x3+relu+conv3x3+slice"]
+    assert dispatch_names(dx.compile_model(m, features=dict(conv_conv_fusion=False)), H=33, W=47) == ["pad+conv3x3+relu", "maxpool", "conv3x3+relu", "concat+upsample+conv3x3+relu", "conv3x3+slice"]
     d = dx.describe(blob, H=33, W=47)
     t = {x["name"]: x for x in d["tensors"] if x.get("name")}
     assert (t["input"]["height"], t["input"]["width"], t["output"]["height"], t["output"]["width"]) == (33, 47, 33, 47)
