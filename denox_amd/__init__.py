@@ -15,4 +15,4 @@ computes on the CPU.
 from ._capi import DenoxHipError, LIB_PATH, build  # noqa: F401
 from .graph import Model, Sym, Tensor  # noqa: F401
 from .module import (Context, Db, Instance, Layout, Module, RuntimeModel, Shape, compile_model, describe, device_info, pinned_empty,  # noqa: F401
-                     last_compile_report, report)
+                     last_compile_report, report, conv_config_names)

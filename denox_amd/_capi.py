@@ -66,6 +66,7 @@ class Timing(Structure):
 # name -> (restype, argtypes); every function include/denox_hip.h declares
 SIGNATURES = {
     "denox_hip_last_error": (c_char_p, []),
+    "denox_hip_conv_config_names": (c_char_p, []),
     "denox_hip_version": (c_char_p, []),
     "denox_hip_set_kernel_paths": (c_int, [c_char_p, c_char_p]),
     "denox_hip_query_device_info": (c_int, [c_int, POINTER(DeviceInfo)]),

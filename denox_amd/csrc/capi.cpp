@@ -277,6 +277,14 @@ int denox_hip_compile(const denox_hip_builder *b, const denox_hip_compile_option
     *out_size = blob.size();
   });
 }
+const char *denox_hip_conv_config_names(void) {
+  static const std::string names = [] {
+    std::string s;
+    for (const auto &n : compiler::conv_config_names()) s += (s.empty() ? "" : ",") + n;
+    return s;
+  }();
+  return names.c_str();
+}
 const char *denox_hip_last_compile_report(void) { return g_lastReport.c_str(); }
 
 int denox_hip_min_cost_subgraph(uint32_t node_count, const uint8_t *is_input, uint32_t edge_count, const uint32_t *edge_input_offsets,

@@ -180,6 +180,8 @@ public:
 };
 
 std::vector<std::unique_ptr<IShader>> get_all_shaders(const hip::HipCompiler *compiler);
+// every name `CompileOptions::forceConvConfig` accepts: the convolution shaders' configuration tables
+std::vector<std::string> conv_config_names();
 
 // Build the super graph: every shader x match x configuration.
 SuperGraph implement(const Model &model, SymGraph &sym, const std::vector<std::unique_ptr<IShader>> &shaders, const CompileOptions &opt);

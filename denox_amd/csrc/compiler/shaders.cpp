@@ -71,7 +71,7 @@ const ConvConfig kConvConfigs[] = {
     {4, 4, 32, false, 0, 0, 16, 1, "m4r4k32x1"}, {8, 2, 32, false, 0, 0, 16, 2, "m8r2k32x2"}, {4, 2, 0, false, 0, 0, 16, 1, "m4r2kfx1"},  {4, 1, 0, false, 0, 0, 16, 2, "m4r1kfx2"},
     {4, 2, 32, false, 0, 32, 16, 2, "m4r2k32x2n"}, {4, 2, 0, false, 0, 32, 16, 1, "m4r2kfx1n"}, {4, 1, 0, false, 0, 48, 16, 1, "m4r1kfx1n"}, {4, 2, 32, false, 0, 48, 16, 1, "m4r2k32x1n"},
     {8, 2, 32, true, 0, 0, 16, 2, "q8r2k32x2"}, {8, 1, 32, true, 0, 0, 16, 2, "q8r1k32x2"}, {4, 2, 32, true, 0, 0, 16, 2, "q4r2k32x2"}, {8, 2, 32, true, 0, 0, 16, 1, "q8r2k32x1"},
-    {8, 2, 64, true, 0, 0, 16, 2, "q8r2k64x2"}, {4, 2, 32, true, 0, 48, 16, 1, "q4r2k32x1n"},
+    {4, 2, 32, true, 0, 48, 16, 1, "q4r2k32x1n"},
     // resident, two-phase schedule
     {16, 1, 16, true, 0, 0, 32, 1, "t16r1k16", true}, {16, 1, 32, true, 0, 0, 32, 1, "t16r1k32", true}, {16, 2, 16, true, 0, 0, 32, 1, "t16r2k16", true},
     {8, 2, 16, true, 0, 0, 32, 1, "t8r2k16", true},   {8, 2, 32, true, 0, 0, 32, 1, "t8r2k32", true},   {8, 4, 16, true, 0, 0, 32, 1, "t8r4k16", true},
@@ -1035,6 +1035,13 @@ public:
 };
 
 } // namespace
+
+std::vector<std::string> conv_config_names() {
+  std::vector<std::string> names;
+  for (const ConvConfig &c : kConvConfigs) names.push_back(c.name);
+  for (const PairConfig &c : kPairConfigs) names.push_back(c.name);
+  return names;
+}
 
 std::vector<std::unique_ptr<IShader>> get_all_shaders(const hip::HipCompiler *c) {
   std::vector<std::unique_ptr<IShader>> s;

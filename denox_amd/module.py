@@ -129,6 +129,11 @@ def describe(dnx: bytes, **extents: int) -> dict:
         _capi.lib().denox_hip_free(p)
 
 
+def conv_config_names() -> List[str]:
+    """Every name `conv_config=` accepts."""
+    return _capi.lib().denox_hip_conv_config_names().decode().split(",")
+
+
 def last_compile_report() -> str:
     return (_capi.lib().denox_hip_last_compile_report() or b"").decode()
 

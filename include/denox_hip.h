@@ -170,6 +170,10 @@ void denox_hip_compile_options_default(denox_hip_compile_options *opt);
  * malloc'ed; release it with denox_hip_free. */
 int denox_hip_compile(const denox_hip_builder *b, const denox_hip_compile_options *opt, const denox_hip_db *db,
                       void **out_dnx, size_t *out_size);
+/* The names `force_conv_config` accepts, separated by commas: the configuration tables of the convolution shaders, the
+ * hand-listed counterpart of the configuration spaces the reference's conv shaders enumerate
+ * (compiler/src/denox/compiler/implement/shaders/conv/DirectConvShaderCM.cpp:40-181).  A static string. */
+const char *denox_hip_conv_config_names(void);
 /* one line per selected dispatch of the most recent compile on this thread */
 const char *denox_hip_last_compile_report(void);
 void denox_hip_free(void *p);

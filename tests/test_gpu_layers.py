@@ -52,14 +52,23 @@ ALL_CONFIGS = ["w4r2k16", "w4r2k32", "w4r4k16", "w4r4k32", "w8r2k16", "w8r2k32",
                "w4r1kfn", "w4r1khn", "w4r2kfn", "w2r2kfn", "w4r1kfm", "w4r2khn"]
 # the 16x16x32 matrix shape: output channels in blocks of 16, tiles 16 or 32 pixels wide
 M16_CONFIGS = ["m4r2k32x2", "m4r2k64x2", "m4r1k32x2", "m4r2k32x1", "m4r4k32x1", "m8r2k32x2", "m4r2kfx1", "m4r1kfx2", "m4r2k32x2n",
-               "m4r2kfx1n", "m4r1kfx1n", "m4r2k32x1n", "q8r2k32x2", "q8r1k32x2", "q4r2k32x2", "q8r2k32x1", "q8r2k64x2", "q4r2k32x1n"]
+               "m4r2kfx1n", "m4r1kfx1n", "m4r2k32x1n", "q8r2k32x2", "q8r1k32x2", "q4r2k32x2", "q8r2k32x1", "q4r2k32x1n"]
 ALL_CONFIGS += M16_CONFIGS
 # two-phase schedule of the persistent kernel
 ALL_CONFIGS += ["t16r1k16", "t16r1k32", "t16r2k16", "t8r2k16", "t8r2k32", "t8r4k16", "t8r1k16", "u8r2k32x2", "u16r1k32x2"]
 
 
+# (tests/test_host.py checks on the CPU that every configuration of the library's table is in one of the lists of this file and
+# compiles for at least one of the layer shapes it is tested on here: a configuration must not be covered by skips alone)
+EVERY_CONFIG_SHAPES = [(80, 64, 45, 70), (73, 96, 130, 300), (16, 32, 300, 530)]
+FOLD_CONFIGS = ["f8r1", "f4r2", "f4r1"]
+FOLD_SHAPES = [(64, 9, 64, 36, 70, False), (16, 0, 32, 18, 34, False), (32, 24, 40, 62, 130, False), (8, 3, 3, 2, 2, False), (24, 9, 16, 40, 52, True),
+               (96, 32, 64, 34, 66, False)]
+STRIDED_ONLY_CONFIGS = ["m2r1k32x1n", "w2r2k16n", "w2r1k16n"]  # offered to strided layers only
+
+
 @pytest.mark.parametrize("config", ALL_CONFIGS)
-@pytest.mark.parametrize("C,K,H,W", [(80, 64, 45, 70), (73, 96, 130, 300), (16, 32, 300, 530)])
+@pytest.mark.parametrize("C,K,H,W", EVERY_CONFIG_SHAPES)
 def test_conv_every_configuration(oracle, config, C, K, H, W):
     rng = np.random.default_rng(7)
     x = rng.standard_normal((H, W, C)).astype(np.float16)
@@ -137,9 +146,8 @@ def test_odd_filter_extents(oracle, R, S, config):
     assert_conv_close(got2, env[o2.name], f"{R}x{S} bare {config}")
 
 
-@pytest.mark.parametrize("config", ["f8r1", "f4r2", "f4r1"])
-@pytest.mark.parametrize("CA,CB,K,H,W,padb", [(64, 9, 64, 36, 70, False), (16, 0, 32, 18, 34, False), (32, 24, 40, 62, 130, False),
-                                              (8, 3, 3, 2, 2, False), (24, 9, 16, 40, 52, True), (96, 32, 64, 34, 66, False)])
+@pytest.mark.parametrize("config", FOLD_CONFIGS)
+@pytest.mark.parametrize("CA,CB,K,H,W,padb", FOLD_SHAPES)
 def test_upsample_folded_into_weights(oracle, config, CA, CB, K, H, W, padb):
     """conv(concat(upsample(A), B)) with the upsample folded into 2x2-tap weights per output parity: the same tensor
     as the layer-by-layer evaluation, within the conv tolerance (the summed weights are rounded to binary16 once)."""
@@ -432,7 +440,7 @@ GEOMETRY_CASES = [  # (R, S, (pad_y, pad_x), (stride_y, stride_x))
 ]
 
 
-@pytest.mark.parametrize("config", [None, "w4r2k16", "s8r2k16", "m4r2k32x2", "p8r2k16", "t16r1k16", "p4r1k32", "q4r2k32x2", "m2r1k32x1n", "w2r2k16n"])
+@pytest.mark.parametrize("config", [None, "w4r2k16", "s8r2k16", "m4r2k32x2", "p8r2k16", "t16r1k16", "p4r1k32", "q4r2k32x2"] + STRIDED_ONLY_CONFIGS)
 @pytest.mark.parametrize("R,S,pad,stride", GEOMETRY_CASES)
 def test_conv_padding_and_stride(oracle, config, R, S, pad, stride):
     """Filter extents 1..7 (even ones too), any zero padding, strides up to 4: out[y, x] reads in[y*sy + r - py, x*sx + s - px]."""

@@ -133,6 +133,51 @@ def test_oidn_unet_schedule_dispatch_geometry_covers_every_pixel():
         assert (out["height"], out["width"], out["channels"]) == (H, W, 3)
 
 
+def test_every_conv_configuration_has_a_live_parity_case():
+    """The GPU parity tests skip a (configuration, layer shape) pair the compiler refuses (not enough LDS or registers for
+    that shape).  Checked here, without a GPU: the tests' lists name exactly the configurations of the library's tables, and
+    every configuration compiles for at least one shape of the test that covers it -- none is tested by skips alone."""
+    import test_gpu_conv_pair as tp
+    import test_gpu_layers as tl
+    from util import he_weights, small_bias
+    listed = set(tl.ALL_CONFIGS) | set(tl.FOLD_CONFIGS) | set(tl.STRIDED_ONLY_CONFIGS) | set(tp.PAIR_CONFIGS)
+    assert listed == set(dx.conv_config_names()), listed ^ set(dx.conv_config_names())
+    rng = np.random.default_rng(0)
+
+    def compiles(m, config):
+        try:
+            dx.compile_model(m, conv_config=config)
+        except dx.DenoxHipError as e:
+            assert e.status == 5
+            return False
+        return config in dx.last_compile_report()
+
+    def plain(C, K, stride=(1, 1), pad=(1, 1), R=3, S=3):
+        m = dx.Model()
+        m.output(m.relu(m.conv2d(m.input("input", "W", "H", C), he_weights(rng, K, C, R, S), small_bias(rng, K), stride=stride, padding=pad)))
+        return m
+
+    def folded(CA, CB, K):
+        m = dx.Model()
+        t = m.upsample(m.input("lo", m.sym("W") // 2, m.sym("H") // 2, CA))
+        if CB:
+            t = m.concat(t, m.input("x", "W", "H", CB))
+        m.output(m.activation(m.conv2d(t, he_weights(rng, K, CA + CB), small_bias(rng, K)), "leaky_relu", 0.25))
+        return m
+
+    dead = [c for c in tl.ALL_CONFIGS if not any(compiles(plain(C, K), c) for C, K, _, _ in tl.EVERY_CONFIG_SHAPES)]
+    dead += [c for c in tl.FOLD_CONFIGS if not any(compiles(folded(CA, CB, K), c) for CA, CB, K, _, _, _ in tl.FOLD_SHAPES)]
+    dead += [c for c in tl.STRIDED_ONLY_CONFIGS if not any(compiles(plain(24, 40, stride, pad, R, S), c) for R, S, pad, stride in tl.GEOMETRY_CASES)]
+    for c in tp.PAIR_CONFIGS:
+        hit = False
+        for C, K1, K2, tail in [(9, 32, 32, "relu"), (16, 32, 32, "relu"), (64, 32, 3, "none")]:
+            m, _ = tp.build(rng, C, K1, K2, tail)
+            hit |= compiles(m, c)
+        if not hit:
+            dead.append(c)
+    assert not dead, dead
+
+
 def test_missing_kernel_is_reported():
     m = dx.Model()
     x = m.input("input", "W", "H", 8)
