@@ -919,17 +919,26 @@ public:
       const unsigned vec = (a.channels % 8 == 0 && b.channels % 8 == 0) ? 8 : 1;
       auto k = m_compiler->read("copy_transform.hip");
       k.define("COUNT", a.channels); k.define("COUNT1", b.channels); k.define("VEC", vec);
-      const unsigned rpt = rowsPerThread(vec);
-      if (rpt > 1) k.define("RPT", rpt);
-      const std::string entry = "concat_c" + std::to_string(a.channels) + "_c" + std::to_string(b.channels) + "v" + std::to_string(vec);
+      // Pixels that are not whole 16-byte vectors are assembled in LDS from aligned loads (FLAT in copy_transform.hip): PQ
+      // consecutive pixels per workgroup, a multiple of 8, at most 64 and as many as keep both staged source ranges within
+      // 16 KB -- measured at 3840 x 2176: 73 + 73 channels 4.7 TB/s with 128 pixels (37 KB, four workgroups per CU), 5.6 with 64
+      // or 32, 5.3 with 16; 64 + 9 channels 5.6 / 5.8 / 5.2 / 3.5 TB/s with 128 / 64 / 32 / 16.
+      const unsigned total = a.channels + b.channels;
+      const unsigned pq = vec == 1 ? std::min(64u, 16u * 1024u / (total * 2u) / 8u * 8u) : 0;
+      const bool flat = pq >= 8;
+      const unsigned rpt = flat ? 1 : rowsPerThread(vec);
+      if (flat) { k.define("FLAT", 1); k.define("PQ", pq); }
+      else if (rpt > 1) k.define("RPT", rpt);
+      const std::string entry = "concat_c" + std::to_string(a.channels) + "_c" + std::to_string(b.channels) + "v" + std::to_string(vec) + (flat ? "f" : "");
       k.define("KERNEL_NAME", entry);
-      auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, chunksPerPixel(a.channels, vec) + chunksPerPixel(b.channels, vec)),
-                                     rowBlocks(sym, out.height, rpt), Sym::Const(1), WG_BANDWIDTH);
+      auto d = flat ? impl.registerDispatch(k, entry, sym.cdiv(sym.mul(out.width, out.height), pq), Sym::Const(1), Sym::Const(1), WG_BANDWIDTH)
+                    : impl.registerDispatch(k, entry, rowGrid(sym, out.width, chunksPerPixel(a.channels, vec) + chunksPerPixel(b.channels, vec)),
+                                            rowBlocks(sym, out.height, rpt), Sym::Const(1), WG_BANDWIDTH);
       d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
       d.addBinding(dnx::Access::ReadOnly, m.inputs[1]);
       d.addBinding(dnx::Access::WriteOnly, m.output);
       d.addPushConstant(out.width); d.addPushConstant(out.height);
-      d.setName("concat-copy"); d.setOperation("concat"); d.setConfig("vec" + std::to_string(vec));
+      d.setName("concat-copy"); d.setOperation("concat"); d.setConfig(std::string("vec") + std::to_string(vec) + (flat ? "/lds" : ""));
       d.setMemoryReads(bytesOf(sym, out)); d.setMemoryWrites(bytesOf(sym, out)); d.setFlops(Sym::Const(0));
       return;
     }

@@ -552,21 +552,23 @@ def test_concat_copy_of_two_sources(oracle, CA, CB):
     moves): bit-exact for aligned and odd channel counts, image heights that are not a multiple of the rows a thread covers,
     and for the same tensor on both sides."""
     rng = np.random.default_rng(CA * 100 + CB)
-    H, W = 21, 37
-    a = rng.standard_normal((H, W, CA)).astype(np.float16)
-    b = rng.standard_normal((H, W, CB)).astype(np.float16)
     m = dx.Model()
     ta, tb = m.input("a", "W", "H", CA), m.input("b", "W", "H", CB)
     cat, twice = m.concat(ta, tb), m.concat(tb, tb)
     m.output(cat)
     m.output(twice)
     mod = dx.Module.compile(m)
-    d = dx.describe(mod.dnx, H=H, W=W)
-    assert [x["name"] for x in d["dispatches"]] == ["concat-copy", "concat-copy"]
-    got_cat, got_twice = mod.instance(H=H, W=W).infer(a, b)
-    assert_bits_equal(got_cat, np.concatenate([a, b], axis=2), "concat of two inputs")
-    assert_bits_equal(got_twice, np.concatenate([b, b], axis=2), "concat of a tensor with itself")
-    assert_bits_equal(got_cat, oracle.concat(a, b), "concat against the oracle")
+    # (21 x 37: a few workgroups; 67 x 129 and 1 x 1: pixel counts that are not a multiple of what a workgroup takes,
+    # and a last 16-byte vector of the result that is only partly inside it)
+    for H, W in [(21, 37), (67, 129), (1, 1), (3, 5)]:
+        a = rng.standard_normal((H, W, CA)).astype(np.float16)
+        b = rng.standard_normal((H, W, CB)).astype(np.float16)
+        d = dx.describe(mod.dnx, H=H, W=W)
+        assert [x["name"] for x in d["dispatches"]] == ["concat-copy", "concat-copy"]
+        got_cat, got_twice = mod.instance(H=H, W=W).infer(a, b)
+        assert_bits_equal(got_cat, np.concatenate([a, b], axis=2), "concat of two inputs")
+        assert_bits_equal(got_twice, np.concatenate([b, b], axis=2), "concat of a tensor with itself")
+        assert_bits_equal(got_cat, oracle.concat(a, b), "concat against the oracle")
 
 
 @pytest.mark.parametrize("C,k", [(3, (2, 2)), (8, (2, 2)), (64, (2, 2)), (16, (3, 3)), (9, (2, 3)), (32, (4, 4))])
