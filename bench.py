@@ -137,6 +137,9 @@ def main() -> int:
     ap.add_argument("--conv-config", default=None)
     ap.add_argument("--db", default=None, help="timing table to select the schedule with (default: measure one now)")
     ap.add_argument("--no-tune", action="store_true", help="skip the timing table; select by roofline estimates")
+    ap.add_argument("--layout-preference", type=int, default=0,
+                    help="1: candidates that read or write a channel-block-major (CHWC8) internal tensor count half their cost, which "
+                         "forces that layout wherever it exists; 0 (default): the measured cost alone decides")
     ap.add_argument("--no-unfused-pass", action="store_true", help="skip the second, unfused schedule that times the stand-alone bandwidth kernels")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -168,7 +171,8 @@ def main() -> int:
         db.populate(model, assume={"H": H, "W": W}, conv_config=args.conv_config, input_layout=lay, output_layout=lay)
         db.bench(min_samples=10, max_relative_error=0.03, max_samples=50, save_progress=bool(args.db))
         tune_s = time.perf_counter() - t0
-    blob = dx.compile_model(model, assume={"H": H, "W": W}, conv_config=args.conv_config, db=db, input_layout=lay, output_layout=lay)
+    blob = dx.compile_model(model, assume={"H": H, "W": W}, conv_config=args.conv_config, db=db, input_layout=lay, output_layout=lay,
+                            features=dict(layout_preference=args.layout_preference))
     report = dx.last_compile_report()
     if args.per_dispatch:
         print(report, file=sys.stderr)
@@ -268,7 +272,9 @@ def main() -> int:
                 "sum_dispatch_ms": sum(a["latency_ms"] for a in acc)}
 
     # Which configuration each dispatch of the schedule runs, and the SHA-256 of its code object.
-    desc = dx.describe(blob, H=H, W=W)["dispatches"]
+    described = dx.describe(blob, H=H, W=W)
+    desc = described["dispatches"]
+    chwc8 = sum(1 for t in described["tensors"] if not t["param"] and t["format"] == 3)
     chosen = [f'{d["name"]}: {d["debug_info"].split(" | ")[0]}' for d in desc]
     dom_desc = desc[acc.index(dom)]
     roofline["kernel_entry_point"] = dom_desc["entry_point"]
@@ -323,7 +329,7 @@ def main() -> int:
                    "schedule": "min-cost over measured dispatch latencies" if db is not None else "min-cost over roofline estimates",
                    "tuning_seconds": round(tune_s, 2), "host_pointer_path_ms_per_frame": round(host_ms, 3), "host_pointer_pipelined_ms_per_frame": round(pipelined_ms, 3),
                    "single_replay_ms_median": round(singles[len(singles) // 2], 4), "single_replay_ms_p95": round(singles[int(len(singles) * 0.95)], 4),
-                   "schedule_configs": chosen},
+                   "layout_preference": args.layout_preference, "internal_tensors_in_chwc8": chwc8, "schedule_configs": chosen},
         "roofline": roofline,
     }
     if non_conv is not None:

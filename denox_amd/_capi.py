@@ -41,7 +41,7 @@ class CompileOptions(Structure):
                 ("output_format", c_int32), ("assumption_count", c_uint32), ("assumption_names", POINTER(c_char_p)),
                 ("assumption_values", POINTER(c_int64)), ("force_conv_config", c_char_p), ("device", c_int32),
                 ("populate_compile_kernels", c_int32), ("kernel_shard_index", c_uint32), ("kernel_shard_count", c_uint32),
-                ("enable_conv_conv_fusion", c_int32)]
+                ("enable_conv_conv_fusion", c_int32), ("enable_blocked_layout", c_int32), ("layout_preference", c_int32)]
 
 
 class DbBenchOptions(Structure):

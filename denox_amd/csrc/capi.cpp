@@ -84,6 +84,8 @@ compiler::CompileOptions toOptions(const denox_hip_compile_options *o) {
   opt.features.enableUpsampleFold = o->enable_upsample_fold != 0;
   opt.features.enableImplicitConcat = o->enable_implicit_concat != 0;
   opt.features.enableConvConvFusion = o->enable_conv_conv_fusion != 0;
+  opt.features.enableBlockedLayout = o->enable_blocked_layout != 0;
+  opt.layoutPreference = o->layout_preference;
   auto fmt = [](int f) {
     switch (f) {
     case 0: case DENOX_HIP_FORMAT_HWC: return dnx::TensorFormat::SSBO_HWC;
@@ -251,6 +253,8 @@ void denox_hip_compile_options_default(denox_hip_compile_options *o) {
   o->enable_upsample_fold = 1;
   o->enable_implicit_concat = 1;
   o->enable_conv_conv_fusion = 1;
+  o->enable_blocked_layout = 1;
+  o->layout_preference = 0;
   o->device = -1;
   o->populate_compile_kernels = 1;
   o->kernel_shard_index = 0;

@@ -52,6 +52,13 @@ static double estimate_dispatch_ms(const ComputeDispatch &d, const std::vector<i
   return (std::max(tMem, tMath) + 3e-6) * 1e3;
 }
 
+// CompileOptions::layoutPreference: a positive value halves the cost of every candidate that touches a CHWC8 tensor
+static double prefer(const SuperGraphEdge &e, const CompileOptions &opt, double cost) {
+  if (opt.layoutPreference <= 0) return cost;
+  const bool blocked = e.outputFormat != 0 || std::any_of(e.inputFormats.begin(), e.inputFormats.end(), [](int f) { return f != 0; });
+  return blocked ? 0.5 * cost : cost;
+}
+
 double edge_cost_ms(const SuperGraphEdge &e, const std::vector<int64_t> &dp, const Db *db, const CompileOptions &opt, bool *measured) {
   double total = 0.0;
   bool all = db != nullptr;
@@ -65,11 +72,11 @@ double edge_cost_ms(const SuperGraphEdge &e, const std::vector<int64_t> &dp, con
     }
   }
   if (measured) *measured = all;
-  if (all) return total;
+  if (all) return prefer(e, opt, total);
   total = 0.0;
   for (const auto &d : e.dispatches) total += estimate_dispatch_ms(d, dp, opt);
   // estimates cannot tell configurations apart; the shader's prior breaks ties
-  return total / std::max(1e-3f, e.speedup);
+  return prefer(e, opt, total / std::max(1e-3f, e.speedup));
 }
 
 namespace {
@@ -143,19 +150,21 @@ std::vector<size_t> minimum_cost_subgraph(const std::vector<bool> &isInput, cons
 }
 
 std::vector<size_t> select_schedule(const Model &model, const SuperGraph &g, const std::vector<double> &edgeCost) {
-  // node 2 t: tensor t in a buffer of its own; node 2 t + 1: tensor t as a channel range of its concat's output
-  // (SuperGraphEdge::outputVariant).  Tensor handles are topologically ordered, and so are these.
-  std::vector<bool> isInput(2 * model.tensors().size(), false);
-  for (size_t i = 0; i < model.tensors().size(); ++i) isInput[2 * i] = model.tensors()[i].isInput;
+  // Tensor t has four nodes, 4 t + 2 f + v: layout f (0 HWC, 1 CHWC8; SuperGraphEdge::outputFormat) and v = 1 for the tensor
+  // as a channel range of its concat's output (SuperGraphEdge::outputVariant, HWC only).  Tensor handles are topologically
+  // ordered, and so are these.  Model inputs and outputs are HWC tensors of their own.
+  std::vector<bool> isInput(4 * model.tensors().size(), false);
+  for (size_t i = 0; i < model.tensors().size(); ++i) isInput[4 * i] = model.tensors()[i].isInput;
   std::vector<HyperEdge> edges;
   for (const auto &e : g.edges) {
     HyperEdge h;
-    for (size_t i = 0; i < e.inputs.size(); ++i) h.inputs.push_back(2 * e.inputs[i] + (e.inputVariants.empty() ? 0 : e.inputVariants[i]));
-    h.output = 2 * e.output + e.outputVariant;
+    for (size_t i = 0; i < e.inputs.size(); ++i)
+      h.inputs.push_back(4 * e.inputs[i] + 2 * (e.inputFormats.empty() ? 0 : e.inputFormats[i]) + (e.inputVariants.empty() ? 0 : e.inputVariants[i]));
+    h.output = 4 * e.output + 2 * e.outputFormat + e.outputVariant;
     edges.push_back(std::move(h));
   }
   std::vector<int> outputs;
-  for (TensorHandle o : model.outputs()) outputs.push_back(2 * o);
+  for (TensorHandle o : model.outputs()) outputs.push_back(4 * o);
   double total = 0.0;
   std::vector<size_t> chosen = minimum_cost_subgraph(isInput, edges, edgeCost, outputs, &total);
   if (total >= kInfiniteCost) fail(Status::Unsupported, "no kernel implements part of this graph (a layer has no matching shader)");

@@ -115,6 +115,14 @@ SuperGraph implement(const Model &model, SymGraph &sym, const std::vector<std::u
     st.name = t.name;
     g.tensors.push_back(std::move(st));
   }
+  // the same tensors stored channel-block-major
+  const size_t N = model.tensors().size();
+  g.modelTensorCount = N;
+  for (size_t i = 0; i < N; ++i) {
+    SuperTensor st = g.tensors[i];
+    st.format = dnx::TensorFormat::SSBO_CHWC8;
+    g.tensors.push_back(std::move(st));
+  }
   for (const auto &shader : shaders) {
     for (const Match &m : shader->matchAll(model, opt)) {
       for (unsigned config : shader->acceptMatch(model, m, opt)) {
@@ -123,7 +131,27 @@ SuperGraph implement(const Model &model, SymGraph &sym, const std::vector<std::u
         impl.edge().speedup = shader->speedup(config);
         impl.edge().outputVariant = m.outputVariant;
         impl.edge().inputVariants = m.inputVariants;
+        impl.edge().outputFormat = m.outputFormat;
+        impl.edge().inputFormats = m.inputFormats;
         shader->implement(impl, model, m, config, sym, opt);
+        if (m.blocked()) {
+          // The shaders bind model tensors by handle; an input or output the match takes in CHWC8 is that tensor's second
+          // super-graph tensor.
+          auto blockedTensor = [&](uint32_t t) -> uint32_t {
+            if (t >= N) return t; // a parameter
+            if (static_cast<int>(t) == m.output && m.outputFormat) return t + static_cast<uint32_t>(N);
+            for (size_t i = 0; i < m.inputs.size(); ++i)
+              if (m.inputs[i] == static_cast<int>(t) && i < m.inputFormats.size() && m.inputFormats[i]) return t + static_cast<uint32_t>(N);
+            return t;
+          };
+          for (auto &d : impl.edge().dispatches)
+            for (auto &b : d.bindings) b.tensor.index = blockedTensor(b.tensor.index);
+          for (auto &mc : impl.edge().memoryConstrains) {
+            mc.src0.index = blockedTensor(mc.src0.index);
+            mc.src1.index = blockedTensor(mc.src1.index);
+            mc.dst.index = blockedTensor(mc.dst.index);
+          }
+        }
         impl.finish();
       }
     }

@@ -17,6 +17,7 @@
 #include "../hip/hip_compiler.hpp"
 #include "model.hpp"
 #include "options.hpp"
+#include <algorithm>
 #include <functional>
 #include <memory>
 #include <string>
@@ -99,13 +100,21 @@ struct SuperGraphEdge {
   // The two are different nodes of the hyper-graph the schedule is selected from.
   int outputVariant = 0;
   std::vector<int> inputVariants; // one per input, empty = all 0
+  // Activation layout of the output / of each input (empty = all 0): 0 pixel-major (HWC), 1 channel-block-major (CHWC8).
+  // As in the reference, where every tensor exists once per candidate layout and the edges are the cross product
+  // (compiler/src/denox/compiler/specialization/specialization.cpp:13-16,112-121,282-306), the two layouts of a tensor
+  // are different nodes of the hyper-graph; a dispatch that reads one layout and writes the other is the conversion.
+  int outputFormat = 0;
+  std::vector<int> inputFormats;
   std::string shader, config;
   float speedup = 1.0f;
 };
 
 struct SuperGraph {
-  std::vector<SuperTensor> tensors;   // [0, modelTensorCount) mirror the model's tensors, parameters follow
+  // [0, N) mirror the model's N tensors in HWC, [N, 2N) the same tensors in CHWC8 (a buffer of its own each), parameters follow
+  std::vector<SuperTensor> tensors;
   std::vector<SuperGraphEdge> edges;
+  size_t modelTensorCount = 0;
 };
 
 class OpImpl;
@@ -164,6 +173,9 @@ struct Match {
   int output = -1;           // tensor handle written
   int outputVariant = 0;     // as SuperGraphEdge::outputVariant
   std::vector<int> inputVariants;
+  int outputFormat = 0;      // as SuperGraphEdge::outputFormat
+  std::vector<int> inputFormats;
+  bool blocked() const { return outputFormat != 0 || std::any_of(inputFormats.begin(), inputFormats.end(), [](int f) { return f != 0; }); }
 };
 
 class IShader {

@@ -20,6 +20,7 @@ struct Features {
   bool enableUpsampleFold = true;     // candidates that fold a fused 2x upsample into the conv weights (2x2 taps per output parity)
   bool enableAlternatingTraversal = true; // consecutive conv dispatches walk their tiles in opposite directions
   bool enableImplicitConcat = true;   // memory-aliasing concat where layouts allow it
+  bool enableBlockedLayout = true;    // offer every internal tensor in CHWC8 beside HWC (reference: specialization.cpp:13-16)
   bool enableConvConvFusion = true;   // two consecutive 3x3 convolutions in one dispatch, the tensor between them kept in LDS
 };
 
@@ -38,6 +39,9 @@ struct CompileOptions {
   DeviceInfo deviceInfo;
   // restrict the conv configuration space to one named configuration ("" = all)
   std::string forceConvConfig;
+  // > 0: candidates that read or write a CHWC8 tensor count half their cost, so that the blocked layout is taken wherever
+  // it is offered (tests and measurements of that path); 0: cost alone decides
+  int layoutPreference = 0;
   bool verbose = false;
 };
 

@@ -85,6 +85,21 @@ const ConvConfig kConvConfigs[] = {
 };
 constexpr unsigned kNumConvConfigs = sizeof(kConvConfigs) / sizeof(kConvConfigs[0]);
 
+// Configurations that are also offered with channel-block-major (CHWC8) sources and / or result: one or two of each kernel
+// family and matrix shape, so that the layout alternative adds half as many candidates again instead of three times as many.
+bool offeredBlocked(const ConvConfig &cfg) {
+  for (const char *n : {"w4r2k16", "w8r2k32", "w4r1kfn", "p16r2k16", "s8r2k16", "t8r2k32", "t16r1k32", "m4r2k32x1", "m8r2k32x2", "m4r2kfx1", "q8r2k32x2", "s12r1k16"})
+    if (std::strcmp(n, cfg.name) == 0) return true;
+  return false;
+}
+
+// A tensor that can exist in the blocked layout: whole 8-channel groups, and not an interface tensor (those keep the layout
+// the caller declared; the conversion from and to it is a dispatch of its own).
+bool canBeBlocked(const Model &model, TensorHandle t) {
+  const TensorNode &n = model.tensors()[t];
+  return n.channels % 8 == 0 && !n.isInput && !n.isOutput;
+}
+
 enum ConvPatternBits : unsigned { PAT_CONCAT = 1, PAT_UPSAMPLE = 2, PAT_ACT = 4, PAT_POOL = 8, PAT_PADA = 16, PAT_PADB = 32, PAT_CROP = 64, PAT_ACT_FIRST = 128 };
 
 struct ConvGeometry {
@@ -353,6 +368,19 @@ public:
             v.outputVariant = 1;
             out.push_back(std::move(v));
           }
+          // the same dispatch with its sources and / or its result in the blocked layout
+          if (opt.features.enableBlockedLayout) {
+            const bool inOk = std::all_of(m.inputs.begin(), m.inputs.end(), [&](int t) { return canBeBlocked(model, t); });
+            const bool outOk = canBeBlocked(model, m.output);
+            for (int fin = 0; fin <= (inOk ? 1 : 0); ++fin)
+              for (int fout = 0; fout <= (outOk ? 1 : 0); ++fout) {
+                if (!fin && !fout) continue;
+                Match v = m;
+                v.inputFormats.assign(m.inputs.size(), fin);
+                v.outputFormat = fout;
+                out.push_back(std::move(v));
+              }
+          }
           out.push_back(std::move(m));
         }
     }
@@ -379,12 +407,17 @@ public:
       if (cfg.fold) {
         const unsigned others = PAT_POOL | PAT_CROP | PAT_PADA;
         FoldGeometry fg;
-        if ((m.pattern & PAT_UPSAMPLE) && !(m.pattern & others) && conv.R == 3 && conv.S == 3 && conv.padX == 1 && conv.padY == 1 && conv.strideX == 1 && conv.strideY == 1 &&
+        if (!m.blocked() && (m.pattern & PAT_UPSAMPLE) && !(m.pattern & others) && conv.R == 3 && conv.S == 3 && conv.padX == 1 && conv.padY == 1 && conv.strideX == 1 && conv.strideY == 1 &&
             opt.features.enableUpsampleFold && chooseFold(cfg, CA, CB, conv.K, opt.deviceInfo, fg))
           out.push_back(c);
         continue;
       }
       if (cfg.wideHalo && conv.strideX == 1 && conv.strideY == 1) continue;
+      if (m.blocked()) {
+        if (!offeredBlocked(cfg)) continue;
+        // block-major sources are read through the per-step buffer resource: every LDS step must lie in one source
+        if (!m.inputFormats.empty() && m.inputFormats[0] && CB && CA % stepChannels(cfg, cpad)) continue;
+      }
       if (cfg.ck > cpad && cfg.ck != kstep) continue; // a larger stage than the whole reduction adds nothing
       if (cfg.ck <= 1 && cpad <= 32) continue;     // "whole / half reduction" duplicates a fixed-size stage for narrow layers
       if ((m.pattern & PAT_POOL) && (cfg.rpw % 2)) continue;
@@ -396,7 +429,7 @@ public:
     }
     bool forcedFold = false; // a forced upsample-folding configuration leaves matches without an upsample to nobody: not an error
     for (unsigned c = 0; c < kNumConvConfigs; ++c) forcedFold |= kConvConfigs[c].fold && forced == kConvConfigs[c].name;
-    if (out.empty() && !forced.empty() && !(forcedFold && !(m.pattern & PAT_UPSAMPLE)))
+    if (out.empty() && !forced.empty() && !m.blocked() && !(forcedFold && !(m.pattern & PAT_UPSAMPLE)))
       fail(Status::Unsupported, "conv configuration '" + forced + "' is not valid for this layer");
     return out;
   }
@@ -450,6 +483,9 @@ public:
     if (!samePad) { k.define("PY", conv.padY); k.define("PX", conv.padX); }
     if (!unitStride) { k.define("SY", conv.strideY); k.define("SX", conv.strideX); }
     if (cfg.mf != 32) { k.define("MF", cfg.mf); k.define("XB", cfg.xb); }
+    const bool blockedIn = !m.inputFormats.empty() && m.inputFormats[0] != 0, blockedOut = m.outputFormat != 0;
+    if (blockedIn) k.define("LAYIN", 1);
+    if (blockedOut) k.define("LAYOUT_OUT", 1);
     const ConcatView view = m.outputVariant ? concatViewOf(model, m.output) : ConcatView{};
     if (m.outputVariant && !view.valid) fail(Status::Internal, "conv match writes into a concat that does not exist");
     const bool ovec = view.valid && view.pitch % 8 == 0 && view.channelOffset % 8 == 0;
@@ -457,7 +493,7 @@ public:
     std::string entry = "conv" + std::to_string(conv.R) + "x" + std::to_string(conv.S) + (samePad ? "" : "p" + std::to_string(conv.padY) + "x" + std::to_string(conv.padX)) +
                         (unitStride ? "" : "s" + std::to_string(conv.strideY) + "x" + std::to_string(conv.strideX)) + "_c" + std::to_string(CA) + (up ? "u" : "") + (padA ? "e" : "") + (CB ? "p" + std::to_string(CB) + (padB ? "e" : "") : "") + "_k" +
                         std::to_string(conv.K) + (act == 1 ? "_relu" : act == 2 ? "_lrelu" : "") + (pool ? "_pool" : "") + (crop ? "_crop" : "") +
-                        (view.valid ? "_into" + std::to_string(view.pitch) + (ovec ? "" : "e") : "") + "_" + cfg.name;
+                        (view.valid ? "_into" + std::to_string(view.pitch) + (ovec ? "" : "e") : "") + (blockedIn ? "_bi" : "") + (blockedOut ? "_bo" : "") + "_" + cfg.name;
     k.define("KERNEL_NAME", entry);
     const Sym W = convIn.width, H = convIn.height;
     const TensorNode &convOut = model.tensors()[conv.output]; // the convolution's own result, whatever is fused behind it
@@ -516,8 +552,9 @@ public:
     if (view.valid) nm += "+concat";
     d.setName(nm);
     d.setOperation(nm);
-    d.setConfig(std::string(cfg.name) + "/kt" + std::to_string(g.KT));
-    impl.edge().config = cfg.name;
+    const std::string layouts = m.blocked() ? std::string("/") + (blockedIn ? "chwc8" : "hwc") + ">" + (blockedOut ? "chwc8" : "hwc") : std::string();
+    d.setConfig(std::string(cfg.name) + "/kt" + std::to_string(g.KT) + layouts);
+    impl.edge().config = cfg.name + layouts;
     // bytes that cross HBM: sources at their stored resolution, weights, bias; the (pooled / cropped) output
     Sym reads = bytesOf(sym, tA);
     if (CB) reads = sym.add(reads, bytesOf(sym, model.tensors()[m.inputs[1]]));
@@ -797,6 +834,15 @@ public:
         v.outputVariant = 1;
         out.push_back(std::move(v));
       }
+      // the same operation on a tensor stored channel-block-major, plane by plane (pool, upsample, activation: what the
+      // reference's shaders take in CHWC8, BasicPoolShader.cpp:150-151; its pad and slice shaders have no such variant)
+      if ((m_kind == OpKind::Pool || m_kind == OpKind::Upsample || m_kind == OpKind::Activation) && opt.features.enableBlockedLayout &&
+          canBeBlocked(model, m.inputs[0]) && canBeBlocked(model, m.output)) {
+        Match v = m;
+        v.inputFormats = {1};
+        v.outputFormat = 1;
+        out.push_back(std::move(v));
+      }
       out.push_back(std::move(m));
     }
     return out;
@@ -804,7 +850,9 @@ public:
 
   // Where a single-source dispatch stores: vector width (16-byte stores need an aligned channel range), the kernel
   // definition and name suffix, and the output binding with the bytes it may touch.
-  struct Placement { ConcatView view; unsigned vec; std::string suffix; };
+  // planes: 0 for a pixel-major tensor, else the number of 8-channel planes of a block-major one -- the kernel is then
+  // compiled for 8 channels and launched once per plane (grid.z)
+  struct Placement { ConcatView view; unsigned vec; std::string suffix; unsigned planes = 0; };
   static Placement placementOf(const Model &model, const Match &m, unsigned channels) {
     Placement p;
     p.view = m.outputVariant ? concatViewOf(model, m.output) : ConcatView{};
@@ -812,11 +860,18 @@ public:
     const bool aligned = !p.view.valid || (p.view.pitch % 8 == 0 && p.view.channelOffset % 8 == 0);
     p.vec = channels % 8 == 0 && aligned ? 8 : 1;
     if (p.view.valid) p.suffix = "_into" + std::to_string(p.view.pitch);
+    if (m.outputFormat) {
+      p.planes = channels / 8;
+      p.suffix = "_planar";
+    }
     return p;
   }
   static void defineOutput(hip::HipCompilerInstance &k, const Placement &p) {
     if (p.view.valid) k.define("OPITCH", p.view.pitch);
+    if (p.planes) { k.define("PLANAR", 1); k.define("CH", 8); } // (overrides the channel count defined before)
   }
+  static unsigned kernelChannels(const Placement &p, unsigned channels) { return p.planes ? 8 : channels; }
+  static Sym gridZ(const Placement &p) { return Sym::Const(p.planes ? p.planes : 1); }
   static void bindOutput(ComputeDispatchBuilder &d, SymGraph &sym, const Model &model, const Match &m, const Placement &p) {
     if (!p.view.valid) { d.addBinding(dnx::Access::WriteOnly, m.output); return; }
     const TensorNode &o = model.tensors()[m.output];
@@ -851,11 +906,12 @@ public:
     defineOutput(k, place);
     const std::string entry = std::string(avg ? "pool_avg_c" : "pool_max_c") + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, chunksPerPixel(in.channels, vec)), out.height, Sym::Const(1), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, chunksPerPixel(kernelChannels(place, in.channels), vec)), out.height, gridZ(place), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     bindOutput(d, sym, model, m, place);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
-    d.setName(std::string(avg ? "avgpool" : "maxpool") + (place.view.valid ? "+concat" : "")); d.setOperation(avg ? "avgpool" : "maxpool"); d.setConfig("vec" + std::to_string(vec));
+    d.setName(std::string(avg ? "avgpool" : "maxpool") + (place.view.valid ? "+concat" : "")); d.setOperation(avg ? "avgpool" : "maxpool"); d.setConfig("vec" + std::to_string(vec) + (place.planes ? "/chwc8" : ""));
+    if (place.planes) impl.edge().config = "chwc8";
     d.setMemoryReads(bytesOf(sym, in)); d.setMemoryWrites(bytesOf(sym, out)); d.setFlops(Sym::Const(0));
   }
 };
@@ -874,11 +930,12 @@ public:
     defineOutput(k, place);
     const std::string entry = "upsample_c" + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, chunksPerPixel(in.channels, vec)), in.height, Sym::Const(1), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, chunksPerPixel(kernelChannels(place, in.channels), vec)), in.height, gridZ(place), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     bindOutput(d, sym, model, m, place);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
-    d.setName(std::string("upsample") + (place.view.valid ? "+concat" : "")); d.setOperation("upsample"); d.setConfig("vec" + std::to_string(vec));
+    d.setName(std::string("upsample") + (place.view.valid ? "+concat" : "")); d.setOperation("upsample"); d.setConfig("vec" + std::to_string(vec) + (place.planes ? "/chwc8" : ""));
+    if (place.planes) impl.edge().config = "chwc8";
     d.setMemoryReads(bytesOf(sym, in)); d.setMemoryWrites(bytesOf(sym, out)); d.setFlops(Sym::Const(0));
   }
 };
@@ -898,6 +955,16 @@ public:
     std::vector<Match> out;
     for (const Match &m : SingleOpShader::matchAll(model, opt)) {
       out.push_back(m);
+      // Block-major sources: the concat is its first source's planes followed by its second source's.  When each source
+      // is read by this concat only, the two are placed behind one another inside the result and no dispatch is needed
+      // (the reference's implicit concat: placement/placement.cpp:232-255, CopyTransformShader.cpp:198-237).
+      if (opt.features.enableImplicitConcat && opt.features.enableBlockedLayout && m.inputs[0] != m.inputs[1] && canBeBlocked(model, m.output) &&
+          canBeBlocked(model, m.inputs[0]) && canBeBlocked(model, m.inputs[1]) && singleUse(model, m.inputs[0]) && singleUse(model, m.inputs[1])) {
+        Match v = m;
+        v.inputFormats = {1, 1};
+        v.outputFormat = 1;
+        out.push_back(std::move(v));
+      }
       if (!opt.features.enableImplicitConcat) continue;
       const bool v0 = concatViewOf(model, m.inputs[0]).valid, v1 = concatViewOf(model, m.inputs[1]).valid;
       for (int a = 0; a <= (v0 ? 1 : 0); ++a)
@@ -912,6 +979,11 @@ public:
   }
   void implement(OpImpl &impl, const Model &model, const Match &m, unsigned, SymGraph &sym, const CompileOptions &) const override {
     const TensorNode &out = model.tensors()[m.output];
+    if (m.outputFormat) { // block-major: aliasing only, no dispatch
+      impl.createImplicitConcatConstrain(m.inputs[0], m.inputs[1], m.output);
+      impl.edge().config = "implicit/chwc8";
+      return;
+    }
     unsigned off = 0;
     impl.edge().config = m.inputVariants.empty() ? "copy" : std::string(m.inputVariants[0] ? "in-place" : "copy") + "/" + (m.inputVariants[1] ? "in-place" : "copy");
     if (m.inputVariants.empty()) { // both sources are copied: one launch that writes whole pixels
@@ -981,12 +1053,13 @@ public:
     defineOutput(k, place);
     const std::string entry = std::string(op.func == ActivationFunction::ReLU ? "relu_c" : "leaky_relu_c") + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, rowGrid(sym, in.width, chunksPerPixel(in.channels, vec)), in.height, Sym::Const(1), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, rowGrid(sym, in.width, chunksPerPixel(kernelChannels(place, in.channels), vec)), in.height, gridZ(place), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     bindOutput(d, sym, model, m, place);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
     const char *nm = op.func == ActivationFunction::ReLU ? "relu" : "leaky_relu";
-    d.setName(std::string(nm) + (place.view.valid ? "+concat" : "")); d.setOperation(nm); d.setConfig("vec" + std::to_string(vec));
+    d.setName(std::string(nm) + (place.view.valid ? "+concat" : "")); d.setOperation(nm); d.setConfig("vec" + std::to_string(vec) + (place.planes ? "/chwc8" : ""));
+    if (place.planes) impl.edge().config = "chwc8";
     d.setMemoryReads(bytesOf(sym, in)); d.setMemoryWrites(bytesOf(sym, in));
     d.setFlops(sym.mul(sym.mul(in.width, in.height), static_cast<int64_t>(in.channels))); // one FLOP per element, as the reference counts it
   }

@@ -5,6 +5,7 @@
 #include <cstdlib>
 #include <dirent.h>
 #include <dlfcn.h>
+#include <fcntl.h>
 #include <fstream>
 #include <hip/hiprtc.h>
 #include <sstream>
@@ -141,6 +142,7 @@ std::vector<uint8_t> HipCompilerInstance::compile() const {
       std::vector<uint8_t> code((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
       if (!code.empty()) {
         ++m_compiler->m_cacheHits;
+        utimensat(AT_FDCWD, cachePath.c_str(), nullptr, 0); // modification time = last use: entries no source produces any more age out
         return code;
       }
     }

@@ -21,6 +21,10 @@ __device__ DNX_INLINE _Float16 act1(_Float16 v) {
 extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
     const ushort_t *__restrict__ IN, ushort_t *__restrict__ OUT, PushConstants pc) {
   constexpr unsigned CV = DNX_CHUNKS(CH);
+#ifdef PLANAR
+  IN += (size_t)DNX_BID_Z * pc.W * pc.H * 8;
+  OUT += (size_t)DNX_BID_Z * pc.W * pc.H * 8;
+#endif
   const unsigned i = DNX_ROW_INDEX();
   if (i >= pc.W * CV) return;
   const unsigned w = i / CV, cv = i - w * CV;

@@ -14,6 +14,8 @@ typedef unsigned short ushort_t;
 typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 
+// PLANAR (pool, upsample, activation): the tensors are channel-block-major (CHWC8, [C/8][H][W][8]): every 8-channel plane is
+// an HWC image of 8 channels, so the kernel is compiled with CH = 8, VEC = 8 and grid.z = C / 8 selects the plane.
 #ifndef WG
 #define WG 256
 #endif

@@ -20,6 +20,10 @@
 //               first channel of the range.  OVEC 0: that range is not 16-byte aligned, store element by element
 //   WAVES, RPW  computing waves per workgroup, output rows per wave -> tile = (WAVES*RPW) x 32 pixels
 //   CK          input channels staged in LDS per step (multiple of 16)
+//   LAYIN       1: the sources are stored channel-block-major (CHWC8: [C/8][H][W][8], the reference's second activation layout,
+//               common/src/denox/memory/tensor/ActivationLayout.hpp:37-66) instead of pixel-major (HWC); needs CA % 8 == 0,
+//               CB % 8 == 0 and every LDS step inside one source
+//   LAYOUT_OUT  1: the result is stored CHWC8; needs KOUT % 8 == 0 and OPITCH == KOUT
 //
 // Mapping onto v_mfma_f32_32x32x16_f16: the weights are the M operand (32 output
 // channels per block, rows permuted so that each lane ends up with 16 consecutive
@@ -49,6 +53,12 @@ typedef unsigned short ushort_t;
 #endif
 #ifndef OVEC
 #define OVEC 1
+#endif
+#ifndef LAYIN
+#define LAYIN 0
+#endif
+#ifndef LAYOUT_OUT
+#define LAYOUT_OUT 0
 #endif
 
 // Matrix-core shape: MF = 32 -> v_mfma_f32_32x32x16_f16 (32 output channels x 32 pixels per block, 16 input
@@ -167,8 +177,9 @@ __device__ DNX_INLINE void src_offsets(int gy, int gx, const PushConstants &pc, 
   const int by = gy, bx = gx;
   const unsigned WB = W;
 #endif
-  pa = ((size_t)ay * WA + (size_t)ax) * CA;
-  pb = ((size_t)by * WB + (size_t)bx) * (CB > 0 ? CB : 1);
+  // element offset of the pixel's first channel; in the block-major layout a pixel of one 8-channel plane is 8 elements
+  pa = ((size_t)ay * WA + (size_t)ax) * (LAYIN ? 8 : CA);
+  pb = ((size_t)by * WB + (size_t)bx) * (LAYIN ? 8 : (CB > 0 ? CB : 1));
 }
 
 typedef uint4v __attribute__((aligned(2))) uint4v_u; // global memory is accessed in unaligned mode
@@ -273,12 +284,14 @@ template <> struct MaskType<true> { typedef unsigned long long type; };
 // resource with 32-bit byte offsets: one add per load, and a lane with nothing to load (halo pixel outside the image,
 // padding channel) passes an offset past the end and gets zeros from the hardware.
 #define SRC_UNIFORM (VEC_SRC && (CB == 0 || CA % CK == 0))
+static_assert(!LAYIN || (SRC_UNIFORM && CA % 8 == 0 && CB % 8 == 0), "block-major sources: whole 8-channel groups, every LDS step inside one source");
 #define NO_LOAD 0xFFFFF000u // past the end of every tensor this code accepts; stays past it when a channel offset is added
 static_assert(2 * CPAD + 16 < 4096, "channel offsets must not wrap the no-access offset");
 
 struct Sources {
   const _Float16 *A, *B;
   unsigned bytesA, bytesB;
+  unsigned planeA, planeB; // bytes of one 8-channel plane (block-major layout)
 };
 
 __device__ DNX_INLINE Sources make_sources(const _Float16 *A, const _Float16 *B, const PushConstants &pc) {
@@ -297,6 +310,8 @@ __device__ DNX_INLINE Sources make_sources(const _Float16 *A, const _Float16 *B,
 #endif
   s.bytesA = pixA * (unsigned)CA * 2u;
   s.bytesB = pixB * (unsigned)CB * 2u;
+  s.planeA = pixA * 16u;
+  s.planeB = pixB * 16u;
   return s;
 }
 
@@ -375,7 +390,14 @@ struct Halo {
     for (int it = 0; it < NV; ++it) {
       const int rel = c0 + m.v8[it] - cbase;
       const int chan = ((CA % 8 == 0 && CB % 8 == 0) || rel + 8 <= cs) ? rel : cs - 8;
-      unsigned off = (unsigned)(fromA ? s.pa[it] : s.pb[it]) + 2u * (unsigned)chan;
+      const unsigned pixoff = (unsigned)(fromA ? s.pa[it] : s.pb[it]);
+#if LAYIN
+      // 8-channel group chan / 8 lives in its own plane; a pixel outside the image must stay outside whatever is added
+      unsigned off = pixoff + (unsigned)(chan >> 3) * (fromA ? src.planeA : src.planeB);
+      off = pixoff == NO_LOAD ? NO_LOAD : off;
+#else
+      unsigned off = pixoff + 2u * (unsigned)chan;
+#endif
       off = (m.v8[it] < L && rel < cs) ? off : NO_LOAD;
       st.v[it] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, LOAD_AUX);
     }
@@ -497,8 +519,26 @@ __device__ DNX_INLINE OutBuf out_buffer(_Float16 *OUT, const PushConstants &pc) 
   return __builtin_amdgcn_make_buffer_rsrc(OUT, 0, (int)(pixels ? ((pixels - 1u) * (unsigned)OPITCH + (unsigned)KOUT) * 2u : 0u), 0x00020000);
 }
 
-// 16 consecutive channels starting at chb of the pixel with linear index `pix`
-__device__ DNX_INLINE void store16(OutBuf out, bool ok, unsigned pix, const half8 (&o)[2], int chb) {
+// bytes of one 8-channel plane of the result (block-major layout)
+__device__ DNX_INLINE unsigned out_plane_bytes(const PushConstants &pc) {
+#if POOL
+  return (CONV_OUT_W(pc) >> 1) * (CONV_OUT_H(pc) >> 1) * 16u;
+#elif CROP
+  return pc.OUT_W * pc.OUT_H * 16u;
+#else
+  return CONV_OUT_W(pc) * CONV_OUT_H(pc) * 16u;
+#endif
+}
+static_assert(!LAYOUT_OUT || (KOUT % 8 == 0 && OPITCH == KOUT), "block-major result: whole 8-channel groups, a tensor of its own");
+
+// 16 consecutive channels starting at chb of the pixel with linear index `pix`; plane: out_plane_bytes() (block-major results only)
+__device__ DNX_INLINE void store16(OutBuf out, bool ok, unsigned pix, const half8 (&o)[2], int chb, unsigned plane = 0) {
+#if LAYOUT_OUT
+  const unsigned offb = (unsigned)(chb >> 3) * plane + pix * 16u; // the two 8-channel groups go to consecutive planes
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, o[0]), out, (ok && chb < KOUT) ? offb : NO_STORE, 0, STORE_AUX);
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, o[1]), out, (ok && chb + 8 < KOUT) ? offb + plane : NO_STORE, 0, STORE_AUX);
+  return;
+#endif
   const unsigned off = (pix * (unsigned)OPITCH + (unsigned)chb) * 2u;
   if (KOUT % 16 == 0 && OPITCH % 8 == 0 && OVEC) {
     const unsigned o0 = (ok && chb < KOUT) ? off : NO_STORE;
@@ -581,6 +621,7 @@ __device__ DNX_INLINE void
 store_packed(const Packed &pk, OutBuf out, int y0, int x0, int kt, int wv, int lane, const PushConstants &pc, int part = 0, int nparts = 1,
              int ystep = 1, int xstep = 1) { // (steps of 2: a kernel that computes every other row / column of the output)
   const unsigned W = CONV_OUT_W(pc), H = CONV_OUT_H(pc);
+  const unsigned plane = LAYOUT_OUT ? out_plane_bytes(pc) : 0u;
   const int l32 = lane & 31;
   const int x = x0 + l32 * xstep;
 #pragma unroll
@@ -593,15 +634,15 @@ store_packed(const Packed &pk, OutBuf out, int y0, int x0, int kt, int wv, int l
 #if POOL
       const unsigned WP = W >> 1, HP = H >> 1;
       const unsigned py = (unsigned)(y0 + wv * RPW + 2 * r) >> 1, px = (unsigned)x >> 1;
-      store16(out, (l32 & 1) == 0 && py < HP && px < WP, py * WP + px, pk.o[kb][r], chb);
+      store16(out, (l32 & 1) == 0 && py < HP && px < WP, py * WP + px, pk.o[kb][r], chb, plane);
 #else
       const int y = y0 + (wv * RPW + r) * ystep;
 #if CROP
       const int oy = y - (int)pc.CROP_T, ox = x - (int)pc.CROP_L;
       store16(out, y < (int)H && x < (int)W && oy >= 0 && oy < (int)pc.OUT_H && ox >= 0 && ox < (int)pc.OUT_W,
-              (unsigned)oy * pc.OUT_W + (unsigned)ox, pk.o[kb][r], chb);
+              (unsigned)oy * pc.OUT_W + (unsigned)ox, pk.o[kb][r], chb, plane);
 #else
-      store16(out, y < (int)H && x < (int)W, (unsigned)y * W + (unsigned)x, pk.o[kb][r], chb);
+      store16(out, y < (int)H && x < (int)W, (unsigned)y * W + (unsigned)x, pk.o[kb][r], chb, plane);
 #endif
 #endif
     }
@@ -671,8 +712,12 @@ struct Acc {
 };
 
 // n = 8 or 4 consecutive channels starting at chb of the pixel with linear index `pix`
-__device__ DNX_INLINE void store_vec(OutBuf out, bool ok, unsigned pix, const _Float16 (&o)[8], int chb, int n) {
+__device__ DNX_INLINE void store_vec(OutBuf out, bool ok, unsigned pix, const _Float16 (&o)[8], int chb, int n, unsigned plane = 0) {
+#if LAYOUT_OUT
+  const unsigned off = (unsigned)(chb >> 3) * plane + pix * 16u + (unsigned)(chb & 7) * 2u; // n = 8: a whole group; n = 4: half of one
+#else
   const unsigned off = (pix * (unsigned)OPITCH + (unsigned)chb) * 2u;
+#endif
   if (KOUT % 8 == 0 && OPITCH % 8 == 0 && OVEC && n == 8) {
     half8 h;
 #pragma unroll
@@ -732,6 +777,7 @@ __device__ DNX_INLINE void pack_tile(const Acc &acc, Packed &pk) {
 __device__ DNX_INLINE void
 store_packed(const Packed &pk, OutBuf out, int y0, int x0, int kt, int wv, int lane, const PushConstants &pc, int part = 0, int nparts = 1) {
   const unsigned W = CONV_OUT_W(pc), H = CONV_OUT_H(pc);
+  const unsigned plane = LAYOUT_OUT ? out_plane_bytes(pc) : 0u;
   const int l16 = lane & 15;
   const int g = lane >> 4;
 #pragma unroll
@@ -749,15 +795,15 @@ store_packed(const Packed &pk, OutBuf out, int y0, int x0, int kt, int wv, int l
 #if POOL
         const unsigned WP = W >> 1, HP = H >> 1;
         const unsigned py = (unsigned)(y0 + wv * RPW + 2 * r) >> 1, px = (unsigned)x >> 1;
-        store_vec(out, (l16 & 1) == 0 && py < HP && px < WP, py * WP + px, pk.o[kp][xb][r], chb, n);
+        store_vec(out, (l16 & 1) == 0 && py < HP && px < WP, py * WP + px, pk.o[kp][xb][r], chb, n, plane);
 #else
         const int y = y0 + wv * RPW + r;
 #if CROP
         const int oy = y - (int)pc.CROP_T, ox = x - (int)pc.CROP_L;
         store_vec(out, y < (int)H && x < (int)W && oy >= 0 && oy < (int)pc.OUT_H && ox >= 0 && ox < (int)pc.OUT_W,
-                  (unsigned)oy * pc.OUT_W + (unsigned)ox, pk.o[kp][xb][r], chb, n);
+                  (unsigned)oy * pc.OUT_W + (unsigned)ox, pk.o[kp][xb][r], chb, n, plane);
 #else
-        store_vec(out, y < (int)H && x < (int)W, (unsigned)y * W + (unsigned)x, pk.o[kp][xb][r], chb, n);
+        store_vec(out, y < (int)H && x < (int)W, (unsigned)y * W + (unsigned)x, pk.o[kp][xb][r], chb, n, plane);
 #endif
 #endif
       }

@@ -25,6 +25,10 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
     const ushort_t *__restrict__ IN, ushort_t *__restrict__ OUT, PushConstants pc) {
   constexpr unsigned CV = DNX_CHUNKS(CH);
   const unsigned W2 = pc.W / KX;
+#ifdef PLANAR
+  IN += (size_t)DNX_BID_Z * pc.W * pc.H * 8;
+  OUT += (size_t)DNX_BID_Z * W2 * (pc.H / KY) * 8;
+#endif
   const unsigned oh = DNX_BID_Y;
   const unsigned i = DNX_ROW_INDEX();
   if (i >= W2 * CV) return;

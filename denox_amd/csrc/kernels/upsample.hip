@@ -14,6 +14,10 @@ struct PushConstants { unsigned int W, H; }; // input extent
 extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
     const ushort_t *__restrict__ IN, ushort_t *__restrict__ OUT, PushConstants pc) {
   constexpr unsigned CV = DNX_CHUNKS(CH);
+#ifdef PLANAR
+  IN += (size_t)DNX_BID_Z * pc.W * pc.H * 8;
+  OUT += (size_t)DNX_BID_Z * pc.W * pc.H * (SCALE * SCALE * 8);
+#endif
   const unsigned h = DNX_BID_Y;
   const unsigned i = DNX_ROW_INDEX();
   if (i >= pc.W * SCALE * CV) return;

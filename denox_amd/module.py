@@ -85,6 +85,8 @@ def _options(features: Optional[dict], input_layout, output_layout, assume: Opti
     o.enable_upsample_fold = int(f.get("upsample_fold", True))
     o.enable_implicit_concat = int(f.get("implicit_concat", True))
     o.enable_conv_conv_fusion = int(f.get("conv_conv_fusion", True))
+    o.enable_blocked_layout = int(f.get("blocked_layout", True))
+    o.layout_preference = int(f.get("layout_preference", 0))
     o.input_format = int(input_layout)
     o.output_format = int(output_layout)
     keep = []

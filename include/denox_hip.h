@@ -164,6 +164,10 @@ typedef struct denox_hip_compile_options {
   uint32_t kernel_shard_count;
   int32_t enable_conv_conv_fusion;   /* two consecutive 3x3 convolutions with at most 32 channels between them in one dispatch,
                                         the tensor between them kept on chip (no counterpart in the reference) */
+  int32_t enable_blocked_layout;     /* offer every internal tensor in CHWC8 beside HWC, as two nodes of the graph the schedule is
+                                        selected from (compiler/src/denox/compiler/specialization/specialization.cpp:13-16,282-306) */
+  int32_t layout_preference;         /* > 0: candidates that touch a CHWC8 tensor count half their cost (to exercise or measure
+                                        that path); 0: cost alone decides */
 } denox_hip_compile_options;
 void denox_hip_compile_options_default(denox_hip_compile_options *opt);
 /* db may be NULL (roofline estimates drive the selection).  The blob is
