@@ -140,6 +140,7 @@ def main() -> int:
     ap.add_argument("--layout-preference", type=int, default=0,
                     help="1: candidates that read or write a channel-block-major (CHWC8) internal tensor count half their cost, which "
                          "forces that layout wherever it exists; 0 (default): the measured cost alone decides")
+    ap.add_argument("--no-blocked-layout", action="store_true", help="internal tensors pixel-major (HWC) only: no CHWC8 candidates")
     ap.add_argument("--no-unfused-pass", action="store_true", help="skip the second, unfused schedule that times the stand-alone bandwidth kernels")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -162,17 +163,18 @@ def main() -> int:
     # The reference workflow: populate the table with every candidate dispatch, time them on
     # this GPU, then compile against the measured latencies (README.md:112-199 of the reference:
     # `denox populate`, `denox bench`, `denox compile --db`).
+    features = dict(layout_preference=args.layout_preference, blocked_layout=not args.no_blocked_layout)
     db = None
     tune_s = 0.0
     if not args.no_tune:
         import tempfile
         t0 = time.perf_counter()
         db = dx.Db(args.db or os.path.join(tempfile.mkdtemp(prefix="denox_hip_"), "gpu.db"))
-        db.populate(model, assume={"H": H, "W": W}, conv_config=args.conv_config, input_layout=lay, output_layout=lay)
+        db.populate(model, assume={"H": H, "W": W}, conv_config=args.conv_config, input_layout=lay, output_layout=lay, features=features)
         db.bench(min_samples=10, max_relative_error=0.03, max_samples=50, save_progress=bool(args.db))
         tune_s = time.perf_counter() - t0
     blob = dx.compile_model(model, assume={"H": H, "W": W}, conv_config=args.conv_config, db=db, input_layout=lay, output_layout=lay,
-                            features=dict(layout_preference=args.layout_preference))
+                            features=features)
     report = dx.last_compile_report()
     if args.per_dispatch:
         print(report, file=sys.stderr)

@@ -665,6 +665,19 @@ public:
           m.ops.insert(m.ops.end(), e.ops.begin(), e.ops.end());
           m.inputs = p.inputs;
           m.output = e.output;
+          // the same dispatch with its sources and / or its result in the blocked layout
+          if (opt.features.enableBlockedLayout) {
+            const bool inOk = std::all_of(m.inputs.begin(), m.inputs.end(), [&](int t) { return canBeBlocked(model, t); });
+            const bool outOk = canBeBlocked(model, m.output);
+            for (int fin = 0; fin <= (inOk ? 1 : 0); ++fin)
+              for (int fout = 0; fout <= (outOk ? 1 : 0); ++fout) {
+                if (!fin && !fout) continue;
+                Match v = m;
+                v.inputFormats.assign(m.inputs.size(), fin);
+                v.outputFormat = fout;
+                out.push_back(std::move(v));
+              }
+          }
           out.push_back(std::move(m));
         }
     }
@@ -691,7 +704,10 @@ public:
       if ((m.pattern & PAT_POOL) && (cfg.rpw % 2)) continue;
       if (cfg.waves * 64 > opt.deviceInfo.maxComputeWorkGroupInvocations) continue;
       PairGeometry g;
-      if (choosePair(cfg, CA, CB, first->K, second->K, (m.pattern & PAT_POOL) != 0, opt.deviceInfo, g)) out.push_back(c);
+      if (!choosePair(cfg, CA, CB, first->K, second->K, (m.pattern & PAT_POOL) != 0, opt.deviceInfo, g)) continue;
+      // block-major sources are read through the per-step buffer resource: every LDS step must lie in one source
+      if (!m.inputFormats.empty() && m.inputFormats[0] && CB && CA % g.ck) continue;
+      out.push_back(c);
     }
     return out;
   }
@@ -740,9 +756,12 @@ public:
     k.define("WAVES", cfg.waves); k.define("RPW", cfg.rpw); k.define("CK", g.ck);
     k.define("SLOTS", g.slots); k.define("NXCD", opt.deviceInfo.xcdCount);
     if (g.tapm) k.define("TAPM", 1);
+    const bool blockedIn = !m.inputFormats.empty() && m.inputFormats[0] != 0, blockedOut = m.outputFormat != 0;
+    if (blockedIn) k.define("LAYIN", 1);
+    if (blockedOut) k.define("LAYOUT_OUT", 1);
     auto actName = [](int a) { return a == 1 ? "_relu" : a == 2 ? "_lrelu" : ""; };
     const std::string entry = "convpair_c" + std::to_string(CA) + (up ? "u" : "") + (padA ? "e" : "") + (CB ? "p" + std::to_string(CB) + (padB ? "e" : "") : "") + "_k" +
-                              std::to_string(first.K) + actName(act1) + "_k" + std::to_string(second.K) + actName(act2) + (pool ? "_pool" : "") + (crop ? "_crop" : "") + "_" + cfg.name;
+                              std::to_string(first.K) + actName(act1) + "_k" + std::to_string(second.K) + actName(act2) + (pool ? "_pool" : "") + (crop ? "_crop" : "") + (blockedIn ? "_bi" : "") + (blockedOut ? "_bo" : "") + "_" + cfg.name;
     k.define("KERNEL_NAME", entry);
     auto d = impl.registerDispatch(k, entry, Sym::Const(opt.deviceInfo.xcdCount * g.slots), Sym::Const(1), Sym::Const(1), cfg.waves * 64);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
@@ -788,8 +807,9 @@ public:
     if (crop) nm += "+slice";
     d.setName(nm);
     d.setOperation(nm);
-    d.setConfig(cfg.name);
-    impl.edge().config = cfg.name;
+    const std::string layouts = m.blocked() ? std::string("/") + (blockedIn ? "chwc8" : "hwc") + ">" + (blockedOut ? "chwc8" : "hwc") : std::string();
+    d.setConfig(cfg.name + layouts);
+    impl.edge().config = cfg.name + layouts;
     Sym reads = bytesOf(sym, tA);
     if (CB) reads = sym.add(reads, bytesOf(sym, model.tensors()[m.inputs[1]]));
     reads = sym.add(reads, static_cast<int64_t>(first.K) * first.C * 9 * 2 + (first.hasBias ? first.K * 2 : 0) + static_cast<int64_t>(second.K) * second.C * 9 * 2 + (second.hasBias ? second.K * 2 : 0));

@@ -264,6 +264,7 @@ __device__ DNX_INLINE void mma_first(const _Float16 *sIn, const _Float16 *sW, in
 __device__ DNX_INLINE void
 store_pair(const Packed &pk, OutBuf out, int ob, int xs, int ylo, int yhi, int wv, int lane, const PushConstants &pc) {
   const unsigned W = CONV_OUT_W(pc), H = CONV_OUT_H(pc);
+  const unsigned plane = LAYOUT_OUT ? out_plane_bytes(pc) : 0u;
   const int l32 = lane & 31;
   const int x = xs + l32;
   const int chb = (lane >> 5) * 16;
@@ -274,15 +275,15 @@ store_pair(const Packed &pk, OutBuf out, int ob, int xs, int ylo, int yhi, int w
     const unsigned WP = W >> 1, HP = H >> 1;
     const unsigned py = (unsigned)(y < 0 ? 0 : y) >> 1, px = (unsigned)x >> 1;
     const bool ok = (l32 & 1) == 0 && l32 < SWO && y >= ylo && y < yhi && py < HP && px < WP;
-    store16(out, ok, py * WP + px, pk.o[0][r], chb);
+    store16(out, ok, py * WP + px, pk.o[0][r], chb, plane);
 #else
     const int y = ob + wv * RPW + r;
     const bool mine = l32 < SWO && (!TAPM || lane < 32) && y >= ylo && y < yhi && x < (int)W && y < (int)H;
 #if CROP
     const int oy = y - (int)pc.CROP_T, ox = x - (int)pc.CROP_L;
-    store16(out, mine && oy >= 0 && oy < (int)pc.OUT_H && ox >= 0 && ox < (int)pc.OUT_W, (unsigned)oy * pc.OUT_W + (unsigned)ox, pk.o[0][r], chb);
+    store16(out, mine && oy >= 0 && oy < (int)pc.OUT_H && ox >= 0 && ox < (int)pc.OUT_W, (unsigned)oy * pc.OUT_W + (unsigned)ox, pk.o[0][r], chb, plane);
 #else
-    store16(out, mine, (unsigned)(y < 0 ? 0 : y) * W + (unsigned)x, pk.o[0][r], chb);
+    store16(out, mine, (unsigned)(y < 0 ? 0 : y) * W + (unsigned)x, pk.o[0][r], chb, plane);
 #endif
 #endif
   }

@@ -124,3 +124,36 @@ def test_full_size_oidn_unet_blocked(oracle):
     assert internal_formats(mod, H=H, W=W).count(3) >= 5
     got = mod.instance(H=H, W=W).infer(x)[0]
     check_crops(oracle, m, x, got, H, W, [(0, 0), (400, 800), (H - 272 + 8, W - 272)], "blocked 1080p")
+
+
+@pytest.mark.parametrize("config", ["x8r2k16", "x4r2k32", "x4r4k16", "x4r2k16"])
+@pytest.mark.parametrize("C,K1,K2,tail", [(64, 32, 32, "pool"), (40, 32, 16, "relu"), (48, 16, 24, "none")])
+def test_conv_pair_reads_and_writes_either_layout(oracle, config, C, K1, K2, tail):
+    """conv -> conv in one dispatch between two block-major tensors."""
+    rng = np.random.default_rng(C + K1 + K2)
+    m = dx.Model()
+    t = m.input("input", "W", "H", 16)
+    a = m.relu(m.conv2d(t, he_weights(rng, C, 16), small_bias(rng, C)))
+    b = m.relu(m.conv2d(a, he_weights(rng, K1, C), small_bias(rng, K1)))
+    c = m.conv2d(b, he_weights(rng, K2, K1), small_bias(rng, K2))
+    if tail in ("relu", "pool"):
+        c = m.relu(c)
+    if tail == "pool":
+        c = m.pool(c)
+    d = m.conv2d(c, he_weights(rng, 40, K2), small_bias(rng, 40))  # more than 32 output channels: never the second half of a pair
+    m.output(d)
+    try:
+        mod = dx.Module.compile(m, conv_config=config, features=BLOCKED)
+    except dx.DenoxHipError as e:
+        assert e.status == 5
+        pytest.skip(str(e))
+    for H, W in [(38, 70), (16, 32), (130, 44)]:
+        names = entries(mod, H=H, W=W)
+        pair = [n for n in names if n.startswith("convpair")]
+        if not (pair and "_bi_bo_" in pair[0]):
+            pytest.skip(f"{config}: no blocked pair for this layer: {names}")
+        x = rng.standard_normal((H, W, 16)).astype(np.float16)
+        fill_lds_with_nans()
+        got = mod.instance(H=H, W=W).infer(x)[0]
+        want = oracle.run_graph(m.to_ops({"H": H, "W": W}), {"input": x}, "fp32")[d.name]
+        assert_conv_close(got, want, f"blocked pair {config} {C}->{K1}->{K2} {H}x{W}")

@@ -415,6 +415,42 @@ def test_measured_latencies_drive_the_selection(tmp_path):
     assert "concat+upsample+conv3x3+relu" in names
 
 
+def test_internal_tensors_have_two_layouts_to_choose_from(tmp_path):
+    """Every internal tensor with a multiple of 8 channels exists pixel-major and channel-block-major (the reference's
+    specialization.cpp:13-16,282-306 clones tensors per format): the table lists candidates for both, the measured cost
+    decides between them, and what the schedule picks is recorded per tensor in the model file."""
+    m, _ = networks.build("oidn_unet")
+    assume = {"H": 64, "W": 64}
+    db = dx.Db(str(tmp_path / "t.db"))
+    db.populate(m, assume=assume)
+    rows = [r.split('","') for r in db.dump_csv().splitlines()[1:]]
+    configs = [r[2] for r in rows]
+    assert any(c.endswith("/hwc>chwc8") for c in configs) and any(c.endswith("/chwc8>hwc") for c in configs) and any(c.endswith("/chwc8>chwc8") for c in configs)
+    assert any(c == "vec8/chwc8" for c in configs) and any(c == "vec8" for c in configs)  # pool / upsample / activation in both layouts
+    assert sum("chwc8" in c for c in configs) < sum("chwc8" not in c for c in configs)    # only selected conv configurations exist blocked
+
+    def formats(blob):
+        return [t["format"] for t in dx.describe(blob, **assume)["tensors"] if not t["param"]]
+
+    # make every blocked candidate look ten times cheaper than the others, then the other way round
+    for cheap_blocked in (True, False):
+        d2 = dx.Db(str(tmp_path / f"t{int(cheap_blocked)}.db"))
+        d2.populate(m, assume=assume)
+        for i, c in enumerate(configs):
+            for _ in range(3):
+                d2.add_sample(i, 1_000.0 if ("chwc8" in c) == cheap_blocked else 10_000.0)
+        f = formats(dx.compile_model(m, assume=assume, db=d2))
+        assert (f.count(3) >= 8) if cheap_blocked else (3 not in f), (cheap_blocked, f)
+    # switched off: no blocked candidate at all, and the switch alone never changes the interface tensors
+    off = dx.Db(str(tmp_path / "off.db"))
+    off.populate(m, assume=assume, features=dict(blocked_layout=False))
+    assert not any("chwc8" in r for r in off.dump_csv().splitlines())
+    f = formats(dx.compile_model(m, assume=assume, features=dict(layout_preference=1)))
+    assert f[0] == 1 and f.count(3) >= 8
+    d = dx.describe(dx.compile_model(m, assume=assume, features=dict(layout_preference=1)), **assume)
+    assert d["tensors"][d["inputs"][0]]["format"] == 1 and d["tensors"][d["outputs"][0]]["format"] == 1
+
+
 # ----------------------------------------------------------------------------- arena planner (runtime/arena_plan.hpp)
 @pytest.fixture(scope="module")
 def arena_probe(tmp_path_factory):
