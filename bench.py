@@ -140,6 +140,7 @@ def main() -> int:
     ap.add_argument("--layout-preference", type=int, default=0,
                     help="1: candidates that read or write a channel-block-major (CHWC8) internal tensor count half their cost, which "
                          "forces that layout wherever it exists; 0 (default): the measured cost alone decides")
+    ap.add_argument("--no-upsample-fold", action="store_true", help="no kernels that fold a fused 2x upsample into the weights")
     ap.add_argument("--no-blocked-layout", action="store_true", help="internal tensors pixel-major (HWC) only: no CHWC8 candidates")
     ap.add_argument("--no-unfused-pass", action="store_true", help="skip the second, unfused schedule that times the stand-alone bandwidth kernels")
     args = ap.parse_args()
@@ -163,7 +164,7 @@ def main() -> int:
     # The reference workflow: populate the table with every candidate dispatch, time them on
     # this GPU, then compile against the measured latencies (README.md:112-199 of the reference:
     # `denox populate`, `denox bench`, `denox compile --db`).
-    features = dict(layout_preference=args.layout_preference, blocked_layout=not args.no_blocked_layout)
+    features = dict(layout_preference=args.layout_preference, blocked_layout=not args.no_blocked_layout, upsample_fold=not args.no_upsample_fold)
     db = None
     tune_s = 0.0
     if not args.no_tune:

@@ -46,8 +46,9 @@ std::string fmtFloat(float v) {
 // resident: weights stay in LDS (persistent launch); pw: extra staging-only waves; maxKT: cap on output channels
 // per workgroup (0 = none); mf: matrix shape 32 (32x32x16) or 16 (16x16x32); xb: 16-pixel blocks per row (mf 16).
 // pp: two-phase schedule of the persistent kernel (two wave groups alternate matrix work and everything else).
-// fold: the 2x upsample of source A folded into the weights (conv3x3_upfold.hip; rpw counts low-resolution rows).
-struct ConvConfig { unsigned waves, rpw, ck; bool resident; unsigned pw; unsigned maxKT; unsigned mf, xb; const char *name; bool pp = false; bool fold = false; bool wideHalo = false; };
+// fold: the 2x upsample of source A folded into the weights (conv3x3_upfold.hip, with pw: conv3x3_upfold_ws.hip; rpw counts low-resolution rows).
+// ntStore: the result is stored with the non-temporal cache policy.
+struct ConvConfig { unsigned waves, rpw, ck; bool resident; unsigned pw; unsigned maxKT; unsigned mf, xb; const char *name; bool pp = false; bool fold = false; bool wideHalo = false; bool ntStore = false; };
 const ConvConfig kConvConfigs[] = {
     // weights streamed per step
     {4, 2, 16, false, 0, 0, 32, 1, "w4r2k16"}, {4, 2, 32, false, 0, 0, 32, 1, "w4r2k32"}, {4, 4, 16, false, 0, 0, 32, 1, "w4r4k16"}, {4, 4, 32, false, 0, 0, 32, 1, "w4r4k32"},
@@ -78,6 +79,11 @@ const ConvConfig kConvConfigs[] = {
     {8, 1, 16, true, 0, 0, 32, 1, "t8r1k16", true},   {8, 2, 32, true, 0, 0, 16, 2, "u8r2k32x2", true}, {16, 1, 32, true, 0, 0, 16, 2, "u16r1k32x2", true},
     // upsample folded into the weights (layers whose source A is upsampled; one parity class of output pixels per workgroup)
     {8, 1, 16, true, 0, 0, 32, 1, "f8r1", false, true},  {4, 2, 16, true, 0, 0, 32, 1, "f4r2", false, true}, {4, 1, 16, true, 0, 0, 32, 1, "f4r1", false, true},
+    // staging-only waves and one row parity (both column parities) per workgroup (conv3x3_upfold_ws.hip; layers with a second source);
+    // ck: channels of the upsampled source per step, 0 = all
+    {4, 1, 0, true, 4, 0, 32, 1, "g4r1", false, true},   {4, 1, 32, true, 4, 0, 32, 1, "g4r1k32", false, true},
+    // ... and non-temporal stores of the result (whole lines written once, never read by this kernel)
+    {4, 1, 0, true, 4, 0, 32, 1, "g4r1n", false, true, false, true}, {4, 1, 32, true, 4, 0, 32, 1, "g4r1k32n", false, true, false, true},
     // the smallest tiles, offered to strided layers only: a stride multiplies the halo of a tile, and a 7 x 7 filter with
     // stride 4 fits the LDS next to its weights with nothing larger
     {2, 1, 16, false, 0, 32, 32, 1, "w2r1k16n", false, false, true}, {2, 1, 32, false, 0, 16, 16, 1, "m2r1k32x1n", false, false, true},
@@ -207,27 +213,42 @@ std::vector<uint8_t> packConvWeights(const Op &conv, const ConvGeometry &g, unsi
 // ---- upsample folded into the weights ------------------------------------------------------------------------
 struct FoldGeometry {
   unsigned CA, CB, CAP, CBP, K, KOUTP, KT, slots, bpitch;
+  unsigned cka; // channels of the upsampled source per step (staging-wave variant; CAP: one step)
   size_t ldsBytes;
 };
 
 bool chooseFold(const ConvConfig &cfg, unsigned CA, unsigned CB, unsigned K, const DeviceInfo &dev, FoldGeometry &g) {
   if (CA % 8 || (CB > 0 && CB < 8)) return false; // whole vectors of A; B's partial last vector is read ending at its last channel
   g.CA = CA; g.CB = CB; g.CAP = (CA + 15) / 16 * 16; g.CBP = CB ? (CB + 15) / 16 * 16 : 0; g.K = K; g.KOUTP = (K + 31) / 32 * 32;
-  const unsigned tlh = cfg.waves * cfg.rpw, threads = cfg.waves * 64;
-  const unsigned aPix = (tlh + 1) * 33, bPix = (2 * tlh + 1) * 65, blocks = g.KOUTP / 32;
-  const unsigned regBudget = std::min(256u, 512u / ((cfg.waves + 3) / 4));
+  const unsigned tlh = cfg.waves * cfg.rpw, threads = (cfg.pw ? cfg.pw : cfg.waves) * 64; // threads that move halos
+  const unsigned classes = cfg.pw ? 2 : 4; // kinds of workgroup: row parities, or row x column parities
+  const unsigned aPix = (tlh + 1) * (cfg.pw ? 34 : 33), bPix = (2 * tlh + 1) * (cfg.pw ? 66 : 65), blocks = g.KOUTP / 32;
+  const unsigned regBudget = std::min(256u, 512u / ((cfg.waves + cfg.pw + 3) / 4));
   const unsigned nva = (aPix * (g.CAP / 8) + threads - 1) / threads, nvb = CB ? (bPix * (g.CBP / 8) + threads - 1) / threads : 0;
+  g.cka = g.CAP;
+  if (cfg.pw) { // staging-wave variant: a second source of one matrix step of channels (its weights live in registers), whole
+                // 32- or 64-channel slices of the result; A in steps of cfg.ck channels
+    if (!CB || g.CBP != 16 || K % 32) return false;
+    if (cfg.ck) {
+      if (cfg.ck >= g.CAP || g.CAP % cfg.ck) return false;
+      g.cka = cfg.ck;
+    }
+  }
+  const unsigned na = g.CAP / g.cka;
   for (unsigned kb = blocks; kb >= 1; --kb) {
     if (blocks % kb) continue;
     if (cfg.maxKT && kb * 32 > cfg.maxKT) continue;
     const unsigned kt = kb * 32;
-    if (kb * cfg.rpw * 24 + (nva + nvb) * 4 + 64 > regBudget) continue; // accumulators, converted tile, halo registers
+    if (cfg.pw && kt > 64) continue;
+    // computing waves: accumulators, converted tile; waves that move halos: their registers and what locates them (3 per vector)
+    if (cfg.pw ? (std::max(2 * kb * cfg.rpw * 24 + 9 * kb * 4 + 64, nva * 7 + nvb * 7 + 24) > regBudget) : (kb * cfg.rpw * 24 + (nva + nvb) * 4 + 64 > regBudget)) continue;
     for (unsigned pitchPad : {8u, 0u}) { // the B halo gives up its bank-conflict padding where LDS is short
-      const size_t lds = (static_cast<size_t>(4 * kt) * (g.CAP + 8) + (CB ? static_cast<size_t>(9 * kt) * (g.CBP + 8) : 8) + static_cast<size_t>(aPix) * (g.CAP + 8) +
-                          (CB ? static_cast<size_t>(bPix) * (g.CBP + pitchPad) : 8) + 2 * kt) * 2u; // the last term: the staged bias, fp32
+      // the staging-wave variant keeps B's weights in registers and the finished tile (tlh rows of 64 pixels) in LDS
+      const size_t lds = (static_cast<size_t>(16 / classes * kt) * (g.CAP + 8) + (cfg.pw ? static_cast<size_t>(tlh) * 64 * kt : CB ? static_cast<size_t>(9 * kt) * (g.CBP + 8) : 8) +
+                          static_cast<size_t>(aPix) * (g.CAP + 8 * na) + (CB ? static_cast<size_t>(bPix) * (g.CBP + pitchPad) : 8) + 2 * kt) * 2u; // the last term: the staged bias, fp32
       if (lds > dev.maxComputeSharedMemory) continue;
       g.KT = kt; g.bpitch = g.CBP + pitchPad; g.ldsBytes = lds;
-      g.slots = std::max(1u, dev.computeUnits / (dev.xcdCount * 4 * (blocks / kb)));
+      g.slots = std::max(1u, dev.computeUnits / (dev.xcdCount * classes * (blocks / kb)));
       return true;
     }
   }
@@ -408,8 +429,13 @@ public:
         const unsigned others = PAT_POOL | PAT_CROP | PAT_PADA;
         FoldGeometry fg;
         if (!m.blocked() && (m.pattern & PAT_UPSAMPLE) && !(m.pattern & others) && conv.R == 3 && conv.S == 3 && conv.padX == 1 && conv.padY == 1 && conv.strideX == 1 && conv.strideY == 1 &&
-            opt.features.enableUpsampleFold && chooseFold(cfg, CA, CB, conv.K, opt.deviceInfo, fg))
+            opt.features.enableUpsampleFold && chooseFold(cfg, CA, CB, conv.K, opt.deviceInfo, fg)) {
+          if (cfg.pw && m.outputVariant) { // the staging-wave variant stores whole 16-byte slots
+            const ConcatView v = concatViewOf(model, m.output);
+            if (!v.valid || v.pitch % 8 || v.channelOffset % 8) continue;
+          }
           out.push_back(c);
+        }
         continue;
       }
       if (cfg.wideHalo && conv.strideX == 1 && conv.strideY == 1) continue;
@@ -464,8 +490,10 @@ public:
     const bool pool = (m.pattern & PAT_POOL) != 0, up = (m.pattern & PAT_UPSAMPLE) != 0, crop = (m.pattern & PAT_CROP) != 0;
     const bool padA = (m.pattern & PAT_PADA) != 0, padB = (m.pattern & PAT_PADB) != 0;
 
-    hip::HipCompilerInstance k = m_compiler->read(cfg.fold ? "conv3x3_upfold.hip" : cfg.resident ? "conv3x3_mfma_ws.hip" : "conv3x3_mfma.hip");
+    hip::HipCompilerInstance k = m_compiler->read(cfg.fold ? (cfg.pw ? "conv3x3_upfold_ws.hip" : "conv3x3_upfold.hip") : cfg.resident ? "conv3x3_mfma_ws.hip" : "conv3x3_mfma.hip");
     if (cfg.fold) k.define("BPITCH", fg.bpitch ? fg.bpitch : 8);
+    if (cfg.fold && cfg.pw) k.define("CKA", fg.cka);
+    if (cfg.ntStore) k.define("STORE_AUX", 2);
     k.define("CA", CA); k.define("CB", CB); k.define("UPA", up ? 1 : 0);
     k.define("KOUT", conv.K); k.define("KT", g.KT);
     k.define("ACT", act);
@@ -500,7 +528,7 @@ public:
     const Sym OW = convOut.width, OH = convOut.height;
     const unsigned th = cfg.waves * cfg.rpw;
     const unsigned nkt = g.KOUTP / g.KT;
-    auto d = cfg.fold ? impl.registerDispatch(k, entry, Sym::Const(opt.deviceInfo.xcdCount * 4 * nkt * g.slots), Sym::Const(1), Sym::Const(1), cfg.waves * 64)
+    auto d = cfg.fold ? impl.registerDispatch(k, entry, Sym::Const(opt.deviceInfo.xcdCount * (cfg.pw ? 2 : 4) * nkt * g.slots), Sym::Const(1), Sym::Const(1), (cfg.waves + cfg.pw) * 64)
            : cfg.resident ? impl.registerDispatch(k, entry, Sym::Const(opt.deviceInfo.xcdCount * nkt * g.slots), Sym::Const(1), Sym::Const(1), (cfg.waves + cfg.pw) * 64)
                           : impl.registerDispatch(k, entry, sym.cdiv(OW, cfg.mf == 32 ? 32 : 16 * cfg.xb), sym.cdiv(OH, th), Sym::Const(nkt), cfg.waves * 64);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);

@@ -61,9 +61,9 @@ ALL_CONFIGS += ["t16r1k16", "t16r1k32", "t16r2k16", "t8r2k16", "t8r2k32", "t8r4k
 # (tests/test_host.py checks on the CPU that every configuration of the library's table is in one of the lists of this file and
 # compiles for at least one of the layer shapes it is tested on here: a configuration must not be covered by skips alone)
 EVERY_CONFIG_SHAPES = [(80, 64, 45, 70), (73, 96, 130, 300), (16, 32, 300, 530)]
-FOLD_CONFIGS = ["f8r1", "f4r2", "f4r1"]
+FOLD_CONFIGS = ["f8r1", "f4r2", "f4r1", "g4r1", "g4r1k32", "g4r1n", "g4r1k32n"]
 FOLD_SHAPES = [(64, 9, 64, 36, 70, False), (16, 0, 32, 18, 34, False), (32, 24, 40, 62, 130, False), (8, 3, 3, 2, 2, False), (24, 9, 16, 40, 52, True),
-               (96, 32, 64, 34, 66, False)]
+               (96, 32, 64, 34, 66, False), (32, 16, 32, 50, 70, True), (48, 12, 96, 22, 134, False), (64, 8, 64, 2, 2, False), (16, 9, 32, 8, 64, False)]
 STRIDED_ONLY_CONFIGS = ["m2r1k32x1n", "w2r2k16n", "w2r1k16n"]  # offered to strided layers only
 
 
@@ -176,6 +176,43 @@ def test_upsample_folded_into_weights(oracle, config, CA, CB, K, H, W, padb):
     got = mod.instance(H=H, W=W).infer(*[feeds[k] for k in ("lo", "x") if k in feeds])[0]
     want = oracle.run_graph(m.to_ops({"H": H, "W": W}), feeds, "fp32")[t.name]
     assert_conv_close(got, want, f"fold {config}")
+
+
+def test_full_size_fold_equals_the_unfolded_kernel_bit_for_bit():
+    """The dominant layer of the 1080p U-Net (upsampled 64 channels + 9 replicate-padded input channels -> 64) at its real
+    extent, with small integers for inputs and weights: every product and sum is exact in binary16 / fp32, so the
+    upsample-folded kernels (weights summed per output parity) must give the unfolded kernel's bits."""
+    rng = np.random.default_rng(11)
+    H, W, CA, CB, K = 1088, 1920, 64, 9, 64
+    w = rng.integers(-1, 2, (K, CA + CB, 3, 3)).astype(np.float16)
+    b = rng.integers(-3, 4, K).astype(np.float16)
+    m = dx.Model()
+    lo = m.input("lo", m.sym("W") // 2, m.sym("H") // 2, CA)
+    x = m.input("x", "W", m.sym("H") - 8, CB)
+    t = m.relu(m.conv2d(m.concat(m.upsample(lo), m.pad(x, 0, 0, 4, 4)), w, b))
+    m.output(t)
+    xa = rng.integers(0, 3, (H // 2, W // 2, CA)).astype(np.float16)
+    xb = rng.integers(0, 3, (H - 8, W, CB)).astype(np.float16)
+    outs = {}
+    for config in ("s8r2k16", "g4r1", "g4r1k32", "g4r1n", "f8r1"):
+        mod = dx.Module.compile(m, conv_config=config, assume={"H": H, "W": W})
+        assert config in dx.last_compile_report() and mod.runtime_model.dispatch_count == 1
+        outs[config] = mod.instance(H=H, W=W).infer(xa, xb)[0]
+    assert outs["s8r2k16"].max() > 100 and np.array_equal(outs["s8r2k16"], np.round(outs["s8r2k16"]))
+    for config in ("g4r1", "g4r1k32", "g4r1n", "f8r1"):
+        assert_bits_equal(outs[config], outs["s8r2k16"], config)
+    # and the unfolded kernel against the definition, on the four corners and a centre patch (float64 on the host)
+    up = np.repeat(np.repeat(xa.astype(np.float64), 2, 0), 2, 1)
+    xp = np.pad(xb.astype(np.float64), ((4, 4), (0, 0), (0, 0)), mode="edge")
+    src = np.pad(np.concatenate([up, xp], 2), ((1, 1), (1, 1), (0, 0)))
+    wf = w.astype(np.float64)
+    for y0, x0 in [(0, 0), (0, W - 24), (H - 24, 0), (H - 24, W - 24), (500, 900)]:
+        acc = np.zeros((24, 24, K))
+        for r in range(3):
+            for q in range(3):
+                acc += src[y0 + r:y0 + r + 24, x0 + q:x0 + q + 24] @ wf[:, :, r, q].T
+        want = np.maximum(acc + b.astype(np.float64), 0)
+        assert np.array_equal(outs["s8r2k16"][y0:y0 + 24, x0:x0 + 24].astype(np.float64), want), (y0, x0)
 
 
 def test_tensor_size_limit_is_reported():
