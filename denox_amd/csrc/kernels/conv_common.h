@@ -318,7 +318,7 @@ __device__ DNX_INLINE Sources make_sources(const _Float16 *A, const _Float16 *B,
 // ---- halo staging ---------------------------------------------------------------------
 // The (TH+2) x 34 pixel halo of one reduction step is moved by NTH threads, 16 bytes
 // (8 channels) per access.  Vector i = t + it*NTH covers pixel i / (CK/8), channel group
-// i % (CK/8).  What does not change between steps is computed once: the LDS slot of each
+// i % (CK/8) (block-major sources: channel group i / HALO_PIX, pixel i % HALO_PIX).  What does not change between steps is computed once: the LDS slot of each
 // of a thread's vectors (HaloMap, per kernel) and the element offsets of its pixels in
 // the sources (HaloSrc, per tile).
 #define VPPK (CK / 8)
@@ -346,8 +346,14 @@ struct Halo {
 #pragma unroll
     for (int it = 0; it < NV; ++it) {
       const int i = t + it * NTH;
+#if LAYIN
+      // block-major sources: consecutive lanes take consecutive pixels of one 8-channel plane (16 consecutive bytes each)
+      const int v = i / HALO_PIX;
+      const int pix = i - v * HALO_PIX;
+#else
       const int pix = i / VPPK;
       const int v = i - pix * VPPK;
+#endif
       m.hy[it] = pix / HALO_W;
       m.hx[it] = pix - m.hy[it] * HALO_W;
       m.v8[it] = v * 8;

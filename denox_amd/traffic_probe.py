@@ -1,0 +1,125 @@
+"""HBM traffic of the benchmark's dominant convolution, per candidate kernel, keyed by the SHA-256 of the code object.
+
+Two steps:
+
+`python3 -m denox_amd.traffic_probe run <map.json> [H W]` compiles the OIDN U-Net once per candidate configuration of its
+most expensive layer (dec_conv1a: concat + replicate pad + 2x upsample + conv 73 -> 64 + ReLU), steering the selection to
+that candidate through a timing table that holds one made-up sample for it, runs every such schedule a few times, runs the
+plain copy kernel of `denox_amd.calibrate`, and writes which entry point belongs to which code object.  Run it under
+`rocprofv3 --pmc FETCH_SIZE` and again under `rocprofv3 --pmc WRITE_SIZE` (counters per dispatch, csv).
+
+`python3 -m denox_amd.traffic_probe summarize <map.json> <FETCH_SIZE csv> <WRITE_SIZE csv>` averages the counters per
+kernel, scales them by what the same counter read for the copy kernel of known size, and prints the JSON that
+bench.py reads (`profiles/dominant_conv_traffic.json`): bytes fetched from and written to memory per launch, per code object.
+"""
+import csv
+import json
+import os
+import re
+import sys
+import tempfile
+
+import numpy as np
+
+# Candidates of the dominant layer that the timing table has been seen to select, in both result layouts
+CANDIDATES = ["g4r1n", "g4r1k32n", "g4r1", "g4r1k32", "s8r2k16", "s8r2k16/hwc>chwc8", "s12r1k16", "s12r1k16/hwc>chwc8", "t8r2k16", "p8r2k16", "f8r1"]
+DOMINANT_OPERATION = "concat+pad+upsample+conv3x3+relu"
+COPY_KERNEL = "memory_slice_c64v8"
+
+
+def _norm(config):
+    """'s8r2k16/kt64/hwc>chwc8' -> 's8r2k16/hwc>chwc8': the output channels per workgroup follow from the layer."""
+    return re.sub(r"/kt\d+", "", config.strip('"'))
+
+
+def run(map_path, H=1080, W=1920, frames=6):
+    import denox_amd as dx
+    from denox_amd import calibrate, networks
+    model, _ = networks.build("oidn_unet", seed=0)
+    x = networks.synthetic_input("oidn_unet", H, W, seed=0)
+    kernels = {}
+    tmp = tempfile.mkdtemp(prefix="denox_hip_probe_")
+    for cand in CANDIDATES:
+        db = dx.Db(os.path.join(tmp, cand.replace("/", "_").replace(">", "_") + ".db"))
+        db.populate(model, assume={"H": H, "W": W})
+        rows = [r.split('","') for r in db.dump_csv().splitlines()[1:]]
+        hits = [i for i, r in enumerate(rows) if r[0].strip('"') == DOMINANT_OPERATION and _norm(r[2]) == cand]
+        if not hits:
+            print(f"traffic_probe: no candidate '{cand}' for {DOMINANT_OPERATION}", file=sys.stderr)
+            continue
+        for i in hits:
+            for _ in range(3):
+                db.add_sample(i, 1000.0)  # 1 us: below every estimate, so the selection takes this candidate
+        blob = dx.compile_model(model, assume={"H": H, "W": W}, db=db)
+        desc = dx.describe(blob, H=H, W=W)["dispatches"]
+        dom = [d for d in desc if d["name"] == DOMINANT_OPERATION]
+        if len(dom) != 1 or _norm(dom[0]["debug_info"].split(" | ")[0]) != cand:
+            print(f"traffic_probe: the schedule did not take '{cand}': {[d['debug_info'].split(' | ')[0] for d in dom]}", file=sys.stderr)
+            continue
+        inst = dx.Module.load(blob).instance(H=H, W=W)
+        inst.infer(x)
+        for _ in range(frames):
+            inst.infer_device(None, None)
+        inst.synchronize()
+        times = inst.bench(warmup=1)
+        for d, t in zip(desc, times):
+            k = kernels.setdefault(d["entry_point"], {"code_sha256": d["code_sha256"], "operation": d["name"], "config": d["debug_info"].split(" | ")[0],
+                                                     "algorithmic_read_bytes": t["memory_reads"], "algorithmic_write_bytes": t["memory_writes"], "flops": t["flops"]})
+            if k["code_sha256"] != d["code_sha256"]:
+                raise RuntimeError(f"two code objects share the entry point {d['entry_point']}")
+        del inst
+    calibrate.main()
+    with open(map_path, "w") as f:
+        json.dump({"height": H, "width": W, "dominant_operation": DOMINANT_OPERATION, "copy_kernel": COPY_KERNEL,
+                   "copy_kernel_bytes": 1088 * 1920 * 64 * 2, "kernels": kernels}, f, indent=1)
+    print(f"traffic_probe: {len(kernels)} kernels -> {map_path}")
+    return 0
+
+
+def per_kernel(csv_path, counter):
+    acc = {}
+    with open(csv_path) as f:
+        for r in csv.DictReader(f):
+            if r["Counter_Name"] == counter:
+                acc.setdefault(r["Kernel_Name"], []).append(float(r["Counter_Value"]))
+    return acc
+
+
+def summarize(map_path, fetch_csv, write_csv):
+    with open(map_path) as f:
+        m = json.load(f)
+    fetch, write = per_kernel(fetch_csv, "FETCH_SIZE"), per_kernel(write_csv, "WRITE_SIZE")
+    n = m["copy_kernel_bytes"]
+    cf, cw = fetch[m["copy_kernel"]], write[m["copy_kernel"]]
+    # skip the first launch of the copy (cold caches)
+    fscale, wscale = n / np.mean(cf[1:]), n / np.mean(cw[1:])
+    out = {"height": m["height"], "width": m["width"], "dominant_operation": m["dominant_operation"],
+           "source": "rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of `python3 -m denox_amd.traffic_probe run` (see profiles/dominant_conv_traffic.md)",
+           "calibration": {"copy_kernel": m["copy_kernel"], "copy_kernel_bytes": n, "fetch_size_per_dispatch": round(float(np.mean(cf[1:])), 1),
+                           "write_size_per_dispatch": round(float(np.mean(cw[1:])), 1), "fetch_bytes_per_unit": round(fscale, 1), "write_bytes_per_unit": round(wscale, 1)},
+           "kernels": {}}
+    for entry, k in sorted(m["kernels"].items()):
+        if entry not in fetch or entry not in write:
+            continue
+        f_, w_ = fetch[entry], write[entry]
+        fb, wb = float(np.mean(f_[1:] if len(f_) > 1 else f_)) * fscale, float(np.mean(w_[1:] if len(w_) > 1 else w_)) * wscale
+        alg = k["algorithmic_read_bytes"] + k["algorithmic_write_bytes"]
+        out["kernels"][k["code_sha256"]] = {"entry_point": entry, "operation": k["operation"], "config": k["config"], "dispatches": [len(f_), len(w_)],
+                                            "fetch_bytes": int(round(fb, -3)), "write_bytes": int(round(wb, -3)),
+                                            "algorithmic_read_bytes": k["algorithmic_read_bytes"], "algorithmic_write_bytes": k["algorithmic_write_bytes"],
+                                            "traffic_over_algorithmic": round((fb + wb) / alg, 3) if alg else None}
+    print(json.dumps(out, indent=1))
+    return 0
+
+
+def main(argv):
+    if len(argv) >= 2 and argv[0] == "run":
+        return run(argv[1], *[int(a) for a in argv[2:4]])
+    if len(argv) == 4 and argv[0] == "summarize":
+        return summarize(*argv[1:])
+    print(__doc__, file=sys.stderr)
+    return 2
+
+
+if __name__ == "__main__":
+    sys.exit(main(sys.argv[1:]))
