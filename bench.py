@@ -332,7 +332,8 @@ def main() -> int:
                    "schedule": "min-cost over measured dispatch latencies" if db is not None else "min-cost over roofline estimates",
                    "tuning_seconds": round(tune_s, 2), "host_pointer_path_ms_per_frame": round(host_ms, 3), "host_pointer_pipelined_ms_per_frame": round(pipelined_ms, 3),
                    "single_replay_ms_median": round(singles[len(singles) // 2], 4), "single_replay_ms_p95": round(singles[int(len(singles) * 0.95)], 4),
-                   "layout_preference": args.layout_preference, "internal_tensors_in_chwc8": chwc8, "schedule_configs": chosen},
+                   "layout_preference": args.layout_preference, "internal_tensors_in_chwc8": chwc8, "schedule_configs": chosen,
+                   "schedule_kernels": [d["entry_point"] for d in desc]},
         "roofline": roofline,
     }
     if non_conv is not None:

@@ -48,7 +48,8 @@ std::string fmtFloat(float v) {
 // pp: two-phase schedule of the persistent kernel (two wave groups alternate matrix work and everything else).
 // fold: the 2x upsample of source A folded into the weights (conv3x3_upfold.hip, with pw: conv3x3_upfold_ws.hip; rpw counts low-resolution rows).
 // ntStore: the result is stored with the non-temporal cache policy.
-struct ConvConfig { unsigned waves, rpw, ck; bool resident; unsigned pw; unsigned maxKT; unsigned mf, xb; const char *name; bool pp = false; bool fold = false; bool wideHalo = false; bool ntStore = false; };
+// ostage: the finished tile goes to memory through LDS, stored by the staging waves (OSTAGE in conv3x3_mfma_ws.hip).
+struct ConvConfig { unsigned waves, rpw, ck; bool resident; unsigned pw; unsigned maxKT; unsigned mf, xb; const char *name; bool pp = false; bool fold = false; bool wideHalo = false; bool ntStore = false; bool ostage = false; };
 const ConvConfig kConvConfigs[] = {
     // weights streamed per step
     {4, 2, 16, false, 0, 0, 32, 1, "w4r2k16"}, {4, 2, 32, false, 0, 0, 32, 1, "w4r2k32"}, {4, 4, 16, false, 0, 0, 32, 1, "w4r4k16"}, {4, 4, 32, false, 0, 0, 32, 1, "w4r4k32"},
@@ -67,6 +68,10 @@ const ConvConfig kConvConfigs[] = {
     {4, 2, 32, true, 0, 32, 32, 1, "p4r2k32n"}, {4, 1, 32, true, 0, 32, 32, 1, "p4r1k32n"},
     // resident + staging-only waves
     {8, 2, 16, true, 4, 0, 32, 1, "s8r2k16"},  {12, 1, 16, true, 4, 0, 32, 1, "s12r1k16"},
+    // resident + staging-only waves that also store the result (whole pixels per store instruction, through LDS)
+    {4, 2, 16, true, 4, 0, 32, 1, "r4r2k16", false, false, false, false, true}, {4, 2, 16, true, 4, 0, 32, 1, "r4r2k16n", false, false, false, true, true},
+    {8, 1, 16, true, 4, 0, 32, 1, "r8r1k16n", false, false, false, true, true}, {4, 2, 32, true, 4, 0, 32, 1, "r4r2k32n", false, false, false, true, true},
+    {4, 1, 16, true, 4, 0, 32, 1, "r4r1k16n", false, false, false, true, true},
     // 16x16x32 matrix shape: output channels in blocks of 16, tiles of 16 or 32 pixels width
     {4, 2, 32, false, 0, 0, 16, 2, "m4r2k32x2"}, {4, 2, 64, false, 0, 0, 16, 2, "m4r2k64x2"}, {4, 1, 32, false, 0, 0, 16, 2, "m4r1k32x2"}, {4, 2, 32, false, 0, 0, 16, 1, "m4r2k32x1"},
     {4, 4, 32, false, 0, 0, 16, 1, "m4r4k32x1"}, {8, 2, 32, false, 0, 0, 16, 2, "m8r2k32x2"}, {4, 2, 0, false, 0, 0, 16, 1, "m4r2kfx1"},  {4, 1, 0, false, 0, 0, 16, 2, "m4r1kfx2"},
@@ -94,7 +99,7 @@ constexpr unsigned kNumConvConfigs = sizeof(kConvConfigs) / sizeof(kConvConfigs[
 // Configurations that are also offered with channel-block-major (CHWC8) sources and / or result: one or two of each kernel
 // family and matrix shape, so that the layout alternative adds half as many candidates again instead of three times as many.
 bool offeredBlocked(const ConvConfig &cfg) {
-  for (const char *n : {"w4r2k16", "w8r2k32", "w4r1kfn", "p16r2k16", "s8r2k16", "t8r2k32", "t16r1k32", "m4r2k32x1", "m8r2k32x2", "m4r2kfx1", "q8r2k32x2", "s12r1k16"})
+  for (const char *n : {"w4r2k16", "w8r2k32", "w4r1kfn", "p16r2k16", "s8r2k16", "t8r2k32", "t16r1k32", "m4r2k32x1", "m8r2k32x2", "m4r2kfx1", "q8r2k32x2", "s12r1k16", "r4r2k16n"})
     if (std::strcmp(n, cfg.name) == 0) return true;
   return false;
 }
@@ -149,7 +154,8 @@ bool chooseKT(const ConvConfig &cfgIn, unsigned CA, unsigned CB, unsigned K, con
     if (accRegs + 64 + (cfg.mf == 16 ? kb * 4 : 0) > regBudget) continue;
     const size_t lds = (cfg.resident ? static_cast<size_t>(taps * kb * blk) * (g.CPAD + 8) * 2u + 2u * static_cast<size_t>(haloPix) * ckp * 2u
                                      : (static_cast<size_t>(haloPix) + taps * kb * blk) * ckp * 2u) +
-                       static_cast<size_t>(kb * blk) * 4u; // + the staged bias (fp32)
+                       static_cast<size_t>(kb * blk) * 4u + // + the staged bias (fp32)
+                       (cfg.ostage ? static_cast<size_t>(th * tw) * (kb * blk / 8 + 1) * 16u : 0u); // + the finished tile (one spare 16-byte slot per pixel)
     if (lds > dev.maxComputeSharedMemory) continue;
     {
       // a thread stages at most 64 halo vectors per step (the kernels' bookkeeping is one bit per vector)
@@ -439,6 +445,13 @@ public:
         continue;
       }
       if (cfg.wideHalo && conv.strideX == 1 && conv.strideY == 1) continue;
+      if (cfg.ostage) { // whole 16-byte slots of a pixel-major result, at least two steps per tile
+        if ((m.pattern & (PAT_POOL | PAT_CROP)) || m.outputFormat || conv.K % 8 || cpad / stepChannels(cfg, cpad) < 2) continue;
+        if (m.outputVariant) {
+          const ConcatView v = concatViewOf(model, m.output);
+          if (!v.valid || v.pitch % 8 || v.channelOffset % 8) continue;
+        }
+      }
       if (m.blocked()) {
         if (!offeredBlocked(cfg)) continue;
         // block-major sources are read through the per-step buffer resource: every LDS step must lie in one source
@@ -494,6 +507,7 @@ public:
     if (cfg.fold) k.define("BPITCH", fg.bpitch ? fg.bpitch : 8);
     if (cfg.fold && cfg.pw) k.define("CKA", fg.cka);
     if (cfg.ntStore) k.define("STORE_AUX", 2);
+    if (cfg.ostage) k.define("OSTAGE", 1);
     k.define("CA", CA); k.define("CB", CB); k.define("UPA", up ? 1 : 0);
     k.define("KOUT", conv.K); k.define("KT", g.KT);
     k.define("ACT", act);

@@ -13,6 +13,11 @@
 //           PW further waves only stage halos, so that address arithmetic, load waits and LDS
 //           writes run beside the matrix work instead of in front of it (all waves of a
 //           workgroup meet at the step barrier, so inside one role nothing overlaps).
+//   OSTAGE  (with PW > 0, pixel-major result, at least two steps per tile) the finished tile goes to memory through
+//           LDS: the computing waves leave it there as binary16, and the staging waves store it during the next tile's
+//           first step with consecutive lanes on consecutive 16 bytes -- whole pixels (KT channels), 1 KiB per store
+//           instruction, instead of 16 bytes per lane at a stride of one pixel.  The computing waves then never wait
+//           for memory at all.
 //
 // Workgroup b serves XCD b % 8 (workgroups are dealt round-robin to the 8 XCDs), and each
 // XCD walks its own contiguous band of tiles so that neighbouring halos meet in one L2.
@@ -29,6 +34,15 @@
 #define NXCD 8 // accelerator dies, each with an L2 of its own; the host sizes the grid with the same number
 #endif
 #define NSTAGE ((PW > 0 ? PW : WAVES) * 64) // threads that stage halos
+#ifndef OSTAGE
+#define OSTAGE 0
+#endif
+#if OSTAGE
+static_assert(PW > 0 && MF == 32 && NCHUNK >= 2 && !POOL && !CROP && !LAYOUT_OUT && OVEC && OPITCH % 8 == 0 && KOUT % 8 == 0, "staged result: see above");
+#define SPP (KT / 8)                             // 16-byte slots of a pixel's KT channels
+#define OSLOTS (SPP + 1)                         // pitch of a pixel in the staged tile: odd, so that 16 consecutive pixels start in 16 different bank groups
+#define NVO ((TH * TW * SPP + NSTAGE - 1) / NSTAGE) // slots per staging thread
+#endif
 
 extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     const _Float16 *__restrict__ A,
@@ -43,6 +57,9 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   __shared__ __attribute__((aligned(16))) _Float16 sW[NTAPS * KT * CPADP];
   __shared__ __attribute__((aligned(16))) _Float16 sIn[2][HALO_PIX * CKP];
   __shared__ __attribute__((aligned(16))) bias_t sBias[KT];
+#if OSTAGE
+  __shared__ uint4v sOut[TH * TW * OSLOTS];
+#endif
 #if CB == 0
   const _Float16 *B = nullptr;
 #endif
@@ -227,6 +244,24 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
       if (++cchunk == NCHUNK)
         cchunk = 0;
     };
+#if OSTAGE
+    // the n-th tile of this workgroup, as the computing waves left it in LDS
+    const int stid = tid - WAVES * 64;
+    auto store_staged = [&](int n) {
+      const int t = tile + n * SLOTS;
+      const int y0 = tileY(t), x0 = tileX(t);
+#pragma unroll
+      for (int it = 0; it < NVO; ++it) {
+        const int i = stid + it * NSTAGE;
+        const int p = i / SPP, sl = i - p * SPP; // pixel of the tile (row-major), slot of the pixel
+        const int y = y0 + p / TW, x = x0 + p % TW;
+        const bool ok = i < TH * TW * SPP && y < (int)CONV_OUT_H(pc) && x < (int)CONV_OUT_W(pc) && kt * KT + sl * 8 < KOUT;
+        const uint4v v = sOut[i < TH * TW * SPP ? p * OSLOTS + sl : 0];
+        const unsigned off = ((unsigned)(y * (int)CONV_OUT_W(pc) + x) * (unsigned)OPITCH + (unsigned)(kt * KT + sl * 8)) * 2u;
+        __builtin_amdgcn_raw_buffer_store_b128(v, out, ok ? off : NO_STORE, 0, STORE_AUX);
+      }
+    };
+#endif
     issue(st0);         // step 0
     issue(st1);         // step 1
     commit(st0, 0);
@@ -237,6 +272,10 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
         commit(st1, g + 1);
         issue(st1);     // step g + 3
       }
+#if OSTAGE
+      if (g > 0 && g % NCHUNK == 0)
+        store_staged(g / NCHUNK - 1); // complete since the barrier above; rewritten after the last barrier of this tile
+#endif
       if (g + 1 >= steps)
         break;
       DNX_SYNC();       // step g + 1 starts
@@ -244,7 +283,15 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
         commit(st0, g + 2);
         issue(st0);     // step g + 4
       }
+#if OSTAGE
+      if ((g + 1) % NCHUNK == 0)
+        store_staged((g + 1) / NCHUNK - 1);
+#endif
     }
+#if OSTAGE
+    DNX_SYNC();         // the last tile is in LDS
+    store_staged(myTiles - 1);
+#endif
   } else {
     // ---- computing waves ----
     Acc acc;
@@ -255,11 +302,27 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
         init_acc(acc, sBias, lane);
       mma_step<CPADP>(sIn[g & 1], sW, cchunk * CK, acc, wv, lane, cchunk);
       if (++cchunk == NCHUNK) {
+#if OSTAGE
+        // the tile as binary16 into LDS: this lane's 16 channels kb * 32 + (lane >> 5) * 16 .. of pixel (wv * RPW + j, lane & 31)
+        Packed pk;
+        pack_tile(acc, pk);
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+          for (int j = 0; j < RPW; ++j)
+#pragma unroll
+            for (int e = 0; e < 2; ++e)
+              sOut[((wv * RPW + j) * TW + (lane & 31)) * OSLOTS + kb * 4 + (lane >> 5) * 2 + e] = __builtin_bit_cast(uint4v, pk.o[kb][j][e]);
+#else
         store_tile(acc, out, tileY(tile), tileX(tile), kt, wv, lane, pc);
+#endif
         cchunk = 0;
         tile += SLOTS;
       }
     }
+#if OSTAGE
+    DNX_SYNC(); // the last tile is in LDS
+#endif
   }
 #endif
 }

@@ -99,7 +99,9 @@ def summarize(map_path, fetch_csv, write_csv):
                            "write_size_per_dispatch": round(float(np.mean(cw[1:])), 1), "fetch_bytes_per_unit": round(fscale, 1), "write_bytes_per_unit": round(wscale, 1)},
            "kernels": {}}
     for entry, k in sorted(m["kernels"].items()):
-        if entry not in fetch or entry not in write:
+        # the dominant layer's candidates and the two conv -> conv dispatches: kernels that run at one extent only
+        # (a name like conv3x3_c96_k96_relu_* serves two layers of different size; a mean over both describes neither)
+        if entry not in fetch or entry not in write or not (k["operation"] == m["dominant_operation"] or entry.startswith("convpair_")):
             continue
         f_, w_ = fetch[entry], write[entry]
         fb, wb = float(np.mean(f_[1:] if len(f_) > 1 else f_)) * fscale, float(np.mean(w_[1:] if len(w_) > 1 else w_)) * wscale

@@ -59,6 +59,36 @@ def test_conv_reads_and_writes_either_layout(oracle, config, C, K, tail):
         assert_conv_close(got, want, f"blocked {config} {C}->{K} {H}x{W}")
 
 
+def test_staged_result_kernel_reads_block_major_sources(oracle, tmp_path):
+    """r4r2k16n (the result goes to memory through LDS, pixel-major only) reading a CHWC8 tensor: no forced configuration
+    reaches that combination, because the producer must write CHWC8 with another configuration, so the selection is
+    steered to it through a timing table with made-up samples for exactly the wanted candidates."""
+    import re
+    rng = np.random.default_rng(21)
+    m = dx.Model()
+    t = m.input("input", "W", "H", 64)
+    a = m.relu(m.conv2d(t, he_weights(rng, 48, 64), small_bias(rng, 48)))
+    b = m.relu(m.conv2d(a, he_weights(rng, 80, 48), small_bias(rng, 80)))
+    c = m.conv2d(b, he_weights(rng, 64, 80), small_bias(rng, 64))
+    m.output(c)
+    wanted = {"conv3x3_c64_k48_relu_bo_w4r2k16", "conv3x3_c48_k80_relu_bi_r4r2k16n", "conv3x3_c80_k64_r4r2k16n"}
+    feats = dict(conv_conv_fusion=False)
+    db = dx.Db(str(tmp_path / "steer.db"))
+    db.populate(m, features=feats)
+    for i, row in enumerate(db.dump_csv().splitlines()[1:]):
+        if re.search(r"KERNEL_NAME=(\S+)", row).group(1) in wanted:
+            for _ in range(3):
+                db.add_sample(i, 1000.0)
+    mod = dx.Module.compile(m, db=db, features=feats)
+    for H, W in [(37, 70), (16, 32), (130, 45)]:
+        assert set(entries(mod, H=H, W=W)) == wanted
+        x = rng.standard_normal((H, W, 64)).astype(np.float16)
+        fill_lds_with_nans()
+        got = mod.instance(H=H, W=W).infer(x)[0]
+        want = oracle.run_graph(m.to_ops({"H": H, "W": W}), {"input": x}, "fp32")[c.name]
+        assert_conv_close(got, want, f"staged result, block-major source {H}x{W}")
+
+
 def test_every_blocked_configuration_runs_somewhere():
     rng = np.random.default_rng(0)
     for config in BLOCKED_CONFIGS:
