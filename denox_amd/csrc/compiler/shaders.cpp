@@ -616,8 +616,11 @@ private:
 // single-convolution shader folds in front of a convolution is available in front of the first one, everything it folds
 // behind a convolution behind the second one.  The reference fuses for the same purpose -- to keep a tensor from
 // crossing memory -- in ConcatConvCMShader (conv/ConcatConvCMShader.cpp:760-965); a conv -> conv fusion it does not have.
-struct PairConfig { unsigned waves, rpw, ck; const char *name; }; // ck: input channels of the first convolution per LDS stage
-const PairConfig kPairConfigs[] = {{8, 2, 16, "x8r2k16"}, {4, 2, 32, "x4r2k32"}, {4, 4, 16, "x4r4k16"}, {4, 2, 16, "x4r2k16"}};
+// ck: input channels of the first convolution per LDS stage; pw: extra waves that only move halos (the others then only compute)
+// w1reg: the first convolution's weights in registers of the computing waves (needs pw)
+struct PairConfig { unsigned waves, rpw, ck; const char *name; unsigned pw = 0; bool w1reg = false; };
+const PairConfig kPairConfigs[] = {{8, 2, 16, "x8r2k16"}, {4, 2, 32, "x4r2k32"}, {4, 4, 16, "x4r4k16"}, {4, 2, 16, "x4r2k16"},
+                                   {4, 2, 32, "y4r2k32", 4}, {4, 2, 64, "z4r2k64", 4, true}};
 constexpr unsigned kNumPairConfigs = sizeof(kPairConfigs) / sizeof(kPairConfigs[0]);
 
 bool isPairConfigName(const std::string &name) {
@@ -632,9 +635,9 @@ bool choosePair(const PairConfig &cfg, unsigned CA, unsigned CB, unsigned K1, un
   if (K1 > 32 || K2 > 32 || cfg.ck % 16 || cfg.ck > 64) return false;
   if (cfg.ck > g.CPAD && cfg.ck != 16) return false; // a larger stage than the whole reduction adds nothing
   g.ck = std::min(cfg.ck, g.CPAD);
-  const unsigned ih = cfg.waves * cfg.rpw, haloPix = (ih + 2) * 34, ckp = g.ck + 8, threads = cfg.waves * 64;
+  const unsigned ih = cfg.waves * cfg.rpw, haloPix = (ih + 2) * 34, ckp = g.ck + 8, threads = (cfg.pw ? cfg.pw : cfg.waves) * 64; // threads that move halos
   if ((haloPix * (g.ck / 8) + threads - 1) / threads > 64) return false;
-  const unsigned regBudget = std::min(256u, 512u / ((cfg.waves + 3) / 4));
+  const unsigned regBudget = std::min(256u, 512u / ((cfg.waves + cfg.pw + 3) / 4));
   // A second convolution with at most 5 output channels carries its three filter columns in the matrix rows (TAPM in
   // conv3x3_pair.hip): a third of the matrix instructions, weights of 3 instead of 9 taps in registers.
   g.tapm = 3 * K2 <= 15 && !pool;
@@ -642,7 +645,8 @@ bool choosePair(const PairConfig &cfg, unsigned CA, unsigned CB, unsigned K1, un
   if ((g.tapm ? 24 : 72) + cfg.rpw * 16 + 96 > regBudget) return false;
   const unsigned nchunk = (g.CPAD + g.ck - 1) / g.ck;
   const unsigned ringRows = nchunk == 1 ? 2 * ih + 2 : ih + 2; // see conv3x3_pair.hip
-  g.ldsBytes = static_cast<size_t>(9 * 32) * (g.CPAD + 8) * 2 + 2 * static_cast<size_t>(haloPix) * ckp * 2 + (static_cast<size_t>(ringRows) * 32 + 2) * 40 * 2 + 2 * 32 * 4;
+  if (cfg.w1reg && 9 * (g.CPAD / 16) * 4 > 144) return false; // the first convolution's weights must fit the register file next to everything else
+  g.ldsBytes = (cfg.w1reg ? 0 : static_cast<size_t>(9 * 32) * (g.CPAD + 8) * 2) + 2 * static_cast<size_t>(haloPix) * ckp * 2 + (static_cast<size_t>(ringRows) * 32 + 2) * 40 * 2 + 2 * 32 * 4;
   if (g.ldsBytes > dev.maxComputeSharedMemory) return false;
   g.slots = std::max(1u, dev.computeUnits / dev.xcdCount);
   return true;
@@ -744,7 +748,7 @@ public:
       const PairConfig &cfg = kPairConfigs[c];
       if (isPairConfigName(opt.forceConvConfig) && opt.forceConvConfig != cfg.name) continue;
       if ((m.pattern & PAT_POOL) && (cfg.rpw % 2)) continue;
-      if (cfg.waves * 64 > opt.deviceInfo.maxComputeWorkGroupInvocations) continue;
+      if ((cfg.waves + cfg.pw) * 64 > opt.deviceInfo.maxComputeWorkGroupInvocations) continue;
       PairGeometry g;
       if (!choosePair(cfg, CA, CB, first->K, second->K, (m.pattern & PAT_POOL) != 0, opt.deviceInfo, g)) continue;
       // block-major sources are read through the per-step buffer resource: every LDS step must lie in one source
@@ -798,6 +802,8 @@ public:
     k.define("WAVES", cfg.waves); k.define("RPW", cfg.rpw); k.define("CK", g.ck);
     k.define("SLOTS", g.slots); k.define("NXCD", opt.deviceInfo.xcdCount);
     if (g.tapm) k.define("TAPM", 1);
+    if (cfg.pw) k.define("PW", cfg.pw);
+    if (cfg.w1reg) k.define("W1REG", 1);
     const bool blockedIn = !m.inputFormats.empty() && m.inputFormats[0] != 0, blockedOut = m.outputFormat != 0;
     if (blockedIn) k.define("LAYIN", 1);
     if (blockedOut) k.define("LAYOUT_OUT", 1);
@@ -805,7 +811,7 @@ public:
     const std::string entry = "convpair_c" + std::to_string(CA) + (up ? "u" : "") + (padA ? "e" : "") + (CB ? "p" + std::to_string(CB) + (padB ? "e" : "") : "") + "_k" +
                               std::to_string(first.K) + actName(act1) + "_k" + std::to_string(second.K) + actName(act2) + (pool ? "_pool" : "") + (crop ? "_crop" : "") + (blockedIn ? "_bi" : "") + (blockedOut ? "_bo" : "") + "_" + cfg.name;
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, Sym::Const(opt.deviceInfo.xcdCount * g.slots), Sym::Const(1), Sym::Const(1), cfg.waves * 64);
+    auto d = impl.registerDispatch(k, entry, Sym::Const(opt.deviceInfo.xcdCount * g.slots), Sym::Const(1), Sym::Const(1), (cfg.waves + cfg.pw) * 64);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     if (CB) d.addBinding(dnx::Access::ReadOnly, m.inputs[1]);
     d.addBinding(dnx::Access::WriteOnly, m.output);

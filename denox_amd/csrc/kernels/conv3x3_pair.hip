@@ -32,6 +32,12 @@
 //   TAPM                          1: the second convolution has so few output channels (3 KOUT <= 15) that its three filter
 //                                 columns ride in the matrix rows (see below); not combined with POOL
 //   SLOTS, NXCD                   the grid is NXCD * SLOTS persistent workgroups
+//   PW                            0: every wave stages its share of the halo and computes; > 0: WAVES waves only compute
+//                                 and PW further waves only move halos from memory to LDS (as in conv3x3_mfma_ws.hip)
+//   W1REG                         1: the first convolution's weights live in registers of the computing waves as well
+//                                 (9 taps x CPAD / 16 fragments), not in LDS.  With 32 output channels a weight fragment
+//                                 serves RPW matrix instructions only, so reading it from LDS is 3 of the 7 LDS reads per
+//                                 6 instructions, and the LDS read rate, not the matrix pipe, sets the pace of such layers
 // KT is 32 for both convolutions.
 #include "conv_common.h"
 
@@ -53,11 +59,14 @@
 #ifndef TAPM
 #define TAPM 0
 #endif
+#ifndef W1REG
+#define W1REG 0
+#endif
 static_assert(!TAPM || (3 * KOUT <= 15 && !POOL), "filter columns in the matrix rows: at most 5 output channels, no pooling");
 
 static_assert(MF == 32 && KT == 32 && KB == 1, "one 32-channel block per convolution");
 static_assert(KR == 3 && KS == 3 && SY == 1 && SX == 1 && PY == 1 && PX == 1, "3x3, stride 1, extent-preserving");
-static_assert(K1 <= 32 && KOUT <= 32 && PW == 0 && PP == 0, "unsupported variant");
+static_assert(K1 <= 32 && KOUT <= 32 && PP == 0, "unsupported variant");
 
 #define CPADP (CPAD + 8)
 #define IH TH             // rows of `mid` per step
@@ -259,6 +268,63 @@ __device__ DNX_INLINE void mma_first(const _Float16 *sIn, const _Float16 *sW, in
   }
 }
 
+#if W1REG
+// The first convolution's weights in registers: fragment [tap][16-channel slice] of weight row lane & 31 (global layout
+// [tap][32 rows][CPAD]).
+struct FirstWeights {
+  half8 w[NTAPS][CPAD / 16];
+};
+__device__ DNX_INLINE void load_first_weights(FirstWeights &fw, const _Float16 *__restrict__ FILT1, int lane) {
+  const int l32 = lane & 31, kq = (lane >> 5) * 8;
+#pragma unroll
+  for (int tap = 0; tap < NTAPS; ++tap)
+#pragma unroll
+    for (int ks = 0; ks < CPAD / 16; ++ks)
+      fw.w[tap][ks] = __builtin_bit_cast(half8, ld16(FILT1 + (size_t)(tap * 32 + l32) * CPAD + ks * 16 + kq));
+}
+
+// mma_first with the weights from registers; CHUNK (compile-time) selects the 16-channel slices CHUNK * CK / 16 ...
+template <int L, int CHUNK>
+__device__ DNX_INLINE void mma_first_reg(const _Float16 *sIn, const FirstWeights &fw, Acc &acc, int wv, int lane) {
+  const int l32 = lane & 31;
+  const int kq = (lane >> 5) * 8;
+  lds_half_t *pxb = lds_opaque(sIn + (wv * RPW * HALO_W + l32) * CKP + kq);
+  constexpr int NG = 3 * (L / 16);
+  half8 px[2][PXROWS];
+  auto load = [&](int g) {
+    const int s = g / (L / 16), ks = g % (L / 16);
+#pragma unroll
+    for (int hr = 0; hr < PXROWS; ++hr)
+      px[g & 1][hr] = *reinterpret_cast<lds_half8_t *>(pxb + (hr * HALO_W + s) * CKP + ks * 16);
+  };
+  load(0);
+#pragma unroll
+  for (int g = 0; g < NG; ++g) {
+    const int s = g / (L / 16), ks = g % (L / 16);
+    if (g + 1 < NG)
+      load(g + 1);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+      for (int j = 0; j < RPW; ++j)
+        acc.v[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw.w[r * 3 + s][CHUNK * (CK / 16) + ks], px[g & 1][j + r], acc.v[0][j], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+// chunk `cchunk` of a step, found by comparison: the register file is indexed by constants only
+template <int C>
+__device__ DNX_INLINE void mma_first_reg_chunk(int cchunk, const _Float16 *sIn, const FirstWeights &fw, Acc &acc, int wv, int lane) {
+  if constexpr (C < NCHUNK) {
+    if (cchunk == C)
+      mma_first_reg<(TAIL == CK || C < NCHUNK - 1) ? CK : TAIL, C>(sIn, fw, acc, wv, lane);
+    else
+      mma_first_reg_chunk<C + 1>(cchunk, sIn, fw, acc, wv, lane);
+  }
+}
+#endif
+
 // Stores the step's outputs: rows ob + wave * RPW + r, columns xs + (lane & 31); only the SWO inner columns and the
 // rows in [ylo, yhi) belong to this step (the rest is another step's, or garbage).
 __device__ DNX_INLINE void
@@ -303,7 +369,9 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     const _Float16 *__restrict__ BIAS2,
 #endif
     PushConstants pc) {
+#if !W1REG
   __shared__ __attribute__((aligned(16))) _Float16 sW1[NTAPS * 32 * CPADP];
+#endif
   __shared__ __attribute__((aligned(16))) _Float16 sIn[2][HALO_PIX * CKP];
   __shared__ __attribute__((aligned(16))) _Float16 sMid[(NS * IW + 2) * C2P];
   __shared__ __attribute__((aligned(16))) bias_t sBias1[32];
@@ -348,6 +416,12 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
 #if HAS_BIAS
   for (int i = tid; i < 32; i += NT) sBias2[i] = (float)BIAS2[i];
 #endif
+#if W1REG
+  static_assert(PW > 0, "weights in registers: computing waves that hold nothing else");
+  FirstWeights w1;
+  if (wv < WAVES)
+    load_first_weights(w1, FILT1, lane);
+#else
   {
     constexpr int VPR = CPAD / 8; // global [tap][32 rows][CPAD] -> LDS rows of CPADP
     for (int i = tid; i < NTAPS * 32 * VPR; i += NT) {
@@ -355,23 +429,23 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
       *reinterpret_cast<uint4v *>(sW1 + row * CPADP + v * 8) = ld16(FILT1 + (size_t)i * 8);
     }
   }
+#endif
   SecondWeights w2;
   load_second_weights(w2, FILT2, lane);
 
   // ---- the fetch cursor walks the same sequence of (unit, step, channel chunk) as the compute cursor, two chunks ahead.
   // Every unit has one step more than it has rows for: the last one only drains the second convolution, its loads are
   // aimed past the end of the sources (they return zeros without touching memory) and its matrix work is skipped. ----
-  typedef Halo<NT> H;
+  typedef Halo<(PW > 0 ? PW : WAVES) * 64> H;
   H::Map map;
   H::Src fsrc;
-  H::map_init(map, tid);
+  H::map_init(map, PW > 0 ? tid - WAVES * 64 : tid); // (computing waves of the specialised variant never use it)
   Geo fg = geometry(unit);
   int funit = unit, fk = 0, fchunk = 0;
   auto aim = [&]() { // source offsets of the fetch cursor's step; a drain step (or none) reads nothing
     const bool real = funit < units && fk < fg.steps;
     H::src_init(fsrc, map, real ? fg.ys - 1 + fk * IH : -0x10000, fg.xs - 1, pc);
   };
-  aim();
   // Past the last step the cursor stays where it is: the loads are issued all the same (and never used), so that the
   // number of loads in flight is the same on every path through the loop.
   auto issue = [&](H::Regs &regs) {
@@ -392,11 +466,8 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   int k = 0, cchunk = 0, buf = 0;
   int wslot = 0; // ring row that takes the first `mid` row of step k
   Acc acc;       // the first convolution's accumulators during a step's chunks, the second's in between
-  auto step = [&](H::Regs &regs) {
-    H::commit_step(regs, sIn[buf], map, cchunk);
-    // One barrier per chunk: buffer `buf` was last read two chunks ago, and every wave has passed the barrier of the
-    // chunk in between since then.  The first barrier of a step also publishes the `mid` rows the previous step wrote.
-    DNX_SYNC();
+  // what the computing side does in one chunk, after the barrier that published the chunk's halo
+  auto compute = [&]() {
     const bool alive = unit < units; // false in a spare chunk behind the last step
     if (cchunk == 0) {
       if (alive && k > 0) { // outputs of step k - 1: its `mid` rows and the two before them are in the ring
@@ -415,13 +486,19 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
       }
       init_acc_first(acc, sBias1, lane);
     }
-    issue(regs); // refill this register set: the chunk after next
+  };
+  auto multiply = [&]() {
+    const bool alive = unit < units;
     const bool real = alive && k < g.steps;
     if (real) {
+#if W1REG
+      mma_first_reg_chunk<0>(cchunk, sIn[buf], w1, acc, wv, lane);
+#else
       if (TAIL == CK || cchunk < NCHUNK - 1)
         mma_first<CK, CPADP>(sIn[buf], sW1, cchunk * CK, acc, wv, lane);
       else
         mma_first<TAIL, CPADP>(sIn[buf], sW1, cchunk * CK, acc, wv, lane);
+#endif
     }
     buf ^= 1;
     if (++cchunk == NCHUNK) {
@@ -439,6 +516,17 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
       }
     }
   };
+#if PW == 0
+  auto step = [&](H::Regs &regs) {
+    H::commit_step(regs, sIn[buf], map, cchunk);
+    // One barrier per chunk: buffer `buf` was last read two chunks ago, and every wave has passed the barrier of the
+    // chunk in between since then.  The first barrier of a step also publishes the `mid` rows the previous step wrote.
+    DNX_SYNC();
+    compute();
+    issue(regs); // refill this register set: the chunk after next
+    multiply();
+  };
+  aim();
   H::Regs st0, st1;
   issue(st0);
   __builtin_amdgcn_sched_barrier(0); // keep the two sets in issue order: the waits count loads in flight
@@ -449,4 +537,47 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     step(st0);
     step(st1);
   } while (unit < units);
+#else
+  // chunks this workgroup runs: both roles execute exactly one barrier per chunk
+  int chunks = 0;
+  for (int u = unit; u < units; u += GRID)
+    chunks += (geometry(u).steps + 1) * NCHUNK;
+  if (wv >= WAVES) {
+    // ---- staging waves: chunk c's halo is written to sIn[c & 1] during chunk c - 1 ----
+    aim();
+    H::Regs st0, st1;
+    int commitChunk = 0; // channel chunk of the halo being written
+    auto commit = [&](H::Regs &regs, int c) {
+      H::commit_step(regs, sIn[c & 1], map, commitChunk);
+      if (++commitChunk == NCHUNK)
+        commitChunk = 0;
+    };
+    issue(st0);   // chunk 0
+    __builtin_amdgcn_sched_barrier(0);
+    issue(st1);   // chunk 1
+    commit(st0, 0);
+    issue(st0);   // chunk 2
+    for (int c = 0; c < chunks; c += 2) {
+      DNX_SYNC(); // chunk c starts: sIn[c & 1] is complete, the other buffer is free
+      if (c + 1 < chunks) {
+        commit(st1, c + 1);
+        issue(st1); // chunk c + 3
+      }
+      if (c + 1 >= chunks)
+        break;
+      DNX_SYNC(); // chunk c + 1 starts
+      if (c + 2 < chunks) {
+        commit(st0, c + 2);
+        issue(st0); // chunk c + 4
+      }
+    }
+  } else {
+    // ---- computing waves ----
+    for (int c = 0; c < chunks; ++c) {
+      DNX_SYNC();
+      compute();
+      multiply();
+    }
+  }
+#endif
 }

@@ -12,7 +12,7 @@ from util import assert_bits_equal, assert_conv_close, fill_lds_with_nans, he_we
 
 pytestmark = pytest.mark.gpu
 
-PAIR_CONFIGS = ["x8r2k16", "x4r4k16", "x4r2k16", "x4r2k32"]
+PAIR_CONFIGS = ["x8r2k16", "x4r4k16", "x4r2k16", "x4r2k32", "y4r2k32", "z4r2k64"]
 
 
 def build(rng, C, K1, K2, tail, pad=False, act1=True, bias=True):
@@ -104,20 +104,21 @@ def integer_pair(x, K1, K2):
     return np.repeat(out[:, :, None], K2, axis=2)
 
 
+@pytest.mark.parametrize("config,C,density", [("x8r2k16", 8, 0.15), ("y4r2k32", 32, 0.04), ("z4r2k64", 64, 0.02)])
 @pytest.mark.parametrize("H,W", [(33, 47), (288, 31), (1080, 1920)])
-def test_pair_exact_on_small_integers(H, W):
+def test_pair_exact_on_small_integers(H, W, config, C, density):
     """Inputs in {0, 1}, all weights one: every intermediate and final value is an integer below 2048, which binary16
     holds exactly, so the fused kernel must reproduce integer arithmetic bit for bit -- at every strip and segment
     border of the benchmark's frame as well."""
     rng = np.random.default_rng(H)
-    C, K1, K2 = 8, 2, 3
-    x = (rng.random((H, W, C)) < 0.15).astype(np.float16)
+    K1, K2 = 2, 3
+    x = (rng.random((H, W, C)) < density).astype(np.float16)
     m = dx.Model()
     y = m.conv2d(m.input("input", "W", "H", C), np.ones((K1, C, 3, 3), np.float16))
     z = m.conv2d(y, np.ones((K2, K1, 3, 3), np.float16))
     m.output(z)
-    mod = dx.Module.compile(m, conv_config="x8r2k16", assume={"H": H, "W": W})
-    assert any(e.startswith("convpair_") for e in entry_points(mod, H=H, W=W))
+    mod = dx.Module.compile(m, conv_config=config, assume={"H": H, "W": W})
+    assert any(e.startswith("convpair_") and e.endswith(config) for e in entry_points(mod, H=H, W=W))
     want = integer_pair(x, K1, K2)
     assert want.max() < 2048
     fill_lds_with_nans()
