@@ -883,6 +883,13 @@ Sym rowBlocks(SymGraph &sym, Sym rows, unsigned rpt) { return rpt == 1 ? rows : 
 Sym rowGrid(SymGraph &sym, Sym w, unsigned vectorsPerPixel) {
   return sym.cdiv(sym.mul(w, static_cast<int64_t>(vectorsPerPixel)), WG_BANDWIDTH);
 }
+// FLAT mode of activation / pad / slice (kernels/common.h): a row is moved as w * channels / 8 + 1 aligned 16-byte vectors; the
+// grid also covers the pixel-by-pixel path of the same kernel (pad with columns added)
+Sym rowGridFlat(SymGraph &sym, Sym w, unsigned channels, unsigned vectorsPerPixel) {
+  const Sym flat = sym.add(sym.cdiv(sym.mul(w, static_cast<int64_t>(channels)), 8), 1);
+  const Sym general = sym.mul(w, static_cast<int64_t>(vectorsPerPixel));
+  return sym.cdiv(sym.max(flat, general), WG_BANDWIDTH);
+}
 
 class SingleOpShader : public IShader {
 public:
@@ -939,6 +946,9 @@ public:
     if (p.planes) { k.define("PLANAR", 1); k.define("CH", 8); } // (overrides the channel count defined before)
   }
   static unsigned kernelChannels(const Placement &p, unsigned channels) { return p.planes ? 8 : channels; }
+  // rows moved as runs of halves (FLAT in kernels/common.h): any channel count that is not moved in aligned vectors anyway,
+  // into a tensor of its own (inside a concat's wider tensor the rows are not contiguous)
+  static bool isFlat(const Placement &p) { return p.vec == 1 && !p.view.valid && !p.planes; }
   static Sym gridZ(const Placement &p) { return Sym::Const(p.planes ? p.planes : 1); }
   static void bindOutput(ComputeDispatchBuilder &d, SymGraph &sym, const Model &model, const Match &m, const Placement &p) {
     if (!p.view.valid) { d.addBinding(dnx::Access::WriteOnly, m.output); return; }
@@ -1119,14 +1129,16 @@ public:
     k.define("CH", in.channels); k.define("VEC", vec); k.define("ACT", op.func == ActivationFunction::ReLU ? 1 : 2);
     if (op.func == ActivationFunction::LeakyReLU) k.define("ALPHA", fmtFloat(op.alpha));
     defineOutput(k, place);
-    const std::string entry = std::string(op.func == ActivationFunction::ReLU ? "relu_c" : "leaky_relu_c") + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
+    const bool flat = isFlat(place);
+    if (flat) k.define("FLAT", 1);
+    const std::string entry = std::string(op.func == ActivationFunction::ReLU ? "relu_c" : "leaky_relu_c") + std::to_string(in.channels) + "v" + std::to_string(vec) + (flat ? "f" : "") + place.suffix;
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, rowGrid(sym, in.width, chunksPerPixel(kernelChannels(place, in.channels), vec)), in.height, gridZ(place), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, flat ? rowGridFlat(sym, in.width, in.channels, 0) : rowGrid(sym, in.width, chunksPerPixel(kernelChannels(place, in.channels), vec)), in.height, gridZ(place), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     bindOutput(d, sym, model, m, place);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
     const char *nm = op.func == ActivationFunction::ReLU ? "relu" : "leaky_relu";
-    d.setName(std::string(nm) + (place.view.valid ? "+concat" : "")); d.setOperation(nm); d.setConfig("vec" + std::to_string(vec) + (place.planes ? "/chwc8" : ""));
+    d.setName(std::string(nm) + (place.view.valid ? "+concat" : "")); d.setOperation(nm); d.setConfig("vec" + std::to_string(vec) + (flat ? "/rows" : "") + (place.planes ? "/chwc8" : ""));
     if (place.planes) impl.edge().config = "chwc8";
     d.setMemoryReads(bytesOf(sym, in)); d.setMemoryWrites(bytesOf(sym, in));
     d.setFlops(sym.mul(sym.mul(in.width, in.height), static_cast<int64_t>(in.channels))); // one FLOP per element, as the reference counts it
@@ -1147,14 +1159,16 @@ public:
     const bool zeros = op.padMode == PaddingMode::Zero;
     if (zeros) k.define("ZERO", 1);
     defineOutput(k, place);
-    const std::string entry = std::string(zeros ? "memory_pad_zero_c" : "memory_pad_c") + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
+    const bool flat = isFlat(place);
+    if (flat) k.define("FLAT", 1);
+    const std::string entry = std::string(zeros ? "memory_pad_zero_c" : "memory_pad_c") + std::to_string(in.channels) + "v" + std::to_string(vec) + (flat ? "f" : "") + place.suffix;
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, chunksPerPixel(in.channels, vec)), out.height, Sym::Const(1), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, flat ? rowGridFlat(sym, out.width, in.channels, chunksPerPixel(in.channels, vec)) : rowGrid(sym, out.width, chunksPerPixel(in.channels, vec)), out.height, Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     bindOutput(d, sym, model, m, place);
     d.addPushConstant(out.width); d.addPushConstant(out.height);
     d.addPushConstant(op.left); d.addPushConstant(op.right); d.addPushConstant(op.top); d.addPushConstant(op.bottom);
-    d.setName(std::string("pad") + (place.view.valid ? "+concat" : "")); d.setOperation("pad"); d.setConfig("vec" + std::to_string(vec));
+    d.setName(std::string("pad") + (place.view.valid ? "+concat" : "")); d.setOperation("pad"); d.setConfig("vec" + std::to_string(vec) + (flat ? "/rows" : ""));
     d.setMemoryReads(bytesOf(sym, in)); d.setMemoryWrites(bytesOf(sym, out)); d.setFlops(Sym::Const(0));
   }
 };
@@ -1171,15 +1185,17 @@ public:
     auto k = m_compiler->read("slice.hip");
     k.define("CH", in.channels); k.define("VEC", vec);
     defineOutput(k, place);
-    const std::string entry = "memory_slice_c" + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
+    const bool flat = isFlat(place);
+    if (flat) k.define("FLAT", 1);
+    const std::string entry = "memory_slice_c" + std::to_string(in.channels) + "v" + std::to_string(vec) + (flat ? "f" : "") + place.suffix;
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, chunksPerPixel(in.channels, vec)), out.height, Sym::Const(1), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, flat ? rowGridFlat(sym, out.width, in.channels, 0) : rowGrid(sym, out.width, chunksPerPixel(in.channels, vec)), out.height, Sym::Const(1), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     bindOutput(d, sym, model, m, place);
     d.addPushConstant(op.top); d.addPushConstant(op.left);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
     d.addPushConstant(out.width); d.addPushConstant(out.height);
-    d.setName(std::string("slice") + (place.view.valid ? "+concat" : "")); d.setOperation("slice"); d.setConfig("vec" + std::to_string(vec));
+    d.setName(std::string("slice") + (place.view.valid ? "+concat" : "")); d.setOperation("slice"); d.setConfig("vec" + std::to_string(vec) + (flat ? "/rows" : ""));
     d.setMemoryReads(bytesOf(sym, out)); d.setMemoryWrites(bytesOf(sym, out)); d.setFlops(Sym::Const(0));
   }
 };

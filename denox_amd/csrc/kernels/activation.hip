@@ -1,7 +1,7 @@
 // activation.hip -- stand-alone elementwise activation in binary16.
 // Replaces compiler/src/denox/compiler/implement/shaders/activation/basic_activation.comp:26-184:
 //   ReLU: max(v, 0);  LeakyReLU: max(v, alpha * v) with alpha and the product in binary16.
-// Definitions: CH, ACT (1 ReLU, 2 LeakyReLU), ALPHA, VEC.  grid.y = rows.
+// Definitions: CH, ACT (1 ReLU, 2 LeakyReLU), ALPHA, VEC; FLAT: rows moved as runs of halves (common.h).  grid.y = rows.
 #include "common.h"
 #ifndef ALPHA
 #define ALPHA 0.0f
@@ -26,6 +26,18 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(WG) void KERNEL_NAME(
   OUT += (size_t)DNX_BID_Z * pc.W * pc.H * 8;
 #endif
   const unsigned i = DNX_ROW_INDEX();
+#ifdef FLAT
+  {
+    const size_t row = (size_t)DNX_BID_Y * pc.W * CH;
+    flat_row(IN + row, OUT + row, pc.W * CH, i, [](vec_t v) {
+      half8 a = __builtin_bit_cast(half8, v);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) a[e] = act1(a[e]);
+      return __builtin_bit_cast(vec_t, a);
+    });
+    return;
+  }
+#endif
   if (i >= pc.W * CV) return;
   const unsigned w = i / CV, cv = i - w * CV;
   const size_t pix = (size_t)DNX_BID_Y * pc.W + w;

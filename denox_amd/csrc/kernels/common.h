@@ -107,5 +107,32 @@ __device__ DNX_INLINE vec_t max_keep_first(vec_t acc, vec_t v) {
   return __builtin_bit_cast(uint4v, a);
 }
 
+// FLAT (activation, pad, slice with VEC = 1 and a result that is a tensor of its own): a row of W pixels of any channel
+// count is one run of W * CH consecutive halves in both tensors, so the row is moved as such a run instead of pixel by
+// pixel.  Thread i stores the i-th 16-byte ALIGNED vector of the destination run -- whole cache lines from consecutive
+// lanes, no 2-, 4- or 8-byte pieces -- and loads the 8 halves that belong there with one 16-byte load at whatever 2-byte
+// alignment the source has.  The first and the last vector of a run may reach into the neighbouring rows: those two are
+// moved element by element, inside the run only.  The grid covers W * CH / 8 + 1 vectors per row.
+// F maps a vector of 8 halves (identity for the copies).
+template <typename F>
+__device__ DNX_INLINE void flat_row(const ushort_t *__restrict__ src, ushort_t *__restrict__ dst, unsigned n, unsigned i, F f) {
+  const unsigned a = (unsigned)(((size_t)dst >> 1) & 7u); // halves between the previous 16-byte boundary and the run's start
+  const int e0 = (int)(i * 8u) - (int)a;                   // first half of this thread's vector, relative to the run
+  if (e0 >= (int)n)
+    return;
+  if (e0 >= 0 && e0 + 8 <= (int)n) {
+    const vec_t v = *reinterpret_cast<const uint4u *>(src + e0);
+    *reinterpret_cast<uint4v *>(dst + e0) = f(v);
+  } else {
+    const int lo = e0 < 0 ? 0 : e0, hi = e0 + 8 < (int)n ? e0 + 8 : (int)n;
+    for (int e = lo; e < hi; ++e) {
+      vec_t v = {};
+      v[0] = src[e];
+      dst[e] = (ushort_t)f(v)[0];
+    }
+  }
+}
+#define DNX_FLAT_VECTORS(w) (((w) * CH + 7u) / 8u + 1u) // vectors a row's grid must cover
+
 // position of this thread inside its row: vector index `i` in [0, rowVectors)
 #define DNX_ROW_INDEX() (DNX_BID_X * WG + (unsigned)DNX_TID)

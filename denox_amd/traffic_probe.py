@@ -3,8 +3,9 @@
 Two steps:
 
 `python3 -m denox_amd.traffic_probe run <map.json> [H W]` compiles the OIDN U-Net once per candidate configuration of its
-most expensive layer (dec_conv1a: concat + replicate pad + 2x upsample + conv 73 -> 64 + ReLU), steering the selection to
-that candidate through a timing table that holds one made-up sample for it, runs every such schedule a few times, runs the
+three longest dispatches (dec_conv1a: concat + replicate pad + 2x upsample + conv 73 -> 64 + ReLU, and the two conv -> conv
+dispatches at the network's ends), steering the selection to those candidates through a timing table that holds made-up
+samples for them, runs every such schedule a few times, runs the
 plain copy kernel of `denox_amd.calibrate`, and writes which entry point belongs to which code object.  Run it under
 `rocprofv3 --pmc FETCH_SIZE` and again under `rocprofv3 --pmc WRITE_SIZE` (counters per dispatch, csv).
 
@@ -21,9 +22,14 @@ import tempfile
 
 import numpy as np
 
-# Candidates of the dominant layer that the timing table has been seen to select, in both result layouts
-CANDIDATES = ["g4r1n", "g4r1k32n", "g4r1", "g4r1k32", "s8r2k16", "s8r2k16/hwc>chwc8", "s12r1k16", "s12r1k16/hwc>chwc8", "t8r2k16", "p8r2k16", "f8r1"]
-DOMINANT_OPERATION = "concat+pad+upsample+conv3x3+relu"
+DOMINANT_OPERATION = "concat+pad+upsample+conv3x3+relu"   # dec_conv1a with everything folded into its loader
+LAST_PAIR = "conv3x3+relu+conv3x3+slice"                   # dec_conv1b -> dec_conv0 -> crop in one dispatch
+FIRST_PAIR = "pad+conv3x3+relu+conv3x3+relu+maxpool"       # enc_conv0 -> enc_conv1 -> pool in one dispatch
+# Schedules to run: {operation: configuration} pairs that the selection is steered to.  The candidates of the three
+# longest dispatches that the timing table has been seen to select, in the layouts it combines them in.
+STEER = ([{DOMINANT_OPERATION: c} for c in ("g4r1n", "g4r1k32n", "g4r1", "g4r1k32", "s8r2k16", "s12r1k16", "t8r2k16", "p8r2k16", "f8r1")] +
+         [{DOMINANT_OPERATION: "g4r1n", LAST_PAIR: c, FIRST_PAIR: "x8r2k16/hwc>chwc8"} for c in ("z4r2k64", "y4r2k32", "x8r2k16")] +
+         [{DOMINANT_OPERATION: d + "/hwc>chwc8", LAST_PAIR: c + "/chwc8>hwc"} for d, c in (("s8r2k16", "z4r2k64"), ("s12r1k16", "y4r2k32"), ("s8r2k16", "x8r2k16"))])
 COPY_KERNEL = "memory_slice_c64v8"
 
 
@@ -39,22 +45,19 @@ def run(map_path, H=1080, W=1920, frames=6):
     x = networks.synthetic_input("oidn_unet", H, W, seed=0)
     kernels = {}
     tmp = tempfile.mkdtemp(prefix="denox_hip_probe_")
-    for cand in CANDIDATES:
-        db = dx.Db(os.path.join(tmp, cand.replace("/", "_").replace(">", "_") + ".db"))
+    for n, steer in enumerate(STEER):
+        db = dx.Db(os.path.join(tmp, f"steer{n}.db"))
         db.populate(model, assume={"H": H, "W": W})
         rows = [r.split('","') for r in db.dump_csv().splitlines()[1:]]
-        hits = [i for i, r in enumerate(rows) if r[0].strip('"') == DOMINANT_OPERATION and _norm(r[2]) == cand]
-        if not hits:
-            print(f"traffic_probe: no candidate '{cand}' for {DOMINANT_OPERATION}", file=sys.stderr)
-            continue
+        hits = [i for i, r in enumerate(rows) if steer.get(r[0].strip('"')) == _norm(r[2])]
         for i in hits:
             for _ in range(3):
                 db.add_sample(i, 1000.0)  # 1 us: below every estimate, so the selection takes this candidate
         blob = dx.compile_model(model, assume={"H": H, "W": W}, db=db)
         desc = dx.describe(blob, H=H, W=W)["dispatches"]
-        dom = [d for d in desc if d["name"] == DOMINANT_OPERATION]
-        if len(dom) != 1 or _norm(dom[0]["debug_info"].split(" | ")[0]) != cand:
-            print(f"traffic_probe: the schedule did not take '{cand}': {[d['debug_info'].split(' | ')[0] for d in dom]}", file=sys.stderr)
+        taken = {d["name"]: _norm(d["debug_info"].split(" | ")[0]) for d in desc}
+        if any(taken.get(op) != cfg for op, cfg in steer.items()):
+            print(f"traffic_probe: the schedule did not follow {steer}: {taken}", file=sys.stderr)
             continue
         inst = dx.Module.load(blob).instance(H=H, W=W)
         inst.infer(x)
@@ -101,7 +104,7 @@ def summarize(map_path, fetch_csv, write_csv):
     for entry, k in sorted(m["kernels"].items()):
         # the dominant layer's candidates and the two conv -> conv dispatches: kernels that run at one extent only
         # (a name like conv3x3_c96_k96_relu_* serves two layers of different size; a mean over both describes neither)
-        if entry not in fetch or entry not in write or not (k["operation"] == m["dominant_operation"] or entry.startswith("convpair_")):
+        if entry not in fetch or entry not in write or k["operation"] not in (DOMINANT_OPERATION, LAST_PAIR, FIRST_PAIR):
             continue
         f_, w_ = fetch[entry], write[entry]
         fb, wb = float(np.mean(f_[1:] if len(f_) > 1 else f_)) * fscale, float(np.mean(w_[1:] if len(w_) > 1 else w_)) * wscale
