@@ -1006,13 +1006,16 @@ public:
     auto k = m_compiler->read("upsample.hip");
     k.define("CH", in.channels); k.define("SCALE", op.scale); k.define("VEC", vec);
     defineOutput(k, place);
-    const std::string entry = "upsample_c" + std::to_string(in.channels) + "v" + std::to_string(vec) + place.suffix;
+    // rows moved as runs of aligned vectors (kernels/upsample.hip): at most one pixel boundary per vector
+    const bool flat = isFlat(place) && in.channels >= 8;
+    if (flat) k.define("FLAT", 1);
+    const std::string entry = "upsample_c" + std::to_string(in.channels) + "v" + std::to_string(vec) + (flat ? "f" : "") + place.suffix;
     k.define("KERNEL_NAME", entry);
-    auto d = impl.registerDispatch(k, entry, rowGrid(sym, out.width, chunksPerPixel(kernelChannels(place, in.channels), vec)), in.height, gridZ(place), WG_BANDWIDTH);
+    auto d = impl.registerDispatch(k, entry, flat ? rowGridFlat(sym, out.width, in.channels, 0) : rowGrid(sym, out.width, chunksPerPixel(kernelChannels(place, in.channels), vec)), in.height, gridZ(place), WG_BANDWIDTH);
     d.addBinding(dnx::Access::ReadOnly, m.inputs[0]);
     bindOutput(d, sym, model, m, place);
     d.addPushConstant(in.width); d.addPushConstant(in.height);
-    d.setName(std::string("upsample") + (place.view.valid ? "+concat" : "")); d.setOperation("upsample"); d.setConfig("vec" + std::to_string(vec) + (place.planes ? "/chwc8" : ""));
+    d.setName(std::string("upsample") + (place.view.valid ? "+concat" : "")); d.setOperation("upsample"); d.setConfig("vec" + std::to_string(vec) + (flat ? "/rows" : "") + (place.planes ? "/chwc8" : ""));
     if (place.planes) impl.edge().config = "chwc8";
     d.setMemoryReads(bytesOf(sym, in)); d.setMemoryWrites(bytesOf(sym, out)); d.setFlops(Sym::Const(0));
   }

@@ -586,6 +586,34 @@ def test_every_channel_remainder(oracle, C):
         assert_bits_equal(g, want[t.name], f"C={C} {t.name}")
 
 
+@pytest.mark.parametrize("H,W,C", [(7, 24, 9), (6, 25, 9), (5, 32, 73), (9, 31, 73), (4, 16, 12), (3, 5, 15), (1, 1, 9), (2, 3, 11), (33, 130, 10)])
+def test_rows_moved_as_runs_of_aligned_vectors(H, W, C):
+    """Channel counts that are not multiples of 8: activation, pad, slice and upsample move a row as one run of halves in
+    aligned 16-byte vectors (the first and last vector of a run element by element, an upsampled vector from one or two
+    source pieces).  Extents whose runs start at every offset from a 16-byte boundary, runs shorter than a vector, rows
+    whose replicas share an alignment and rows that do not; checked against numpy, bit for bit."""
+    rng = np.random.default_rng(H * 1000 + W * 10 + C)
+    x = rng.standard_normal((H, W, C)).astype(np.float16)
+    m = dx.Model()
+    inp = m.input("input", "W", "H", C)
+    outs = [m.relu(inp), m.pad(inp, 0, 0, 2, 3), m.pad(inp, 0, 0, 1, 0, mode="zero"), m.pad(inp, 1, 2, 0, 1), m.slice(inp, 0, "W", 0, m.sym("H") - 0),
+            m.upsample(inp)]
+    if H > 2 and W > 2:
+        outs += [m.slice(inp, 0, "W", 1, m.sym("H") - 1), m.slice(inp, 1, m.sym("W") - 1, 1, "H")]
+    for t in outs:
+        m.output(t)
+    mod = dx.Module.compile(m)
+    names = [d_["entry_point"] for d_ in dx.describe(mod.dnx, H=H, W=W)["dispatches"]]
+    assert all(n.endswith("f") for n in names), names
+    got = mod.instance(H=H, W=W).infer(x)
+    want = [np.maximum(x, np.float16(0)), np.pad(x, ((2, 3), (0, 0), (0, 0)), mode="edge"), np.pad(x, ((1, 0), (0, 0), (0, 0))),
+            np.pad(x, ((0, 1), (1, 2), (0, 0)), mode="edge"), x, np.repeat(np.repeat(x, 2, 0), 2, 1)]
+    if H > 2 and W > 2:
+        want += [x[1:H - 1], x[1:, 1:W - 1]]
+    for t, g, w in zip(outs, got, want):
+        assert_bits_equal(g, w, f"{t.name} {H}x{W}x{C}")
+
+
 @pytest.mark.parametrize("CA,CB", [(3, 3), (9, 64), (64, 9), (8, 8), (12, 20), (73, 7), (16, 24), (1, 1), (5, 17)])
 def test_concat_copy_of_two_sources(oracle, CA, CB):
     """Both sources copied by one launch that writes whole pixels (model inputs cannot be written in place, so neither source
