@@ -66,7 +66,7 @@ ALL_CONFIGS += OSTAGE_CONFIGS
 EVERY_CONFIG_SHAPES = [(80, 64, 45, 70), (73, 96, 130, 300), (16, 32, 300, 530)]
 FOLD_CONFIGS = ["f8r1", "f4r2", "f4r1", "g4r1", "g4r1k32", "g4r1n", "g4r1k32n"]
 FOLD_SHAPES = [(64, 9, 64, 36, 70, False), (16, 0, 32, 18, 34, False), (32, 24, 40, 62, 130, False), (8, 3, 3, 2, 2, False), (24, 9, 16, 40, 52, True),
-               (96, 32, 64, 34, 66, False), (32, 16, 32, 50, 70, True), (48, 12, 96, 22, 134, False), (64, 8, 64, 2, 2, False), (16, 9, 32, 8, 64, False)]
+               (96, 32, 64, 34, 66, False), (32, 16, 32, 50, 70, True), (48, 12, 96, 22, 134, False), (64, 8, 64, 2, 2, False), (16, 9, 32, 8, 64, False), (128, 9, 128, 20, 70, True)]
 STRIDED_ONLY_CONFIGS = ["m2r1k32x1n", "w2r2k16n", "w2r1k16n"]  # offered to strided layers only
 
 
