@@ -339,6 +339,7 @@ int denox_hip_dnx_describe(const void *dnxbuf, size_t size, const char *const *n
         if (vn.name == names[i] && vn.value.symbolic && static_cast<uint64_t>(vn.value.value) < vars.size()) vars[static_cast<size_t>(vn.value.value)] = values[i];
     }
     const std::vector<int64_t> dp = m.sym_ir.eval(vars);
+    if (n > 0) m.checkRequirements(dp); // (without extents every variable reads as zero: a listing, not an evaluation)
     std::ostringstream o;
     o << "{\"producer\":"; jsonEscape(o, m.info.producer);
     o << ",\"var_count\":" << m.sym_ir.varCount << ",\"sym_ops\":" << m.sym_ir.ops.size();

@@ -26,7 +26,8 @@ enum ModelInfo { MI_producer = 0, MI_producer_version = 1, MI_model_version = 2 
 enum ValueName { VN_name = 0, VN_value_type = 1, VN_value = 2 };                  // dnx.fbs:164-167
 enum ShaderBinary { SB_spirv = 0, SB_code_object = 1 };                           // dnx.fbs:169-171 + code object
 enum Model { M_version = 0, M_required_features = 1, M_info = 2, M_tensors = 3, M_initializers = 4, M_inputs = 5, M_outputs = 6, M_buffers = 7, M_dispatches = 8,
-             M_shader_binaries = 9, M_sym_ir = 10, M_value_names = 11 };          // dnx.fbs:173-192
+             M_shader_binaries = 9, M_sym_ir = 10, M_value_names = 11, M_requirements = 12 }; // dnx.fbs:173-192 + requirements
+enum Requirement { RQ_lhs_type = 0, RQ_lhs = 1, RQ_rhs_type = 2, RQ_rhs = 3, RQ_relation = 4, RQ_what = 5 }; // (not in dnx.fbs)
 } // namespace id
 constexpr uint8_t SRC_NONE = 0, SRC_LITERAL = 1, SRC_SYMBOLIC = 2;                // union ScalarSource, dnx.fbs:27-30
 constexpr char IDENTIFIER[4] = {'d', 'n', 'x', 'x'};                               // dnx.fbs:4
@@ -110,6 +111,16 @@ std::vector<uint8_t> serialize(const Model &m) {
     b.startTable(3);
     b.addOffset(id::VN_name, name);
     w.addSource(id::VN_value_type, v.value, val);
+    return b.endTable();
+  });
+
+  const fb::Off requirements = w.tables(m.requirements, [&](const Requirement &q) {
+    const fb::Off what = b.createString(q.what), lhs = w.source(q.lhs), rhs = w.source(q.rhs);
+    b.startTable(6);
+    w.addSource(id::RQ_lhs_type, q.lhs, lhs);
+    w.addSource(id::RQ_rhs_type, q.rhs, rhs);
+    b.addScalar<uint8_t>(id::RQ_relation, q.relation, 0);
+    b.addOffset(id::RQ_what, what);
     return b.endTable();
   });
 
@@ -238,7 +249,7 @@ std::vector<uint8_t> serialize(const Model &m) {
   const fb::Off info = b.endTable();
   const fb::Off features = b.createVector(m.required_features.data(), 4, 4, m.required_features.size());
 
-  b.startTable(12);
+  b.startTable(13);
   b.addScalar<uint16_t>(id::M_version, m.version, 0);
   b.addOffset(id::M_required_features, features);
   b.addOffset(id::M_info, info);
@@ -251,7 +262,16 @@ std::vector<uint8_t> serialize(const Model &m) {
   b.addOffset(id::M_shader_binaries, binaries);
   b.addOffset(id::M_sym_ir, symIr);
   b.addOffset(id::M_value_names, valueNames);
+  if (!m.requirements.empty()) b.addOffset(id::M_requirements, requirements);
   return b.finish(b.endTable(), IDENTIFIER);
+}
+
+void Model::checkRequirements(const std::vector<int64_t> &dp) const {
+  for (const auto &q : requirements) {
+    const int64_t a = q.lhs.eval(dp), b = q.rhs.eval(dp);
+    if (q.relation == 0 ? a != b : a > b)
+      fail(Status::InvalidArgument, q.what + ": " + std::to_string(a) + (q.relation == 0 ? " != " : " > ") + std::to_string(b) + " at these extents");
+  }
 }
 
 Model deserialize(const void *data, size_t size) {
@@ -287,6 +307,16 @@ Model deserialize(const void *data, size_t size) {
     const fb::Table t = valueNames.table(i);
     m.value_names[i].name = t.str(id::VN_name);
     m.value_names[i].value = r.source(t, id::VN_value_type);
+  }
+
+  const fb::Vector requirements = root.vector(id::M_requirements, 4, 4);
+  m.requirements.resize(requirements.size());
+  for (uint32_t i = 0; i < requirements.size(); ++i) {
+    const fb::Table t = requirements.table(i);
+    m.requirements[i].lhs = r.source(t, id::RQ_lhs_type);
+    m.requirements[i].rhs = r.source(t, id::RQ_rhs_type);
+    m.requirements[i].relation = t.scalar<uint8_t>(id::RQ_relation, 0);
+    m.requirements[i].what = t.str(id::RQ_what);
   }
 
   const fb::Vector buffers = root.vector(id::M_buffers, 4, 4);
@@ -418,6 +448,11 @@ void validate(const Model &m) {
     if (!(o.opcode & SYM_RHSC) && (o.rhs < 0 || static_cast<size_t>(o.rhs) >= lim)) fail(Status::InvalidModel, "SymIR forward reference");
   }
   for (const auto &v : m.value_names) chk(v.value);
+  for (const auto &q : m.requirements) {
+    chk(q.lhs);
+    chk(q.rhs);
+    if (q.relation > 1) fail(Status::InvalidModel, "dnx: unknown relation in a requirement");
+  }
   for (const auto &b : m.buffers) { chk(b.size); if (b.alignment == 0) fail(Status::InvalidModel, "zero buffer alignment"); }
   for (const auto &t : m.tensors) {
     if (t.buffer >= m.buffers.size()) fail(Status::InvalidModel, "tensor references missing buffer");

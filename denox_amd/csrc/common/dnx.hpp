@@ -76,6 +76,10 @@ struct TensorInfo {
 struct Tensor { uint32_t buffer = 0; ScalarSource offset, size; TensorInfo info; };
 struct TensorInitializer { uint32_t tensor; std::vector<uint8_t> data; };
 struct ValueName { std::string name; ScalarSource value; };
+// A relation between two extents that the model's graph needs and that symbolic extents only settle when an instance gets its
+// values: lhs == rhs (relation 0) or lhs <= rhs (1).  `what` names the layer for the error message.  (No counterpart in dnx.fbs:
+// the reference leaves such extents to the caller; a trailing field of `Model`, skipped by readers of the unchanged schema.)
+struct Requirement { ScalarSource lhs, rhs; uint8_t relation = 0; std::string what; };
 struct ShaderBinary { std::vector<uint8_t> code_object; uint32_t spirv_words = 0; };
 struct ModelInfo { std::string producer, producer_version, model_version; };
 
@@ -91,6 +95,9 @@ struct Model {
   std::vector<ShaderBinary> shader_binaries;
   SymIR sym_ir;
   std::vector<ValueName> value_names;
+  std::vector<Requirement> requirements;
+  // Error(InvalidArgument) naming the first requirement that the evaluated symbol table `dp` violates
+  void checkRequirements(const std::vector<int64_t> &dp) const;
 };
 
 std::vector<uint8_t> serialize(const Model &m);

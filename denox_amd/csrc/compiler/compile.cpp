@@ -377,6 +377,7 @@ std::vector<uint8_t> compile(const Model &modelIn, const hip::HipCompiler &hipc,
 
   out.sym_ir = sym.compile();
   for (const auto &nv : model.valueNames()) out.value_names.push_back(dnx::ValueName{nv.name, src(nv.value)});
+  for (const auto &q : model.requirements()) out.requirements.push_back(dnx::Requirement{src(q.lhs), src(q.rhs), static_cast<uint8_t>(q.relation), q.what});
   out.required_features = {1u}; // HipCodeObject: the binaries are gfx950 code objects, not SPIR-V
   dnx::validate(out);
   dnx::requireExecutable(out);

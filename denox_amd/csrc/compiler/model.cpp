@@ -83,12 +83,23 @@ TensorHandle Model::pool(TensorHandle src, unsigned kx, unsigned ky, unsigned px
   return m_ops.back().output;
 }
 
+// A relation that constants violate is an error now; one that involves a symbol is recorded and checked per instance.
+void Model::require(Sym lhs, Sym rhs, int relation, const std::string &what) {
+  if (lhs == rhs) return;
+  if (lhs.isConst() && rhs.isConst()) {
+    if (relation == 0 ? lhs.v != rhs.v : lhs.v > rhs.v)
+      fail(Status::InvalidArgument, what + ": " + std::to_string(lhs.v) + (relation == 0 ? " != " : " > ") + std::to_string(rhs.v));
+    return;
+  }
+  m_requirements.push_back(Requirement{lhs, rhs, relation, what});
+}
+
 TensorHandle Model::concat(TensorHandle src0, TensorHandle src1) {
   const TensorNode a = get(src0), b = get(src1);
-  // extents must agree; when both are constants this is checked here, symbolic
-  // extents are the caller's responsibility (as in the reference importer)
-  if (a.width.isConst() && b.width.isConst() && a.width.v != b.width.v) fail(Status::InvalidArgument, "concat: widths differ");
-  if (a.height.isConst() && b.height.isConst() && a.height.v != b.height.v) fail(Status::InvalidArgument, "concat: heights differ");
+  // extents must agree (the reference's importer leaves symbolic extents to the caller; here they are checked when an
+  // instance is created: kernels index the sources with the result's extents)
+  require(a.width, b.width, 0, "concat: widths of the sources differ");
+  require(a.height, b.height, 0, "concat: heights of the sources differ");
   Op op;
   op.kind = OpKind::Concat;
   op.inputs = {src0, src1};
@@ -118,6 +129,12 @@ TensorHandle Model::slice(TensorHandle src, Sym left, Sym right, Sym top, Sym bo
   op.kind = OpKind::Slice;
   op.inputs = {src};
   op.left = left; op.right = right; op.top = top; op.bottom = bottom;
+  require(Sym::Const(0), left, 1, "slice: left bound below zero");
+  require(Sym::Const(0), top, 1, "slice: top bound below zero");
+  require(left, right, 1, "slice: left bound beyond the right one");
+  require(top, bottom, 1, "slice: top bound beyond the bottom one");
+  require(right, in.width, 1, "slice: right bound beyond the source's width");
+  require(bottom, in.height, 1, "slice: bottom bound beyond the source's height");
   // [left, right) x [top, bottom) in source coordinates (frontend/model/Model.cpp:233-253 of the reference)
   op.output = newTensor(m_sym.sub(right, left), m_sym.sub(bottom, top), in.channels, static_cast<int>(m_ops.size()));
   m_tensors[src].consumers.push_back(static_cast<int>(m_ops.size()));

@@ -79,6 +79,10 @@ public:
   const std::vector<TensorHandle> &inputs() const { return m_inputs; }
   const std::vector<TensorHandle> &outputs() const { return m_outputs; }
   const std::vector<NamedValue> &valueNames() const { return m_valueNames; }
+  // relations between extents that a layer needs and that are not settled while the model is built (symbolic extents):
+  // lhs == rhs (relation 0) or lhs <= rhs (1); checked when an instance is created
+  struct Requirement { Sym lhs, rhs; int relation; std::string what; };
+  const std::vector<Requirement> &requirements() const { return m_requirements; }
 
 private:
   TensorHandle newTensor(Sym w, Sym h, unsigned c, int producer);
@@ -88,6 +92,8 @@ private:
   std::vector<Op> m_ops;
   std::vector<TensorHandle> m_inputs, m_outputs;
   std::vector<NamedValue> m_valueNames;
+  std::vector<Requirement> m_requirements;
+  void require(Sym lhs, Sym rhs, int relation, const std::string &what);
 };
 
 } // namespace denox::compiler

@@ -108,6 +108,7 @@ Instance::Instance(ModelHandle model, const std::vector<ValueSpec> &specs) : m_m
     if (vn.value.symbolic && vn.value.value >= 0 && static_cast<uint64_t>(vn.value.value) < vars.size() && !set[static_cast<size_t>(vn.value.value)])
       fail(Status::InvalidArgument, "no value given for dynamic extent '" + vn.name + "'");
   m_sym = m.sym_ir.eval(vars);
+  m.checkRequirements(m_sym); // extents the graph needs to agree (concat sources, slice bounds)
 
   // tensors must fit their buffers
   m_bufferSizes.resize(m.buffers.size());

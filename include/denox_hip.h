@@ -251,7 +251,8 @@ void denox_hip_model_destroy(denox_hip_model *m);
 int denox_hip_model_dispatch_count(const denox_hip_model *m, uint32_t *out);
 
 /* names/values: the dynamic extents ("H", "W", ...); unknown names are ignored,
- * a missing one is an error */
+ * a missing one is an error.  Extents that the graph cannot take (sources of a concat that differ in width or height, a
+ * slice that leaves its source) are DENOX_HIP_INVALID_ARGUMENT; a tensor of 4 GiB or more is DENOX_HIP_UNSUPPORTED. */
 int denox_hip_instance_create(denox_hip_model *m, const char *const *names, const int64_t *values, uint32_t n, denox_hip_instance **out);
 void denox_hip_instance_destroy(denox_hip_instance *inst);
 int denox_hip_instance_input_count(const denox_hip_instance *inst, uint32_t *out);

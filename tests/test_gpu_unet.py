@@ -174,7 +174,7 @@ def test_threads_with_their_own_handles_run_at_once():
     compile and infer at the same time (the kernel cache, the last-error string and the compile report are the shared or
     thread-local state).  Each thread's results must equal the ones computed alone."""
     import threading
-    nets = [("oidn_unet", 40, 56), ("tiny_unet", 64, 96), ("oidn_unet", 33, 47), ("tiny_unet", 37, 61)]
+    nets = [("oidn_unet", 40, 56), ("tiny_unet", 64, 96), ("oidn_unet", 33, 47), ("tiny_unet", 38, 62)]  # (the miniature has no alignment pad: even extents only)
     alone = []
     for i, (net, H, W) in enumerate(nets):
         m, _ = networks.build(net, seed=i)
@@ -409,3 +409,17 @@ def test_frame_sequence_matches_frame_by_frame(net, H, W, layout, pinned):
     inst.infer_device(None, None)
     inst.synchronize()
     assert inst.infer_many([]) == []
+
+
+def test_instance_refuses_extents_the_graph_cannot_take():
+    """Without the pad to a multiple of 16 the U-Net only takes extents that halve evenly four times: upsample(pool(x)) and the
+    skip tensor differ otherwise, and the concat kernels would index one of them out of range.  The instance is refused
+    with the layer and the numbers, before anything runs; good extents still work on the same module."""
+    m, _ = networks.build("oidn_unet", seed=1, align=False)
+    mod = dx.Module.compile(m)
+    for H, W in [(66, 64), (64, 70), (8, 8)]:
+        with pytest.raises(dx.DenoxHipError) as e:
+            mod.instance(H=H, W=W)
+        assert e.value.status == 1 and "concat" in str(e.value)
+    x = networks.synthetic_input("oidn_unet", 32, 48, seed=1)
+    assert np.isfinite(mod.instance(H=32, W=48).infer(x)[0]).all()

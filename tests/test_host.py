@@ -363,6 +363,38 @@ def test_min_cost_selection_against_exhaustive_enumeration():
     assert total == 7 and chosen == [0, 1, 2]
 
 
+def test_extents_the_graph_needs_are_checked_per_instance():
+    """Symbolic extents leave two things open until an instance gets its values: whether the sources of a concat agree in
+    width and height, and whether a slice stays inside its source.  Both are recorded in the model file and checked when
+    extents are supplied (describe here, instance creation on the GPU), with the layer and the numbers in the message;
+    with constant extents the builder refuses at once."""
+    m, _ = networks.build("oidn_unet", align=False)  # no pad to a multiple of 16: upsample(pool(x)) only matches x for such extents
+    blob = dx.compile_model(m)
+    assert len(dx.describe(blob, H=64, W=96)["dispatches"]) > 7
+    for H, W, what in [(66, 64, "heights"), (64, 70, "widths"), (16, 64, None), (8, 64, "heights")]:
+        if what is None:
+            dx.describe(blob, H=H, W=W)  # 16 rows: every one of the four levels still halves evenly
+            continue
+        with pytest.raises(dx.DenoxHipError) as e:
+            dx.describe(blob, H=H, W=W)
+        assert e.value.status == 1 and "concat" in str(e.value) and what in str(e.value)
+    dx.describe(blob)  # a listing without extents evaluates nothing
+    m2 = dx.Model()
+    t = m2.input("input", "W", "H", 8)
+    m2.output(m2.slice(t, 2, 40, 1, m2.sym("H") - 1))
+    b2 = dx.compile_model(m2)
+    dx.describe(b2, H=10, W=64)
+    for H, W in [(10, 30), (1, 64)]:
+        with pytest.raises(dx.DenoxHipError) as e:
+            dx.describe(b2, H=H, W=W)
+        assert e.value.status == 1 and "slice" in str(e.value)
+    # the record survives the file: damaged relation codes are refused by the reader's validation
+    assert dx.describe(bytes(blob), H=64, W=96)["dispatches"]
+    with pytest.raises(dx.DenoxHipError):
+        m3 = dx.Model()
+        m3.concat(m3.input("a", 8, 8, 4), m3.input("b", 9, 8, 4))
+
+
 # ----------------------------------------------------------------------------- timing table
 def test_db_running_statistics_and_persistence(tmp_path):
     path = str(tmp_path / "gpu.db")
