@@ -29,7 +29,11 @@ FIRST_PAIR = "pad+conv3x3+relu+conv3x3+relu+maxpool"       # enc_conv0 -> enc_co
 # longest dispatches that the timing table has been seen to select, in the layouts it combines them in.
 STEER = ([{DOMINANT_OPERATION: c} for c in ("g4r1n", "g4r1k32n", "g4r1", "g4r1k32", "s8r2k16", "s12r1k16", "t8r2k16", "p8r2k16", "f8r1")] +
          [{DOMINANT_OPERATION: "g4r1n", LAST_PAIR: c, FIRST_PAIR: "x8r2k16/hwc>chwc8"} for c in ("z4r2k64", "y4r2k32", "x8r2k16")] +
-         [{DOMINANT_OPERATION: d + "/hwc>chwc8", LAST_PAIR: c + "/chwc8>hwc"} for d, c in (("s8r2k16", "z4r2k64"), ("s12r1k16", "y4r2k32"), ("s8r2k16", "x8r2k16"))])
+         [{DOMINANT_OPERATION: d + "/hwc>chwc8", LAST_PAIR: c + "/chwc8>hwc"} for d, c in (("s8r2k16", "z4r2k64"), ("s12r1k16", "y4r2k32"), ("s8r2k16", "x8r2k16"))] +
+         # the same layers as four dispatches (conv -> conv fusion off, pixel-major), for comparison with the pairs
+         [{"features": dict(conv_conv_fusion=False, blocked_layout=False)}])
+# dispatches of that last schedule whose traffic is reported beside the pairs': entry point prefixes
+UNFUSED_PAIR_LAYERS = ("conv3x3_c9e_k32_", "conv3x3_c32_k32_relu_pool_", "conv3x3_c64_k32_relu_", "conv3x3_c32_k3_crop_")
 COPY_KERNEL = "memory_slice_c64v8"
 
 
@@ -46,14 +50,16 @@ def run(map_path, H=1080, W=1920, frames=6):
     kernels = {}
     tmp = tempfile.mkdtemp(prefix="denox_hip_probe_")
     for n, steer in enumerate(STEER):
+        steer = dict(steer)
+        features = steer.pop("features", {})
         db = dx.Db(os.path.join(tmp, f"steer{n}.db"))
-        db.populate(model, assume={"H": H, "W": W})
+        db.populate(model, assume={"H": H, "W": W}, features=features)
         rows = [r.split('","') for r in db.dump_csv().splitlines()[1:]]
         hits = [i for i, r in enumerate(rows) if steer.get(r[0].strip('"')) == _norm(r[2])]
         for i in hits:
             for _ in range(3):
                 db.add_sample(i, 1000.0)  # 1 us: below every estimate, so the selection takes this candidate
-        blob = dx.compile_model(model, assume={"H": H, "W": W}, db=db)
+        blob = dx.compile_model(model, assume={"H": H, "W": W}, db=db, features=features)
         desc = dx.describe(blob, H=H, W=W)["dispatches"]
         taken = {d["name"]: _norm(d["debug_info"].split(" | ")[0]) for d in desc}
         if any(taken.get(op) != cfg for op, cfg in steer.items()):
@@ -104,7 +110,7 @@ def summarize(map_path, fetch_csv, write_csv):
     for entry, k in sorted(m["kernels"].items()):
         # the dominant layer's candidates and the two conv -> conv dispatches: kernels that run at one extent only
         # (a name like conv3x3_c96_k96_relu_* serves two layers of different size; a mean over both describes neither)
-        if entry not in fetch or entry not in write or k["operation"] not in (DOMINANT_OPERATION, LAST_PAIR, FIRST_PAIR):
+        if entry not in fetch or entry not in write or not (k["operation"] in (DOMINANT_OPERATION, LAST_PAIR, FIRST_PAIR) or entry.startswith(UNFUSED_PAIR_LAYERS)):
             continue
         f_, w_ = fetch[entry], write[entry]
         fb, wb = float(np.mean(f_[1:] if len(f_) > 1 else f_)) * fscale, float(np.mean(w_[1:] if len(w_) > 1 else w_)) * wscale
