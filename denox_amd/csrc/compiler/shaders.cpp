@@ -232,9 +232,9 @@ bool chooseFold(const ConvConfig &cfg, unsigned CA, unsigned CB, unsigned K, con
   const unsigned regBudget = std::min(256u, 512u / ((cfg.waves + cfg.pw + 3) / 4));
   const unsigned nva = (aPix * (g.CAP / 8) + threads - 1) / threads, nvb = CB ? (bPix * (g.CBP / 8) + threads - 1) / threads : 0;
   g.cka = g.CAP;
-  if (cfg.pw) { // staging-wave variant: a second source of one matrix step of channels (its weights live in registers), whole
+  if (cfg.pw) { // staging-wave variant: a second source of at most two matrix steps of channels (its weights live in registers), whole
                 // 32- or 64-channel slices of the result; A in steps of cfg.ck channels
-    if (!CB || g.CBP != 16 || K % 32) return false;
+    if (!CB || g.CBP > 32 || K % 32) return false;
     if (cfg.ck) {
       if (cfg.ck >= g.CAP || g.CAP % cfg.ck) return false;
       g.cka = cfg.ck;
@@ -247,7 +247,8 @@ bool chooseFold(const ConvConfig &cfg, unsigned CA, unsigned CB, unsigned K, con
     const unsigned kt = kb * 32;
     if (cfg.pw && kt > 64) continue;
     // computing waves: accumulators, converted tile; waves that move halos: their registers and what locates them (3 per vector)
-    if (cfg.pw ? (std::max(2 * kb * cfg.rpw * 24 + 9 * kb * 4 + 64, nva * 7 + nvb * 7 + 24) > regBudget) : (kb * cfg.rpw * 24 + (nva + nvb) * 4 + 64 > regBudget)) continue;
+    if (cfg.pw && 9 * (g.CBP / 16) * kb * 4 > 96) continue; // the second source's weights live in registers
+    if (cfg.pw ? (std::max(2 * kb * cfg.rpw * 24 + 9 * (g.CBP / 16) * kb * 4 + 64, nva * 7 + nvb * 7 + 24) > regBudget) : (kb * cfg.rpw * 24 + (nva + nvb) * 4 + 64 > regBudget)) continue;
     for (unsigned pitchPad : {8u, 0u}) { // the B halo gives up its bank-conflict padding where LDS is short
       // the staging-wave variant keeps B's weights in registers and the finished tile (tlh rows of 64 pixels) in LDS
       const size_t lds = (static_cast<size_t>(16 / classes * kt) * (g.CAP + 8) + (cfg.pw ? static_cast<size_t>(tlh) * 64 * kt : CB ? static_cast<size_t>(9 * kt) * (g.CBP + 8) : 8) +

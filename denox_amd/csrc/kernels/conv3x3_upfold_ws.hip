@@ -15,11 +15,11 @@
 // last read NA steps ago, and at once issue the loads of the same step of the next tile.  The finished tile goes to
 // memory through LDS as well: the computing waves leave it there as binary16 and the staging waves store it during the
 // next tile's first step -- whole output rows, 1 KiB of consecutive addresses per store instruction, instead of 16
-// bytes per lane at a stride of two pixels.  The 9-tap weights of B (at most 16 channels) live in registers of the
+// bytes per lane at a stride of two pixels.  The 9-tap weights of B (at most 32 channels) live in registers of the
 // computing waves, which is what makes room for that tile in LDS.
 //
 // Compile-time interface: as conv3x3_upfold.hip, plus PW (staging waves) and CKA (channels of A per step, divides CAP);
-// 8 <= CB <= 16; KT = 32 or 64 and KOUT a multiple of KT; the result 16-byte aligned (OVEC).  Packed weights as there:
+// 8 <= CB <= 32 (its 9-tap weights must fit the registers); KT = 32 or 64 and KOUT a multiple of KT; the result 16-byte aligned (OVEC).  Packed weights as there:
 // [class a*2+b][kt][A taps ty*2+tx][KT][CAP][B taps r*3+s][KT][CBP].
 #include "conv_common.h"
 
@@ -39,7 +39,7 @@ static_assert(CA % 8 == 0 && CB >= 8 && PW > 0, "whole 8-channel vectors of A; a
 #define CKA CAP
 #endif
 static_assert(CAP % CKA == 0 && CKA % 16 == 0, "whole steps");
-static_assert(CBP == 16, "the weights of B are kept in registers: one matrix step of channels");
+static_assert(9 * (CBP / 16) * KB * 4 <= 96, "the weights of B are kept in registers: 9 taps x channel steps x output blocks fragments");
 static_assert((KT == 32 || KT == 64) && KOUT % KT == 0 && OVEC && OPITCH % 8 == 0 && !LAYOUT_OUT && !LAYIN, "whole 16-byte slots of a pixel-major result");
 #define NA (CAP / CKA)
 #define WAP (CAP + 8)    // pitch of the A weights
@@ -260,14 +260,16 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     const int l32 = lane & 31;
     const int kq = (lane >> 5) * 8;
     // the 9 taps of B: the same for every class (class (ca, 0)'s copy), one matrix step of channels, in registers
-    half8 wB[9][KB];
+    half8 wB[9][CBP / 16][KB];
     {
       const _Float16 *w = FILT + (size_t)((ca * 2) * NKT + kt) * KT * (4 * CAP + 9 * CBP) + 4 * KT * CAP;
 #pragma unroll
       for (int tap = 0; tap < 9; ++tap)
 #pragma unroll
-        for (int kb = 0; kb < KB; ++kb)
-          wB[tap][kb] = *reinterpret_cast<const half8 *>(w + ((tap * KT + kb * 32 + l32) * CBP + kq));
+        for (int ks = 0; ks < CBP / 16; ++ks)
+#pragma unroll
+          for (int kb = 0; kb < KB; ++kb)
+            wB[tap][ks][kb] = *reinterpret_cast<const half8 *>(w + ((tap * KT + kb * 32 + l32) * CBP + ks * 16 + kq));
     }
     Acc acc[2]; // column parity b = 0, 1
     for (int n = 0; n < myTiles; ++n) {
@@ -310,8 +312,9 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
       // ---- the 9 taps over the full-resolution source: class (ca, b), tap (r, s) reads halo row 2 (y - yl0) + r,
       // halo column 2 (x - xl0) + b + s, which the de-interleaved halo holds at [parity (b + s) & 1][(x - xl0) + (b + s) / 2]
       DNX_SYNC();
-      {
-        const int kk = kq;
+#pragma unroll
+      for (int ks = 0; ks < CBP / 16; ++ks) {
+        const int kk = ks * 16 + kq;
 #pragma unroll
         for (int r = 0; r < 3; ++r) {
           half8 px[RPW][4];
@@ -328,7 +331,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
               for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
                 for (int j = 0; j < RPW; ++j)
-                  acc[b].v[kb][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wB[r * 3 + s2][kb], px[j][b + s2], acc[b].v[kb][j], 0, 0, 0);
+                  acc[b].v[kb][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wB[r * 3 + s2][ks][kb], px[j][b + s2], acc[b].v[kb][j], 0, 0, 0);
         }
       }
       // the tile as binary16 into LDS: this lane's 16 channels kb * 32 + (lane >> 5) * 16 .. of the pixels 2 l32 + b
