@@ -49,7 +49,9 @@ std::string fmtFloat(float v) {
 // fold: the 2x upsample of source A folded into the weights (conv3x3_upfold.hip, with pw: conv3x3_upfold_ws.hip; rpw counts low-resolution rows).
 // ntStore: the result is stored with the non-temporal cache policy.
 // ostage: the finished tile goes to memory through LDS, stored by the staging waves (OSTAGE in conv3x3_mfma_ws.hip).
-struct ConvConfig { unsigned waves, rpw, ck; bool resident; unsigned pw; unsigned maxKT; unsigned mf, xb; const char *name; bool pp = false; bool fold = false; bool wideHalo = false; bool ntStore = false; bool ostage = false; };
+// ksplit: computing waves share a tile's rows AND its output channels (KSP in conv3x3_upfold_ws.hip): wave w takes block
+// w % ksplit of the 32-channel blocks and row group w / ksplit.
+struct ConvConfig { unsigned waves, rpw, ck; bool resident; unsigned pw; unsigned maxKT; unsigned mf, xb; const char *name; bool pp = false; bool fold = false; bool wideHalo = false; bool ntStore = false; bool ostage = false; unsigned ksplit = 1; };
 const ConvConfig kConvConfigs[] = {
     // weights streamed per step
     {4, 2, 16, false, 0, 0, 32, 1, "w4r2k16"}, {4, 2, 32, false, 0, 0, 32, 1, "w4r2k32"}, {4, 4, 16, false, 0, 0, 32, 1, "w4r4k16"}, {4, 4, 32, false, 0, 0, 32, 1, "w4r4k32"},
@@ -89,6 +91,9 @@ const ConvConfig kConvConfigs[] = {
     {4, 1, 0, true, 4, 0, 32, 1, "g4r1", false, true},   {4, 1, 32, true, 4, 0, 32, 1, "g4r1k32", false, true},
     // ... and non-temporal stores of the result (whole lines written once, never read by this kernel)
     {4, 1, 0, true, 4, 0, 32, 1, "g4r1n", false, true, false, true}, {4, 1, 32, true, 4, 0, 32, 1, "g4r1k32n", false, true, false, true},
+    // ... and two rows of half the output channels per wave instead of one row of all of them (fewer LDS reads per matrix instruction)
+    {4, 2, 0, true, 4, 0, 32, 1, "h4r2", false, true, false, false, false, 2}, {4, 2, 0, true, 4, 0, 32, 1, "h4r2n", false, true, false, true, false, 2},
+    {4, 2, 32, true, 4, 0, 32, 1, "h4r2k32n", false, true, false, true, false, 2},
     // the smallest tiles, offered to strided layers only: a stride multiplies the halo of a tile, and a 7 x 7 filter with
     // stride 4 fits the LDS next to its weights with nothing larger
     {2, 1, 16, false, 0, 32, 32, 1, "w2r1k16n", false, false, true}, {2, 1, 32, false, 0, 16, 16, 1, "m2r1k32x1n", false, false, true},
@@ -226,7 +231,8 @@ struct FoldGeometry {
 bool chooseFold(const ConvConfig &cfg, unsigned CA, unsigned CB, unsigned K, const DeviceInfo &dev, FoldGeometry &g) {
   if (CA % 8 || (CB > 0 && CB < 8)) return false; // whole vectors of A; B's partial last vector is read ending at its last channel
   g.CA = CA; g.CB = CB; g.CAP = (CA + 15) / 16 * 16; g.CBP = CB ? (CB + 15) / 16 * 16 : 0; g.K = K; g.KOUTP = (K + 31) / 32 * 32;
-  const unsigned tlh = cfg.waves * cfg.rpw, threads = (cfg.pw ? cfg.pw : cfg.waves) * 64; // threads that move halos
+  if (cfg.waves % cfg.ksplit) return false;
+  const unsigned tlh = cfg.waves / cfg.ksplit * cfg.rpw, threads = (cfg.pw ? cfg.pw : cfg.waves) * 64; // threads that move halos
   const unsigned classes = cfg.pw ? 2 : 4; // kinds of workgroup: row parities, or row x column parities
   const unsigned aPix = (tlh + 1) * (cfg.pw ? 34 : 33), bPix = (2 * tlh + 1) * (cfg.pw ? 66 : 65), blocks = g.KOUTP / 32;
   const unsigned regBudget = std::min(256u, 512u / ((cfg.waves + cfg.pw + 3) / 4));
@@ -246,9 +252,11 @@ bool chooseFold(const ConvConfig &cfg, unsigned CA, unsigned CB, unsigned K, con
     if (cfg.maxKT && kb * 32 > cfg.maxKT) continue;
     const unsigned kt = kb * 32;
     if (cfg.pw && kt > 64) continue;
+    if (kb % cfg.ksplit) continue;
+    const unsigned kbw = kb / cfg.ksplit; // blocks per computing wave
     // computing waves: accumulators, converted tile; waves that move halos: their registers and what locates them (3 per vector)
-    if (cfg.pw && 9 * (g.CBP / 16) * kb * 4 > 96) continue; // the second source's weights live in registers
-    if (cfg.pw ? (std::max(2 * kb * cfg.rpw * 24 + 9 * (g.CBP / 16) * kb * 4 + 64, nva * 7 + nvb * 7 + 24) > regBudget) : (kb * cfg.rpw * 24 + (nva + nvb) * 4 + 64 > regBudget)) continue;
+    if (cfg.pw && 9 * (g.CBP / 16) * kbw * 4 > 96) continue; // the second source's weights live in registers
+    if (cfg.pw ? (std::max(2 * kbw * cfg.rpw * 24 + 9 * (g.CBP / 16) * kbw * 4 + 64, nva * 7 + nvb * 7 + 24) > regBudget) : (kb * cfg.rpw * 24 + (nva + nvb) * 4 + 64 > regBudget)) continue;
     for (unsigned pitchPad : {8u, 0u}) { // the B halo gives up its bank-conflict padding where LDS is short
       // the staging-wave variant keeps B's weights in registers and the finished tile (tlh rows of 64 pixels) in LDS
       const size_t lds = (static_cast<size_t>(16 / classes * kt) * (g.CAP + 8) + (cfg.pw ? static_cast<size_t>(tlh) * 64 * kt : CB ? static_cast<size_t>(9 * kt) * (g.CBP + 8) : 8) +
@@ -507,6 +515,7 @@ public:
     hip::HipCompilerInstance k = m_compiler->read(cfg.fold ? (cfg.pw ? "conv3x3_upfold_ws.hip" : "conv3x3_upfold.hip") : cfg.resident ? "conv3x3_mfma_ws.hip" : "conv3x3_mfma.hip");
     if (cfg.fold) k.define("BPITCH", fg.bpitch ? fg.bpitch : 8);
     if (cfg.fold && cfg.pw) k.define("CKA", fg.cka);
+    if (cfg.ksplit > 1) k.define("KSP", cfg.ksplit);
     if (cfg.ntStore) k.define("STORE_AUX", 2);
     if (cfg.ostage) k.define("OSTAGE", 1);
     k.define("CA", CA); k.define("CB", CB); k.define("UPA", up ? 1 : 0);
@@ -619,9 +628,11 @@ private:
 // crossing memory -- in ConcatConvCMShader (conv/ConcatConvCMShader.cpp:760-965); a conv -> conv fusion it does not have.
 // ck: input channels of the first convolution per LDS stage; pw: extra waves that only move halos (the others then only compute)
 // w1reg: the first convolution's weights in registers of the computing waves (needs pw)
-struct PairConfig { unsigned waves, rpw, ck; const char *name; unsigned pw = 0; bool w1reg = false; };
+// c2stage: the second convolution, its epilogue and its stores on the staging waves (needs pw == waves)
+struct PairConfig { unsigned waves, rpw, ck; const char *name; unsigned pw = 0; bool w1reg = false; bool c2stage = false; };
 const PairConfig kPairConfigs[] = {{8, 2, 16, "x8r2k16"}, {4, 2, 32, "x4r2k32"}, {4, 4, 16, "x4r4k16"}, {4, 2, 16, "x4r2k16"},
-                                   {4, 2, 32, "y4r2k32", 4}, {4, 2, 64, "z4r2k64", 4, true}};
+                                   {4, 2, 32, "y4r2k32", 4}, {4, 2, 64, "z4r2k64", 4, true},
+                                   {4, 2, 64, "v4r2k64", 4, true, true}, {4, 2, 16, "v4r2k16", 4, true, true}, {4, 2, 32, "u4r2k32", 4, false, true}};
 constexpr unsigned kNumPairConfigs = sizeof(kPairConfigs) / sizeof(kPairConfigs[0]);
 
 bool isPairConfigName(const std::string &name) {
@@ -644,6 +655,11 @@ bool choosePair(const PairConfig &cfg, unsigned CA, unsigned CB, unsigned K1, un
   g.tapm = 3 * K2 <= 15 && !pool;
   // the second convolution's weights (taps x 2 fragments of 4 registers), one accumulator set, fragments, the converted tile, halo registers
   if ((g.tapm ? 24 : 72) + cfg.rpw * 16 + 96 > regBudget) return false;
+  if (cfg.c2stage) {
+    // a staging wave then holds, besides its two sets of halo registers, what the second convolution needs
+    const unsigned nv = (haloPix * (g.ck / 8) + threads - 1) / threads;
+    if (cfg.pw != cfg.waves || 2 * nv * 4 + (g.tapm ? 24 : 72) + cfg.rpw * 16 + 2 * (cfg.rpw + 2) * 4 + 48 > regBudget) return false;
+  }
   const unsigned nchunk = (g.CPAD + g.ck - 1) / g.ck;
   const unsigned ringRows = nchunk == 1 ? 2 * ih + 2 : ih + 2; // see conv3x3_pair.hip
   if (cfg.w1reg && 9 * (g.CPAD / 16) * 4 > 144) return false; // the first convolution's weights must fit the register file next to everything else
@@ -805,6 +821,7 @@ public:
     if (g.tapm) k.define("TAPM", 1);
     if (cfg.pw) k.define("PW", cfg.pw);
     if (cfg.w1reg) k.define("W1REG", 1);
+    if (cfg.c2stage) k.define("C2STAGE", 1);
     const bool blockedIn = !m.inputFormats.empty() && m.inputFormats[0] != 0, blockedOut = m.outputFormat != 0;
     if (blockedIn) k.define("LAYIN", 1);
     if (blockedOut) k.define("LAYOUT_OUT", 1);

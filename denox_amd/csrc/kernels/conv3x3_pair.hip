@@ -38,6 +38,13 @@
 //                                 (9 taps x CPAD / 16 fragments), not in LDS.  With 32 output channels a weight fragment
 //                                 serves RPW matrix instructions only, so reading it from LDS is 3 of the 7 LDS reads per
 //                                 6 instructions, and the LDS read rate, not the matrix pipe, sets the pace of such layers
+//   C2STAGE                       1 (needs PW == WAVES): the second convolution, its epilogue and its stores run on the staging
+//                                 waves, which otherwise wait for memory most of the time: staging wave i does for the rows
+//                                 of computing wave i, in the first chunk of step k + 1, what that wave would do itself.  A
+//                                 computing wave then issues nothing but the first convolution's LDS reads, matrix
+//                                 instructions and ring writes, and the latencies of the second convolution's epilogue
+//                                 (cross-lane sums, conversions, narrow stores) overlap the matrix work of the wave that
+//                                 shares its SIMD instead of preceding it
 // KT is 32 for both convolutions.
 #include "conv_common.h"
 
@@ -62,6 +69,10 @@
 #ifndef W1REG
 #define W1REG 0
 #endif
+#ifndef C2STAGE
+#define C2STAGE 0
+#endif
+static_assert(!C2STAGE || PW == WAVES, "second convolution on the staging waves: one staging wave per computing wave");
 static_assert(!TAPM || (3 * KOUT <= 15 && !POOL), "filter columns in the matrix rows: at most 5 output channels, no pooling");
 
 static_assert(MF == 32 && KT == 32 && KB == 1, "one 32-channel block per convolution");
@@ -214,9 +225,13 @@ __device__ DNX_INLINE void mma_mid(const _Float16 *sMid, int rslot0, const Secon
 
 #if TAPM
 // Epilogue of the TAPM form: lane x of the lower half adds the partial sums of filter columns 1 and 2 held by lanes
-// x + 1 and x + 2 (registers KOUT + k and 2 KOUT + k) to its own (register k), then activation and rounding.
-__device__ DNX_INLINE void pack_tapm(const Acc &acc, Packed &pk, int lane) {
-  const int from1 = ((lane + 1) & 63) * 4, from2 = ((lane + 2) & 63) * 4;
+// x + 1 and x + 2 (registers KOUT + k and 2 KOUT + k) to its own (register k), then activation and rounding.  The
+// neighbours' values arrive by DPP wave shifts (a vector ALU operand modifier); as LDS permutes each of them was a
+// round trip through the LDS queue that the sum had to wait for.
+__device__ DNX_INLINE float from_next_lane(float v) { // lane i: v of lane i + 1 (wave_shl:1); lane 63: 0
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x130, 0xf, 0xf, true));
+}
+__device__ DNX_INLINE void pack_tapm(const Acc &acc, Packed &pk) {
 #pragma unroll
   for (int j = 0; j < RPW; ++j) {
 #pragma unroll
@@ -224,9 +239,7 @@ __device__ DNX_INLINE void pack_tapm(const Acc &acc, Packed &pk, int lane) {
       float v = 0.0f;
       if (i < KOUT) {
         const float p1 = acc.v[0][j][KOUT + i], p2 = acc.v[0][j][2 * KOUT + i]; // (a vector element is no object: copy it before reinterpreting its bits)
-        const float t1 = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(from1, __builtin_bit_cast(int, p1)));
-        const float t2 = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(from2, __builtin_bit_cast(int, p2)));
-        v = (acc.v[0][j][i] + t1) + t2;
+        v = (acc.v[0][j][i] + from_next_lane(p1)) + from_next_lane(from_next_lane(p2));
       }
       pk.o[0][j][i >> 3][i & 7] = finish1(v);
     }
@@ -431,7 +444,8 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   }
 #endif
   SecondWeights w2;
-  load_second_weights(w2, FILT2, lane);
+  if (!C2STAGE || wv >= WAVES) // (with C2STAGE the computing waves never touch them: dead there, no registers)
+    load_second_weights(w2, FILT2, lane);
 
   // ---- the fetch cursor walks the same sequence of (unit, step, channel chunk) as the compute cursor, two chunks ahead.
   // Every unit has one step more than it has rows for: the last one only drains the second convolution, its loads are
@@ -466,25 +480,45 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   int k = 0, cchunk = 0, buf = 0;
   int wslot = 0; // ring row that takes the first `mid` row of step k
   Acc acc;       // the first convolution's accumulators during a step's chunks, the second's in between
+  // outputs of step k - 1, in the first chunk of step k: its `mid` rows and the two before them are in the ring.
+  // rw: the wave whose rows these are
+  auto second = [&](int rw) {
+    if (cchunk == 0 && unit < units && k > 0) { // (unit >= units: a spare chunk behind the last step)
+      init_acc(acc, sBias2, lane);
+      int rslot = wslot - IH - 2;
+      rslot = rslot < 0 ? rslot + NS : rslot;
+      rslot = rslot < 0 ? rslot + NS : rslot;
+      mma_mid(sMid, rslot, w2, acc, rw, lane);
+      Packed pk;
+#if TAPM
+      pack_tapm(acc, pk);
+#else
+      pack_tile(acc, pk);
+#endif
+      store_pair(pk, out, g.ys + (k - 1) * IH - 2, g.xs, g.ys, g.ye, rw, lane, pc);
+    }
+  };
   // what the computing side does in one chunk, after the barrier that published the chunk's halo
   auto compute = [&]() {
-    const bool alive = unit < units; // false in a spare chunk behind the last step
-    if (cchunk == 0) {
-      if (alive && k > 0) { // outputs of step k - 1: its `mid` rows and the two before them are in the ring
-        init_acc(acc, sBias2, lane);
-        int rslot = wslot - IH - 2;
-        rslot = rslot < 0 ? rslot + NS : rslot;
-        rslot = rslot < 0 ? rslot + NS : rslot;
-        mma_mid(sMid, rslot, w2, acc, wv, lane);
-        Packed pk;
-#if TAPM
-        pack_tapm(acc, pk, lane);
-#else
-        pack_tile(acc, pk);
+#if !C2STAGE
+    second(wv);
 #endif
-        store_pair(pk, out, g.ys + (k - 1) * IH - 2, g.xs, g.ys, g.ye, wv, lane, pc);
-      }
+    if (cchunk == 0)
       init_acc_first(acc, sBias1, lane);
+  };
+  // moves the cursor (unit, k, cchunk, wslot) one chunk on
+  auto advance = [&]() {
+    if (++cchunk == NCHUNK) {
+      cchunk = 0;
+      wslot += IH;
+      wslot = wslot >= NS ? wslot - NS : wslot;
+      if (unit < units && ++k > g.steps) { // the drain step is done: next unit
+        k = 0;
+        wslot = 0;
+        unit += GRID;
+        if (unit < units)
+          g = geometry(unit);
+      }
     }
   };
   auto multiply = [&]() {
@@ -501,20 +535,9 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
 #endif
     }
     buf ^= 1;
-    if (++cchunk == NCHUNK) {
-      cchunk = 0;
-      if (real)
-        store_mid(acc, sMid, wslot, g.ys - 1 + k * IH, g.xs - 1, Hc, Wc, wv, lane);
-      wslot += IH;
-      wslot = wslot >= NS ? wslot - NS : wslot;
-      if (alive && ++k > g.steps) { // the drain step is done: next unit
-        k = 0;
-        wslot = 0;
-        unit += GRID;
-        if (unit < units)
-          g = geometry(unit);
-      }
-    }
+    if (real && cchunk == NCHUNK - 1)
+      store_mid(acc, sMid, wslot, g.ys - 1 + k * IH, g.xs - 1, Hc, Wc, wv, lane);
+    advance();
   };
 #if PW == 0
   auto step = [&](H::Regs &regs) {
@@ -557,12 +580,21 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     issue(st1);   // chunk 1
     commit(st0, 0);
     issue(st0);   // chunk 2
+    // with C2STAGE: the second convolution of the step the cursor (unit, k, ...) has just left, for the rows of
+    // computing wave wv - WAVES, after the chunk's memory work is under way
+    auto rest = [&]() {
+#if C2STAGE
+      second(wv - WAVES);
+      advance();
+#endif
+    };
     for (int c = 0; c < chunks; c += 2) {
       DNX_SYNC(); // chunk c starts: sIn[c & 1] is complete, the other buffer is free
       if (c + 1 < chunks) {
         commit(st1, c + 1);
         issue(st1); // chunk c + 3
       }
+      rest();
       if (c + 1 >= chunks)
         break;
       DNX_SYNC(); // chunk c + 1 starts
@@ -570,6 +602,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
         commit(st0, c + 2);
         issue(st0); // chunk c + 4
       }
+      rest();
     }
   } else {
     // ---- computing waves ----

@@ -18,6 +18,11 @@
 // bytes per lane at a stride of two pixels.  The 9-tap weights of B (at most 32 channels) live in registers of the
 // computing waves, which is what makes room for that tile in LDS.
 //
+// KSP = 2 divides the work of a tile among the computing waves by output channels as well as by rows: wave w takes the 32
+// channels w % 2 of the 64 and the RPW rows of row group w / 2 (KSP = 1: all channels, RPW rows of group w).  A weight
+// fragment read from LDS then feeds RPW = 2 matrix instructions instead of one, a pixel fragment as many as before:
+// 17 instead of 22 LDS reads per 16 matrix instructions in the steps over A, whose pace the LDS read rate sets.
+//
 // Compile-time interface: as conv3x3_upfold.hip, plus PW (staging waves) and CKA (channels of A per step, divides CAP);
 // 8 <= CB <= 32 (its 9-tap weights must fit the registers); KT = 32 or 64 and KOUT a multiple of KT; the result 16-byte aligned (OVEC).  Packed weights as there:
 // [class a*2+b][kt][A taps ty*2+tx][KT][CAP][B taps r*3+s][KT][CBP].
@@ -39,7 +44,12 @@ static_assert(CA % 8 == 0 && CB >= 8 && PW > 0, "whole 8-channel vectors of A; a
 #define CKA CAP
 #endif
 static_assert(CAP % CKA == 0 && CKA % 16 == 0, "whole steps");
-static_assert(9 * (CBP / 16) * KB * 4 <= 96, "the weights of B are kept in registers: 9 taps x channel steps x output blocks fragments");
+#ifndef KSP
+#define KSP 1
+#endif
+#define KBW (KB / KSP) // 32-channel blocks of the result per computing wave
+static_assert(KB % KSP == 0 && WAVES % KSP == 0, "whole blocks and whole row groups per wave");
+static_assert(9 * (CBP / 16) * KBW * 4 <= 96, "the weights of B are kept in registers: 9 taps x channel steps x output blocks fragments");
 static_assert((KT == 32 || KT == 64) && KOUT % KT == 0 && OVEC && OPITCH % 8 == 0 && !LAYOUT_OUT && !LAYIN, "whole 16-byte slots of a pixel-major result");
 #define NA (CAP / CKA)
 #define WAP (CAP + 8)    // pitch of the A weights
@@ -48,7 +58,7 @@ static_assert((KT == 32 || KT == 64) && KOUT % KT == 0 && OVEC && OPITCH % 8 == 
 #ifndef BPITCH
 #define BPITCH (CBP + 8) // pitch of a B halo pixel (CBP: no padding, where LDS is short)
 #endif
-#define TLH (WAVES * RPW)
+#define TLH (WAVES / KSP * RPW)
 #define AH (TLH + 1)
 #define AW 34
 #define BH (2 * TLH + 1)
@@ -259,8 +269,10 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     // ---- computing waves -------------------------------------------------------------------------------------
     const int l32 = lane & 31;
     const int kq = (lane >> 5) * 8;
+    const int rg = wv / KSP;           // row group: low-resolution rows rg * RPW .. of the tile
+    const int kb0 = (wv % KSP) * KBW;  // first of this wave's 32-channel blocks
     // the 9 taps of B: the same for every class (class (ca, 0)'s copy), one matrix step of channels, in registers
-    half8 wB[9][CBP / 16][KB];
+    half8 wB[9][CBP / 16][KBW];
     {
       const _Float16 *w = FILT + (size_t)((ca * 2) * NKT + kt) * KT * (4 * CAP + 9 * CBP) + 4 * KT * CAP;
 #pragma unroll
@@ -268,10 +280,10 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
 #pragma unroll
         for (int ks = 0; ks < CBP / 16; ++ks)
 #pragma unroll
-          for (int kb = 0; kb < KB; ++kb)
-            wB[tap][ks][kb] = *reinterpret_cast<const half8 *>(w + ((tap * KT + kb * 32 + l32) * CBP + ks * 16 + kq));
+          for (int kb = 0; kb < KBW; ++kb)
+            wB[tap][ks][kb] = *reinterpret_cast<const half8 *>(w + ((tap * KT + (kb0 + kb) * 32 + l32) * CBP + ks * 16 + kq));
     }
-    Acc acc[2]; // column parity b = 0, 1
+    Acc acc[2]; // column parity b = 0, 1; blocks kb0 .. kb0 + KBW - 1 in v[0 .. KBW - 1]
     for (int n = 0; n < myTiles; ++n) {
       // ---- the folded 2x2 taps over the low-resolution source, CKA channels per step: class (ca, b), tap (ty, tx)
       // reads low-resolution row y + ca - 1 + ty, column x + b - 1 + tx = halo column (x - xl0) + b + tx
@@ -279,8 +291,15 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
       for (int c = 0; c < NA; ++c) {
         DNX_SYNC();
         if (c == 0) { // the staged bias is visible after the first barrier
-          init_acc(acc[0], sBias, lane);
-          init_acc(acc[1], sBias, lane);
+#pragma unroll
+          for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int kb = 0; kb < KBW; ++kb)
+#pragma unroll
+              for (int j = 0; j < RPW; ++j)
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                  acc[b].v[kb][j][i] = HAS_BIAS ? sBias[(kb0 + kb) * 32 + (lane >> 5) * 16 + i] : 0.0f;
         }
 #pragma unroll
         for (int ks = 0; ks < CKA / 16; ++ks) {
@@ -290,19 +309,19 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
           for (int t = 0; t < RPW + 1; ++t)
 #pragma unroll
             for (int cc = 0; cc < 3; ++cc)
-              px[t][cc] = *reinterpret_cast<const half8 *>(sA[c] + ((wv * RPW + t) * AW + l32 + cc) * APITCH + kk);
+              px[t][cc] = *reinterpret_cast<const half8 *>(sA[c] + ((rg * RPW + t) * AW + l32 + cc) * APITCH + kk);
 #pragma unroll
           for (int ty = 0; ty < 2; ++ty)
 #pragma unroll
             for (int tx = 0; tx < 2; ++tx)
 #pragma unroll
               for (int b = 0; b < 2; ++b) {
-                half8 wf[KB];
+                half8 wf[KBW];
 #pragma unroll
-                for (int kb = 0; kb < KB; ++kb)
-                  wf[kb] = *reinterpret_cast<const half8 *>(sWA[b] + ((ty * 2 + tx) * KT + kb * 32 + l32) * WAP + c * CKA + kk);
+                for (int kb = 0; kb < KBW; ++kb)
+                  wf[kb] = *reinterpret_cast<const half8 *>(sWA[b] + ((ty * 2 + tx) * KT + (kb0 + kb) * 32 + l32) * WAP + c * CKA + kk);
 #pragma unroll
-                for (int kb = 0; kb < KB; ++kb)
+                for (int kb = 0; kb < KBW; ++kb)
 #pragma unroll
                   for (int j = 0; j < RPW; ++j)
                     acc[b].v[kb][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[kb], px[j + ty][b + tx], acc[b].v[kb][j], 0, 0, 0);
@@ -322,13 +341,13 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
           for (int j = 0; j < RPW; ++j)
 #pragma unroll
             for (int cc = 0; cc < 4; ++cc)
-              px[j][cc] = *reinterpret_cast<const half8 *>(sB + ((2 * (wv * RPW + j) + r) * BW + (cc & 1) * 33 + l32 + (cc >> 1)) * BPITCH + kk);
+              px[j][cc] = *reinterpret_cast<const half8 *>(sB + ((2 * (rg * RPW + j) + r) * BW + (cc & 1) * 33 + l32 + (cc >> 1)) * BPITCH + kk);
 #pragma unroll
           for (int s2 = 0; s2 < 3; ++s2)
 #pragma unroll
             for (int b = 0; b < 2; ++b)
 #pragma unroll
-              for (int kb = 0; kb < KB; ++kb)
+              for (int kb = 0; kb < KBW; ++kb)
 #pragma unroll
                 for (int j = 0; j < RPW; ++j)
                   acc[b].v[kb][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wB[r * 3 + s2][ks][kb], px[j][b + s2], acc[b].v[kb][j], 0, 0, 0);
@@ -336,17 +355,19 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
       }
       // the tile as binary16 into LDS: this lane's 16 channels kb * 32 + (lane >> 5) * 16 .. of the pixels 2 l32 + b
 #pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        Packed done;
-        pack_tile(acc[b], done);
+      for (int b = 0; b < 2; ++b)
 #pragma unroll
-        for (int kb = 0; kb < KB; ++kb)
+        for (int kb = 0; kb < KBW; ++kb)
 #pragma unroll
-          for (int j = 0; j < RPW; ++j)
+          for (int j = 0; j < RPW; ++j) {
+            float v[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) v[i] = acc[b].v[kb][j][i];
+            const half8 done[2] = {finish8(v), finish8(v + 8)}; // activation, rounding
 #pragma unroll
             for (int e = 0; e < 2; ++e)
-              sOut[OUT_SLOT(wv * RPW + j, 2 * l32 + b, kb * 4 + (lane >> 5) * 2 + e)] = __builtin_bit_cast(uint4v, done.o[kb][j][e]);
-      }
+              sOut[OUT_SLOT(rg * RPW + j, 2 * l32 + b, (kb0 + kb) * 4 + (lane >> 5) * 2 + e)] = __builtin_bit_cast(uint4v, done[e]);
+          }
     }
     DNX_SYNC(); // the last tile is in LDS
   }

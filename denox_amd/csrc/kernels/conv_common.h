@@ -504,6 +504,22 @@ __device__ DNX_INLINE ushort_t dpp_xor1(ushort_t v) {
   // quad_perm [1,0,3,2]: exchange with the neighbouring lane
   return (ushort_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xF, 0xF, true);
 }
+// The 2x2 maximum of a pooled result: the rows are two accumulators of this lane, the columns this lane and its
+// neighbour.  Bias, ReLU and the rounding to binary16 never decrease when their argument grows, so the largest of the
+// four sums finished once is the largest of the four finished values: two instructions per window and one conversion,
+// where finishing all four and comparing the halves took a dozen.  (LeakyReLU with a negative slope is not monotonic:
+// it keeps the element-wise form.)
+#define POOL_MAX_FIRST (POOL && ACT <= 1)
+__device__ DNX_INLINE float pool_max(float top, float bottom) {
+  // The median of (x, y, +inf) is the larger of x and y in one instruction; fmaxf first quiets both operands, three
+  // instructions -- and the compiler turns a median with a constant infinity back into that, so the infinity is a
+  // register whose value it cannot see.
+  float inf = __builtin_inff();
+  asm("" : "+v"(inf));
+  const float a = __builtin_amdgcn_fmed3f(top, bottom, inf);
+  const float n = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, a), 0xB1, 0xF, 0xF, true));
+  return __builtin_amdgcn_fmed3f(a, n, inf);
+}
 
 // ---- output stores ---------------------------------------------------------------------
 // The output is written through a buffer resource: a lane that has nothing to store (pixel outside the image or the
@@ -594,6 +610,13 @@ __device__ DNX_INLINE void pack_tile(const Acc &acc, Packed &pk) {
 #if POOL
 #pragma unroll
     for (int j = 0; j < RPW; j += 2) {
+#if POOL_MAX_FIRST
+      float m[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) m[i] = pool_max(acc.v[kb][j][i], acc.v[kb][j + 1][i]);
+      pk.o[kb][j >> 1][0] = finish8(m);
+      pk.o[kb][j >> 1][1] = finish8(m + 8);
+#else
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const _Float16 v0 = finish1(acc.v[kb][j][i]);
@@ -607,6 +630,7 @@ __device__ DNX_INLINE void pack_tile(const Acc &acc, Packed &pk) {
         m = n1 > m ? n1 : m;
         pk.o[kb][j >> 1][i >> 3][i & 7] = m;
       }
+#endif
     }
 #else
 #pragma unroll
@@ -758,7 +782,9 @@ __device__ DNX_INLINE void pack_tile(const Acc &acc, Packed &pk) {
           const int kb = 2 * kp + (i >> 2) < KB ? 2 * kp + (i >> 2) : 0;
           _Float16 m = (_Float16)0.0f;
           if (i < n) {
-#if POOL
+#if POOL_MAX_FIRST
+            m = finish1(pool_max(acc.v[kb][2 * r][xb][i & 3], acc.v[kb][2 * r + 1][xb][i & 3]));
+#elif POOL
             const _Float16 v0 = finish1(acc.v[kb][2 * r][xb][i & 3]);
             const _Float16 v1 = finish1(acc.v[kb][2 * r + 1][xb][i & 3]);
             const _Float16 n0 = __builtin_bit_cast(_Float16, dpp_xor1(__builtin_bit_cast(ushort_t, v0)));
