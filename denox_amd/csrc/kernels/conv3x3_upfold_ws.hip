@@ -226,20 +226,36 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
           }
       }
     };
-    // the n-th tile of this workgroup, as the computing waves left it in LDS: whole rows of 64 pixels, consecutive
-    // lanes storing consecutive 16 bytes
-    auto store_tile_n = [&](int n) {
-      const int t = tile0 + n * SLOTS;
-      const int yl0 = tileY(t), x0 = 2 * tileX(t);
+    // The finished tile, as the computing waves left it in LDS, goes to memory as whole rows of 64 pixels, consecutive
+    // lanes storing consecutive 16 bytes.  It is read from LDS in the next tile's first step (the only interval in
+    // which it is complete and not yet being rewritten) and stored in portions, one per step of that tile: a store
+    // instruction waits for room in the memory pipeline, and eight of them in a row made the first step's staging work
+    // longer than its matrix work while the last step's staging waves idled.  The last step takes a quarter of the
+    // vectors, the steps over A share the rest.
+    uint4v ov[NVO];
+    auto read_tile = [&]() {
 #pragma unroll
       for (int it = 0; it < NVO; ++it) {
         const int i = st + it * NSTG;
         const int r = i / (64 * SPP), rem = i - r * (64 * SPP);
         const int p = rem / SPP, sl = rem - p * SPP;
+        ov[it] = sOut[i < TLH * 64 * SPP ? OUT_SLOT(r, p, sl) : 0];
+      }
+    };
+    constexpr int NV_LAST = NVO / 4, NV_STEP = (NVO - NV_LAST + NA - 1) / NA;
+    auto store_part = [&](int n, int first, int last) { // vectors [first, last) of this workgroup's n-th tile
+      const int t = tile0 + n * SLOTS;
+      const int yl0 = tileY(t), x0 = 2 * tileX(t);
+#pragma unroll
+      for (int it = 0; it < NVO; ++it) {
+        if (it < first || it >= last)
+          continue;
+        const int i = st + it * NSTG;
+        const int r = i / (64 * SPP), rem = i - r * (64 * SPP);
+        const int p = rem / SPP, sl = rem - p * SPP;
         const bool ok = n >= 0 && i < TLH * 64 * SPP && yl0 + r < HL && x0 + p < (int)pc.IN_W;
-        const uint4v v = sOut[i < TLH * 64 * SPP ? OUT_SLOT(r, p, sl) : 0];
         const unsigned off = ((unsigned)((2 * (yl0 + r) + ca) * (int)pc.IN_W + x0 + p) * (unsigned)OPITCH + (unsigned)(kt * KT + sl * 8)) * 2u;
-        __builtin_amdgcn_raw_buffer_store_b128(v, out, ok ? off : NO_STORE, 0, STORE_AUX);
+        __builtin_amdgcn_raw_buffer_store_b128(ov[it], out, ok ? off : NO_STORE, 0, STORE_AUX);
       }
     };
 #pragma unroll
@@ -260,11 +276,16 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
         commit(nk);
         issue(nk, nn + 1);
         if (k == 0)
-          store_tile_n(n - 1); // complete since the barrier above; rewritten only after the next one
+          read_tile(); // tile n - 1: complete since the barrier above, rewritten only after this tile's last barrier
+        constexpr int cut = NVO - NV_LAST;
+        const int first = k == NA ? cut : (k * NV_STEP < cut ? k * NV_STEP : cut);
+        const int last = k == NA ? NVO : ((k + 1) * NV_STEP < cut ? (k + 1) * NV_STEP : cut);
+        store_part(n - 1, first, last);
       }
     }
     DNX_SYNC(); // the last tile is in LDS
-    store_tile_n(myTiles - 1);
+    read_tile();
+    store_part(myTiles - 1, 0, NVO);
   } else {
     // ---- computing waves -------------------------------------------------------------------------------------
     const int l32 = lane & 31;
