@@ -456,23 +456,36 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   H::map_init(map, PW > 0 ? tid - WAVES * 64 : tid); // (computing waves of the specialised variant never use it)
   Geo fg = geometry(unit);
   int funit = unit, fk = 0, fchunk = 0;
+#if SRC_UNIFORM
+  H::Cols fcols; // the column part of the offsets: one strip, one set of columns
+  H::cols_init(fcols, PW > 0 ? tid - WAVES * 64 : tid, fg.xs - 1, pc);
+#endif
   auto aim = [&]() { // source offsets of the fetch cursor's step; a drain step (or none) reads nothing
     const bool real = funit < units && fk < fg.steps;
+#if SRC_UNIFORM
+    H::rows_init(fsrc, fcols, map, real ? fg.ys - 1 + fk * IH : -0x10000, pc);
+#else
     H::src_init(fsrc, map, real ? fg.ys - 1 + fk * IH : -0x10000, fg.xs - 1, pc);
+#endif
   };
   // Past the last step the cursor stays where it is: the loads are issued all the same (and never used), so that the
   // number of loads in flight is the same on every path through the loop.
   auto issue = [&](H::Regs &regs) {
+    if (fchunk == 0)
+      aim(); // (here rather than after the cursor has moved: the offsets then live in registers only until the loads are out)
     H::fetch_step(srcs, regs, map, fsrc, fchunk);
     if (++fchunk == NCHUNK) {
       fchunk = 0;
       if (funit < units && ++fk > fg.steps) {
         fk = 0;
         funit += GRID;
-        if (funit < units)
+        if (funit < units) {
           fg = geometry(funit);
+#if SRC_UNIFORM
+          H::cols_init(fcols, PW > 0 ? tid - WAVES * 64 : tid, fg.xs - 1, pc);
+#endif
+        }
       }
-      aim();
     }
   };
 
@@ -549,7 +562,6 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     issue(regs); // refill this register set: the chunk after next
     multiply();
   };
-  aim();
   H::Regs st0, st1;
   issue(st0);
   __builtin_amdgcn_sched_barrier(0); // keep the two sets in issue order: the waits count loads in flight
@@ -567,7 +579,6 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     chunks += (geometry(u).steps + 1) * NCHUNK;
   if (wv >= WAVES) {
     // ---- staging waves: chunk c's halo is written to sIn[c & 1] during chunk c - 1 ----
-    aim();
     H::Regs st0, st1;
     int commitChunk = 0; // channel chunk of the halo being written
     auto commit = [&](H::Regs &regs, int c) {

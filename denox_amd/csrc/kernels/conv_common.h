@@ -362,6 +362,40 @@ struct Halo {
   }
 
   static __device__ DNX_INLINE void src_init(Src &s, const Map &m, int y0, int x0, const PushConstants &pc) {
+#if SRC_UNIFORM
+    // Byte offsets below 4 GiB (a buffer resource addresses no more), in 32-bit arithmetic and without a branch: the
+    // coordinates of a pixel outside the image are clamped (or shifted) like any other and the result replaced.
+    const unsigned W = pc.IN_W;
+    constexpr unsigned pixA = LAYIN ? 16 : CA * 2, pixB = LAYIN ? 16 : (CB > 0 ? CB : 1) * 2;
+#if PADA
+    const unsigned rowA = pc.SRC_W * pixA;
+#else
+    const unsigned rowA = (UPA ? (W >> 1) : W) * pixA;
+#endif
+#if PADB
+    const unsigned rowB = pc.SRC_W * pixB;
+#else
+    const unsigned rowB = W * pixB;
+#endif
+#pragma unroll
+    for (int it = 0; it < NV; ++it) {
+      const int gy = y0 * SY + m.hy[it] - PY; // (y0, x0): the tile's first output pixel
+      const int gx = x0 * SX + m.hx[it] - PX;
+      const bool inside = m.lds[it] >= 0 && gy >= 0 && gy < (int)pc.IN_H && gx >= 0 && gx < (int)pc.IN_W;
+#if PADA
+      const int ay = clampi(gy - (int)pc.PAD_T, 0, (int)pc.SRC_H - 1), ax = clampi(gx - (int)pc.PAD_L, 0, (int)pc.SRC_W - 1);
+#else
+      const int ay = UPA ? (gy >> 1) : gy, ax = UPA ? (gx >> 1) : gx;
+#endif
+#if PADB
+      const int by = clampi(gy - (int)pc.PAD_T, 0, (int)pc.SRC_H - 1), bx = clampi(gx - (int)pc.PAD_L, 0, (int)pc.SRC_W - 1);
+#else
+      const int by = gy, bx = gx;
+#endif
+      s.pa[it] = inside ? (int)((unsigned)ay * rowA + (unsigned)ax * pixA) : (int)NO_LOAD;
+      s.pb[it] = inside ? (int)((unsigned)by * rowB + (unsigned)bx * pixB) : (int)NO_LOAD;
+    }
+#else
 #pragma unroll
     for (int it = 0; it < NV; ++it) {
       const int gy = y0 * SY + m.hy[it] - PY; // (y0, x0): the tile's first output pixel
@@ -370,15 +404,80 @@ struct Halo {
       const bool inside = m.lds[it] >= 0 && gy >= 0 && gy < (int)pc.IN_H && gx >= 0 && gx < (int)pc.IN_W;
       if (inside)
         src_offsets(gy, gx, pc, pa, pb);
-#if SRC_UNIFORM
-      s.pa[it] = inside ? (int)((unsigned)pa * 2u) : (int)NO_LOAD;
-      s.pb[it] = inside ? (int)((unsigned)pb * 2u) : (int)NO_LOAD;
-#else
       s.pa[it] = inside ? (int)pa : -1;
       s.pb[it] = (int)pb;
+    }
 #endif
+  }
+
+#if SRC_UNIFORM
+  // src_init in two parts, for a kernel that walks down a strip of tiles: the column of a vector's pixel, and with it
+  // everything src_init derives from gx, stays the same from tile to tile.  cols_init computes that part once per strip
+  // (byte offset of the column inside a source row, -1: no such vector or a column outside the image); rows_init adds
+  // the row: half a dozen 32-bit instructions per vector and no branch, where src_init takes some twenty with 64-bit
+  // multiplies -- instructions that a staging wave has to get issued between the matrix instructions of the
+  // computing wave on its SIMD.  Offsets are bytes below 4 GiB (the buffer resources address no more).
+  struct Cols {
+    int ca[NV], cb[NV];
+  };
+  // (t: the thread's index among the NTH, as for map_init; the halo column is derived again rather than kept in the
+  // map, whose hx then occupies no registers in a kernel that never calls src_init)
+  static __device__ DNX_INLINE void cols_init(Cols &c, int t, int x0, const PushConstants &pc) {
+#pragma unroll
+    for (int it = 0; it < NV; ++it) {
+      const int i = t + it * NTH;
+#if LAYIN
+      const int pix = i % HALO_PIX;
+#else
+      const int pix = i / VPPK;
+#endif
+      const int gx = x0 * SX + pix % HALO_W - PX;
+      const bool inside = i < HALO_PIX * VPPK && gx >= 0 && gx < (int)pc.IN_W;
+#if PADA
+      const int ax = clampi(gx - (int)pc.PAD_L, 0, (int)pc.SRC_W - 1);
+#else
+      const int ax = UPA ? (gx >> 1) : gx;
+#endif
+#if PADB
+      const int bx = clampi(gx - (int)pc.PAD_L, 0, (int)pc.SRC_W - 1);
+#else
+      const int bx = gx;
+#endif
+      c.ca[it] = inside ? ax * (LAYIN ? 16 : CA * 2) : -1;
+      c.cb[it] = inside ? bx * (LAYIN ? 16 : (CB > 0 ? CB : 1) * 2) : -1;
     }
   }
+  static __device__ DNX_INLINE void rows_init(Src &s, const Cols &c, const Map &m, int y0, const PushConstants &pc) {
+    const unsigned W = pc.IN_W;
+#if PADA
+    const unsigned rowA = pc.SRC_W * (unsigned)(LAYIN ? 16 : CA * 2);
+#else
+    const unsigned rowA = (UPA ? (W >> 1) : W) * (unsigned)(LAYIN ? 16 : CA * 2);
+#endif
+#if PADB
+    const unsigned rowB = pc.SRC_W * (unsigned)(LAYIN ? 16 : (CB > 0 ? CB : 1) * 2);
+#else
+    const unsigned rowB = W * (unsigned)(LAYIN ? 16 : (CB > 0 ? CB : 1) * 2);
+#endif
+#pragma unroll
+    for (int it = 0; it < NV; ++it) {
+      const int gy = y0 * SY + m.hy[it] - PY;
+      const bool inside = gy >= 0 && gy < (int)pc.IN_H && c.ca[it] >= 0;
+#if PADA
+      const int ay = clampi(gy - (int)pc.PAD_T, 0, (int)pc.SRC_H - 1);
+#else
+      const int ay = UPA ? (gy >> 1) : gy;
+#endif
+#if PADB
+      const int by = clampi(gy - (int)pc.PAD_T, 0, (int)pc.SRC_H - 1);
+#else
+      const int by = gy;
+#endif
+      s.pa[it] = inside ? (int)((unsigned)ay * rowA + (unsigned)c.ca[it]) : (int)NO_LOAD;
+      s.pb[it] = inside ? (int)((unsigned)by * rowB + (unsigned)c.cb[it]) : (int)NO_LOAD;
+    }
+  }
+#endif
 
   // Issue the loads of the L channels starting at c0 into registers ...
   template <int L>
