@@ -335,6 +335,35 @@ def test_fused_patterns_agree(oracle, features, CA, CB, K, H, W):
     assert n == (1 if not features else n)  # the default schedule is a single dispatch
 
 
+@pytest.mark.parametrize("config", ["s8r2k16", "w4r2k16", "m8r2k32x2", "q8r2k32x2", "t8r2k16", "x8r2k16"])
+@pytest.mark.parametrize("act", ["relu", "none"])
+def test_pooled_epilogue_equals_conv_then_pool(config, act):
+    """The fused epilogue takes the maximum of the four fp32 sums and finishes it once (bias, ReLU and rounding are
+    monotonic); the unfused schedule rounds all four and lets the stand-alone pool compare the halves.  Same values,
+    element for element (a zero's sign aside), on random data with negative and repeated values."""
+    rng = np.random.default_rng(11)
+    C, K, H, W = 32, 32, 44, 70
+    pair = config.startswith("x")
+    x = np.round(rng.standard_normal((H, W, C)) * 4).astype(np.float16) / 4  # a coarse grid: ties inside the windows
+    m = dx.Model()
+    t = m.input("input", "W", "H", C)
+    if pair:
+        t = m.relu(m.conv2d(t, he_weights(rng, 32, C), small_bias(rng, 32)))
+    y = m.conv2d(t, he_weights(rng, K, 32 if pair else C), small_bias(rng, K))
+    y = m.relu(y) if act == "relu" else y
+    m.output(m.pool(y))
+    fused = dx.Module.compile(m, conv_config=config)
+    assert fused.runtime_model.dispatch_count == 1 and config in dx.last_compile_report()
+    split = dx.Module.compile(m, conv_config=None if pair else config, features={"pool_fusion": False, "conv_conv_fusion": False})
+    assert split.runtime_model.dispatch_count == (3 if pair else 2)
+    got = fused.instance(H=H, W=W).infer(x)[0]
+    want = split.instance(H=H, W=W).infer(x)[0]
+    if pair:  # the fused pair sums the second convolution in another order than the stand-alone kernel: the conv tolerance
+        assert np.abs(got.astype(np.float32) - want.astype(np.float32)).max() <= 2e-2 * max(1.0, float(np.abs(want).max()))
+    else:
+        assert np.array_equal(got, want), f"{int((got != want).sum())} elements differ"
+
+
 IN_PLACE_CASES = [  # (C, K0, K1, tail): channel range aligned / not aligned to 16 bytes, narrow and wide, a pooled and an activated producer
     (8, 16, 24, "none"), (8, 16, 24, "conv"), (3, 3, 4, "none"), (9, 9, 16, "conv"), (16, 8, 3, "none"), (16, 64, 32, "conv"),
     (8, 16, 16, "pool"), (12, 40, 24, "relu"), (32, 48, 80, "conv")]
