@@ -595,7 +595,11 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     // computing wave wv - WAVES, after the chunk's memory work is under way
     auto rest = [&]() {
 #if C2STAGE
+      // (a raised wave priority for this part: its dozen matrix instructions compete with the computing wave's stream
+      // for the pipe, and the step ends when this wave is done: 2 - 3 % per launch)
+      __builtin_amdgcn_s_setprio(1);
       second(wv - WAVES);
+      __builtin_amdgcn_s_setprio(0);
       advance();
 #endif
     };
