@@ -105,7 +105,7 @@ def integer_pair(x, K1, K2):
 
 
 @pytest.mark.parametrize("config,C,density", [("x8r2k16", 8, 0.15), ("y4r2k32", 32, 0.04), ("z4r2k64", 64, 0.02), ("v4r2k64", 64, 0.02), ("v4r2k16", 8, 0.15), ("u4r2k32", 32, 0.04)])
-@pytest.mark.parametrize("H,W", [(33, 47), (288, 31), (1080, 1920)])
+@pytest.mark.parametrize("H,W", [(33, 47), (288, 31), (1080, 1920), (24, 9000)])  # the last: more strips than workgroups
 def test_pair_exact_on_small_integers(H, W, config, C, density):
     """Inputs in {0, 1}, all weights one: every intermediate and final value is an integer below 2048, which binary16
     holds exactly, so the fused kernel must reproduce integer arithmetic bit for bit -- at every strip and segment
