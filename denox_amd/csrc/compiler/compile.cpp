@@ -319,6 +319,12 @@ std::vector<uint8_t> compile(const Model &modelIn, const hip::HipCompiler &hipc,
     else out.inputs.push_back(relayout(t, f, dnx::TensorFormat::SSBO_HWC, true));
   }
 
+  // A tensor that lives inside another one (concat without a copy).  The tensor it lives in may itself be the source of a
+  // later concat, so buffers and offsets are resolved once every selected edge has been seen, by following each chain to
+  // the tensor that owns its memory (the reference unions the tensors with offsets, placement.cpp:232-255).
+  struct Alias { uint32_t parent; Sym offset; };
+  std::map<uint32_t, Alias> aliasOf;
+
   double total = 0.0;
   unsigned walk = 0; // alternates the tile walk of consecutive tiled dispatches
   for (size_t e : chosen) {
@@ -338,17 +344,14 @@ std::vector<uint8_t> compile(const Model &modelIn, const hip::HipCompiler &hipc,
     // implicit concat: src0 at offset 0, src1 behind it, dst aliases both (placement.cpp:253-255 of the reference)
     for (const auto &mc : edge.memoryConstrains) {
       const uint32_t a = place(mc.src0.index), b = place(mc.src1.index), dd = place(mc.dst.index);
-      out.tensors[a].buffer = out.tensors[dd].buffer;
-      out.tensors[b].buffer = out.tensors[dd].buffer;
-      out.tensors[a].offset = src(Sym::Const(0));
-      out.tensors[b].offset = out.tensors[a].size;
+      aliasOf[a] = Alias{dd, Sym::Const(0)};
+      aliasOf[b] = Alias{dd, g.tensors[mc.src0.index].byteSize};
     }
     // pixel-major concat without a copy: the source is a channel range of the destination, from its first channel
     // to the end of the destination
     for (const auto &vc : edge.viewConstrains) {
       const uint32_t a = place(vc.src.index), dd = place(vc.dst.index);
-      out.tensors[a].buffer = out.tensors[dd].buffer;
-      out.tensors[a].offset = src(Sym::Const(static_cast<int64_t>(vc.byteOffset)));
+      aliasOf[a] = Alias{dd, Sym::Const(static_cast<int64_t>(vc.byteOffset))};
       out.tensors[a].size = src(sym.sub(g.tensors[vc.dst.index].byteSize, static_cast<int64_t>(vc.byteOffset)));
     }
     total += cost[e];
@@ -356,6 +359,19 @@ std::vector<uint8_t> compile(const Model &modelIn, const hip::HipCompiler &hipc,
       report->schedule.push_back(ScheduleEntry{edge.shader, edge.config, edge.dispatches.empty() ? "" : edge.dispatches[0].info.name, cost[e], measured[e]});
       if (db && !measured[e]) report->warnings.push_back("no measured latency for " + edge.shader + " " + edge.config + "; used the roofline estimate");
     }
+  }
+
+  for (const auto &kv : aliasOf) {
+    uint32_t root = kv.second.parent;
+    Sym off = kv.second.offset;
+    size_t hops = 0;
+    for (auto it = aliasOf.find(root); it != aliasOf.end(); it = aliasOf.find(root)) {
+      if (++hops > aliasOf.size()) fail(Status::Internal, "tensors placed inside each other form a cycle");
+      off = sym.add(off, it->second.offset);
+      root = it->second.parent;
+    }
+    out.tensors[kv.first].buffer = out.tensors[root].buffer;
+    out.tensors[kv.first].offset = src(off);
   }
 
   for (size_t i = 0; i < model.outputs().size(); ++i) {

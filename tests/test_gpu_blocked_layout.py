@@ -133,6 +133,28 @@ def test_data_movement_on_blocked_tensors_is_bit_exact(oracle):
     assert_bits_equal(got, plain.instance(H=H, W=W).infer(x)[0], "blocked vs pixel-major")
 
 
+@pytest.mark.parametrize("widths", [(16, 24, 8), (64, 64, 64), (8, 24, 16, 40)])
+@pytest.mark.parametrize("features", [{}, BLOCKED], ids=["default", "blocked"])
+def test_concat_of_concats(oracle, widths, features):
+    """concat(concat(a, b), c) and a three-deep nest with channel counts that are multiples of 8: when the concats are
+    aliasing only, every leaf must land inside the outermost result.  Bit for bit against the schedule without block-major
+    tensors (which copies or writes in place per pixel), and against the oracle."""
+    from test_host import _nested_concat_model
+    m, _, out = _nested_concat_model(widths)
+    feats = dict(conv_conv_fusion=False)
+    mod = dx.Module.compile(m, conv_config="w4r2k16", features=dict(feats, **features))
+    plain = dx.Module.compile(m, conv_config="w4r2k16", features=dict(feats, blocked_layout=False))
+    rng = np.random.default_rng(5)
+    for H, W in [(32, 32), (19, 45)]:
+        x = rng.standard_normal((H, W, 16)).astype(np.float16)
+        got = mod.instance(H=H, W=W).infer(x)[0]
+        want = oracle.run_graph(m.to_ops({"H": H, "W": W}), {"input": x}, "fp32")[out.name]
+        assert_conv_close(got, want, f"nested concat {widths} {H}x{W}")
+        assert_bits_equal(got, plain.instance(H=H, W=W).infer(x)[0], f"nested concat {widths}: blocked vs pixel-major")
+    if features:
+        assert not any(n.startswith("concat") or n.startswith("copy") for n in entries(mod, H=32, W=32)), entries(mod, H=32, W=32)
+
+
 @pytest.mark.parametrize("H,W", [(64, 96), (75, 101), (16, 16), (33, 250)])
 def test_oidn_unet_with_blocked_internal_tensors(oracle, H, W):
     m, _ = networks.build("oidn_unet", seed=6)

@@ -247,6 +247,54 @@ def test_concat_sources_that_cannot_move():
 
 
 # ----------------------------------------------------------------------------- serialised model
+def _nested_concat_model(widths, depth_first=True):
+    """convs over one 16-channel input, concatenated pairwise into one tensor, then a conv over the lot."""
+    rng = np.random.default_rng(sum(widths))
+    m = dx.Model()
+    t = m.input("input", "W", "H", 16)
+    leaves = [m.relu(m.conv2d(t, (rng.standard_normal((k, 16, 3, 3)) * 0.1).astype(np.float16), (rng.standard_normal(k) * 0.01).astype(np.float16))) for k in widths]
+    acc = leaves[0]
+    for leaf in leaves[1:]:
+        acc = m.concat(acc, leaf) if depth_first else m.concat(leaf, acc)
+    total = sum(widths)
+    out = m.conv2d(acc, (rng.standard_normal((16, total, 3, 3)) * 0.05).astype(np.float16), np.zeros(16, np.float16))
+    m.output(out)
+    return m, leaves, out
+
+
+@pytest.mark.parametrize("widths", [(16, 24, 8), (64, 64, 64), (8, 24, 16, 40)])
+@pytest.mark.parametrize("features", [{}, {"layout_preference": 1}])
+def test_concat_of_concats_without_dispatches_shares_one_buffer(widths, features):
+    """A zero-dispatch (CHWC8) concat whose result is the source of another one: every leaf has to end up inside the
+    outermost result, at the sum of the offsets along the chain, not inside a buffer that the inner result has left."""
+    m, leaves, out = _nested_concat_model(widths)
+    H = W = 32
+    d = dx.describe(dx.compile_model(m, features=dict(features, conv_conv_fusion=False)), H=H, W=W)
+    names = [x["debug_info"].split(" | ")[0] for x in d["dispatches"]]
+    if any("concat" in x["name"] for x in d["dispatches"]):
+        pytest.skip(f"this selection copies: {names}")
+    act = [t for t in d["tensors"] if not t["param"] and t["format"] == 3]
+    by_channels = {}
+    for t in act:
+        by_channels.setdefault(t["channels"], []).append(t)
+    whole = by_channels[sum(widths)][0]
+    last = d["dispatches"][-1]
+    assert whole["buffer"] in [d["tensors"][b["tensor"]]["buffer"] for b in last["bindings"]], "the last conv reads the outermost concat"
+    # leaves, in concat order, tile the outermost tensor without gaps
+    leaf_tensors = sorted((t for t in act if t["buffer"] == whole["buffer"] and t["channels"] in widths and t is not whole), key=lambda t: t["offset"])
+    assert len(leaf_tensors) == len(widths), (len(leaf_tensors), names)
+    off = 0
+    for t, k in zip(leaf_tensors, widths):
+        assert t["offset"] == off and t["channels"] == k and t["size"] == H * W * k * 2, (t, off)
+        off += t["size"]
+    assert off == whole["size"]
+    # the partial concats start where the outermost one does
+    for c in itertools.accumulate(widths):
+        for t in by_channels.get(c, []):
+            if t["channels"] not in widths:
+                assert t["buffer"] == whole["buffer"] and t["offset"] == 0, t
+
+
 def test_dnx_round_trip_and_corruption():
     m, _ = networks.build("tiny_unet")
     blob = dx.compile_model(m)
