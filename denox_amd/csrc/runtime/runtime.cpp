@@ -22,6 +22,7 @@ Context::Context(int device) : m_device(device) {
   hipCheck(hipStreamCreateWithFlags(&m_stream, hipStreamNonBlocking), "hipStreamCreateWithFlags");
   try {
     m_staticScratch = staticScratchAddress(device); // set-up time: the allocation-free entry point must not have to ask
+    hipCheck(hipEventCreateWithFlags(&m_staticDone, hipEventDisableTiming), "hipEventCreateWithFlags");
   } catch (...) {
     (void)hipStreamDestroy(m_stream);
     throw;
@@ -29,6 +30,9 @@ Context::Context(int device) : m_device(device) {
 }
 
 Context::~Context() {
+  if (m_stream) (void)hipStreamSynchronize(m_stream);
+  staticScratchForget(m_device, this);
+  if (m_staticDone) (void)hipEventDestroy(m_staticDone);
   if (m_stream) (void)hipStreamDestroy(m_stream);
 }
 
@@ -364,10 +368,14 @@ void Instance::rebind(const void *const *inputs, void *const *outputs) {
     if (p != m_boundOutputs[i]) { changed = true; m_boundOutputs[i] = p; }
     out[i] = p ? p : tensorPtr(m.outputs[i]);
   }
-  if (!changed) return;
+  if (!changed && !m_graphStale) return;
   patchInterface(in, out);
   if (!m_useGraph) return; // plain launches read the argument buffers at launch time
+  // Until a graph for these addresses is in place the bindings count as unfinished: if the capture fails, the next call with
+  // the same addresses tries again instead of taking "nothing changed" for "a graph exists".
+  m_graphStale = true;
   selectGraph();
+  m_graphStale = false;
 }
 
 // Makes m_graph / m_graphExec the captured dispatch list for the interface addresses bound now (m_boundInputs /
@@ -540,6 +548,8 @@ void Instance::inferDeviceStatic(const void *const *inputs, void *const *outputs
   if (m_arenaBytes && !m_arena) fail(Status::Unsupported, "the allocation-free path needs the intermediate buffers in one arena (DENOX_HIP_NO_ALIAS is set)");
   if (!m_model->context()->staticScratch()) fail(Status::HipError, "the static scratch array has no device address");
   m_model->context()->makeCurrent();
+  const Context *ctx = m_model->context().get();
+  if (m_arenaBytes) staticScratchAcquire(ctx->device(), ctx);
   for (auto &l : m_launches)
     for (const auto &slot : l.ptrSlots) {
       if (slot.iface < 0) continue;
@@ -550,6 +560,7 @@ void Instance::inferDeviceStatic(const void *const *inputs, void *const *outputs
     }
   hipStream_t s = m_model->context()->stream();
   for (auto &l : m_launches) launchOne(l.fn, l.grid, l.block, l.staticArgs, s);
+  if (m_arenaBytes) staticScratchRecord(ctx->device(), ctx, ctx->staticScratchDone(), s);
 }
 
 void Instance::synchronize() {

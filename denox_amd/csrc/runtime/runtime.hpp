@@ -34,18 +34,27 @@ public:
   const hipDeviceProp_t &props() const { return m_props; }
   // this device's copy of the library's static scratch array (static_scratch.hip); resolved when the context is made
   void *staticScratch() const { return m_staticScratch; }
+  // recorded behind every call of the allocation-free entry point (created with the context: that call creates nothing)
+  hipEvent_t staticScratchDone() const { return m_staticDone; }
 
 private:
   int m_device;
   hipStream_t m_stream = nullptr;
   hipDeviceProp_t m_props;
   void *m_staticScratch = nullptr;
+  hipEvent_t m_staticDone = nullptr;
 };
 
 // The library's allocation-free path keeps intermediate results in a file-scope device array of this many bytes per GPU.
 constexpr uint64_t kStaticScratchBytes = 64ull << 20;
 // Device address of that array on `device`, which must be current (hipGetSymbolAddress once per device, then cached).
 void *staticScratchAddress(int device);
+// One user at a time per GPU.  Acquire: refuses (InvalidArgument) while a call made through another context is still running.
+// Record: marks `context` as the user, with `done` recorded on `stream` behind the launches.  Forget: a context that is being
+// destroyed (its stream already synchronized) gives the array up.
+void staticScratchAcquire(int device, const void *context);
+void staticScratchRecord(int device, const void *context, hipEvent_t done, hipStream_t stream);
+void staticScratchForget(int device, const void *context);
 using ContextHandle = std::shared_ptr<Context>;
 
 struct ModelDispatch {
@@ -126,7 +135,7 @@ public:
   void *inputDevicePtr(size_t i) const { return tensorPtr(m_model->dnx().inputs.at(i)); }
   void *outputDevicePtr(size_t i) const { return tensorPtr(m_model->dnx().outputs.at(i)); }
   uint64_t deviceBytes() const { return m_deviceBytes; }
-  bool usesGraph() const { return m_useGraph; }
+  bool usesGraph() const { return m_graphExec != nullptr; } // false while plain launches stand in (no graph wanted, or none captured yet)
 
 private:
   struct Launch {
@@ -166,6 +175,7 @@ private:
   std::vector<CachedGraph> m_graphCache;
   uint64_t m_graphUse = 0;
   bool m_useGraph = false;
+  bool m_graphStale = false; // the bound interface addresses have no captured graph yet (a capture failed)
   void selectGraph();
   void destroyGraphs();
   uint64_t m_deviceBytes = 0;

@@ -272,16 +272,24 @@ int denox_hip_instance_infer_many(denox_hip_instance *inst, uint32_t frames, con
 int denox_hip_host_alloc(size_t bytes, void **out);
 void denox_hip_host_free(void *p);
 /* asynchronous on the context's stream; device arrays, entries (or the arrays
- * themselves) may be NULL to use the instance's own tensors */
+ * themselves) may be NULL to use the instance's own tensors.  The dispatch list is captured into a graph once per set of
+ * interface addresses and the graphs of the last four sets are kept: a caller that rotates through more than four sets of
+ * buffers pays a stream synchronisation and a new capture per call (keep to four, or copy into fixed buffers). */
 int denox_hip_instance_infer_device(denox_hip_instance *inst, const void *const *dev_inputs, void *const *dev_outputs);
-/* denox_hip_instance_infer_device for callers that cannot allocate (code under HIP graph capture, serving loops and
- * harnesses that forbid hipMalloc): same arguments, same results bit for bit, and no allocation of any kind on the
- * device -- plain kernel launches on the context's stream (no graph is captured or instantiated), with the instance's
- * intermediate tensors kept in a static device array that the library holds on every GPU it runs on
- * (DENOX_HIP_STATIC_SCRATCH_BYTES, resolved when the context is created).  It has no counterpart in the reference,
- * whose Instance allocates every buffer it uses (runtime/src/denox/runtime/instance.cpp:65-113).
- * Returns DENOX_HIP_UNSUPPORTED, with the size needed in the error text, when the instance's intermediate tensors need more than that.  All instances on one GPU share the array and each call
- * overwrites it: calls that overlap in time on one GPU race, and nothing in it survives from one call to the next. */
+/* denox_hip_instance_infer_device for callers that cannot allocate (serving loops and harnesses that forbid hipMalloc and
+ * its relatives once they are running): same arguments, same results bit for bit, and no allocation of any kind on the
+ * device or through the runtime -- plain kernel launches on the context's stream (no graph is captured or instantiated;
+ * the launches go to the context's own stream, so a caller that is capturing a stream of its own does not capture them),
+ * with the instance's intermediate tensors kept in a static device array that the library holds on every GPU it runs on
+ * (DENOX_HIP_STATIC_SCRATCH_BYTES of device memory per GPU and process from the moment the library is loaded there,
+ * used or not, and not counted in denox_hip_instance_device_bytes; its address is resolved when the context is created).
+ * It has no counterpart in the reference, whose Instance allocates every buffer it uses
+ * (runtime/src/denox/runtime/instance.cpp:65-113).
+ * Returns DENOX_HIP_UNSUPPORTED, with the size needed in the error text, when the instance's intermediate tensors need more
+ * than that.  All instances on one GPU share the array and each call overwrites it; nothing in it survives from one call to
+ * the next.  Calls through one context are ordered by its stream.  Calls through different contexts of one GPU are not:
+ * while an earlier call through another context has not finished, the call is refused with DENOX_HIP_INVALID_ARGUMENT
+ * (synchronize the other context first) rather than run into that call's tensors. */
 #define DENOX_HIP_STATIC_SCRATCH_BYTES (64ull << 20)
 int denox_hip_instance_infer_device_static(denox_hip_instance *inst, const void *const *dev_inputs, void *const *dev_outputs);
 int denox_hip_instance_synchronize(denox_hip_instance *inst);

@@ -163,8 +163,8 @@ def test_oidn_unet_with_blocked_internal_tensors(oracle, H, W):
     fmts = internal_formats(mod, H=H, W=W)
     assert fmts.count(3) >= 5, fmts
     got = mod.instance(H=H, W=W).infer(x)[0]
-    want = oracle.run_graph(m.to_ops({"H": H, "W": W}), {"input": x}, "fp32")[m.outputs[0].name]
-    assert_conv_close(got, want, f"oidn blocked {H}x{W}")
+    from test_gpu_unet import check_net
+    check_net(oracle, m, x, got, H, W, f"oidn blocked {H}x{W}")
 
 
 def test_full_size_oidn_unet_blocked(oracle):

@@ -5,7 +5,7 @@ torch (test/__init__.py:45-101).  Here the same layers are built with the graph 
 layouts are used, and the expectation comes from the CPU oracle: bit-exact for data movement, the fp32-evaluation
 tolerance for convs.
 
-  test_conv.py:126-501        conv3x3 'same', (C_in, C_out) below, HWC and CHWC8 interfaces and mixed
+  test_conv.py:9-501          conv3x3 'same', all 50 cases: HWC, CHWC8 and mixed interfaces, up to 256 -> 256
   test_conv_relu.py:20-94     conv3x3 + ReLU
   test_max_pool.py            MaxPool2d(2, 2), C in {3, 8, 9, 16, 24, 32, 48, 64, 80} HWC, {8..80} CHWC8
   test_upsampling.py          Upsample(scale_factor=2), same channel sets
@@ -59,20 +59,25 @@ def run_case(oracle, build, C, in_layout=HWC, out_layout=HWC, H=100, W=100, exac
         assert_reference_allclose(got, oracle.run_graph(m.to_ops({"H": H, "W": W}), {"input": x}, "f16")[t.name])
 
 
-CONV_SHAPES = [(3, 3), (3, 32), (32, 3), (8, 16), (16, 8), (16, 32), (32, 16), (32, 32), (64, 64), (24, 24), (32, 48), (48, 48),
-               (64, 32), (64, 80), (67, 64), (80, 96), (96, 96), (112, 112), (128, 64), (160, 96), (160, 112)]
+# test_conv.py of the reference, case for case: (input channels, input layout, output channels, output layout).  The reference
+# relaxes its own bar for the wide ones (128: atol 1e-2, rtol 0; 256: atol 1e-1, rtol 0; test_conv.py:100-123,282-290,322-330,
+# 394-417,478-501); here every case is held to the same two bars, so nothing is relaxed.
+H_, C8 = "hwc", "chwc8"
+REFERENCE_CONV_CASES = (
+    [(ci, H_, co, H_) for ci, co in [(3, 3), (3, 32), (32, 3), (8, 16), (16, 8), (16, 32), (32, 16), (24, 24), (32, 32), (64, 64), (128, 128), (256, 256)]] +
+    [(ci, C8, co, C8) for ci, co in [(8, 16), (16, 8), (16, 32), (32, 16), (32, 32), (32, 48), (48, 48), (64, 64), (96, 96), (128, 64), (64, 32), (128, 128),
+                                     (160, 112), (112, 112), (160, 96), (256, 256)]] +
+    [(64, C8, 80, H_), (80, H_, 96, H_), (96, H_, 96, C8), (128, C8, 64, H_), (67, H_, 64, C8), (32, C8, 3, H_)] +
+    [(ci, H_, co, C8) for ci, co in [(8, 16), (16, 8), (16, 32), (32, 16), (32, 32), (64, 64), (128, 128), (256, 256)]] +
+    [(ci, C8, co, H_) for ci, co in [(8, 16), (16, 8), (16, 32), (32, 16), (32, 32), (64, 64), (128, 128), (256, 256)]])
+# shapes of this build's own networks that the reference's list lacks
+EXTRA_CONV_CASES = [(ci, H_, co, H_) for ci, co in [(32, 48), (48, 48), (64, 32), (64, 80), (67, 64), (96, 96), (112, 112), (128, 64), (160, 96), (160, 112)]]
 
 
-@pytest.mark.parametrize("cin,cout", CONV_SHAPES)
-def test_conv_hwc(oracle, cin, cout):
-    run_case(oracle, lambda m, x, rng: m.conv2d(x, he_weights(rng, cout, cin), small_bias(rng, cout)), cin, exact=False)
-
-
-@pytest.mark.parametrize("cin,cout,li,lo", [(8, 16, CHWC8, CHWC8), (16, 8, CHWC8, CHWC8), (16, 32, CHWC8, CHWC8), (32, 16, CHWC8, CHWC8),
-                                            (32, 32, CHWC8, CHWC8), (64, 64, CHWC8, CHWC8), (96, 96, CHWC8, CHWC8), (128, 64, CHWC8, CHWC8),
-                                            (8, 16, HWC, CHWC8), (16, 8, CHWC8, HWC), (32, 32, HWC, CHWC8), (64, 64, CHWC8, HWC)])
-def test_conv_chwc8_and_mixed_interfaces(oracle, cin, cout, li, lo):
-    run_case(oracle, lambda m, x, rng: m.conv2d(x, he_weights(rng, cout, cin), small_bias(rng, cout)), cin, li, lo, exact=False)
+@pytest.mark.parametrize("cin,li,cout,lo", REFERENCE_CONV_CASES + EXTRA_CONV_CASES, ids=lambda v: str(v))
+def test_conv(oracle, cin, li, cout, lo):
+    lay = {H_: HWC, C8: CHWC8}
+    run_case(oracle, lambda m, x, rng: m.conv2d(x, he_weights(rng, cout, cin), small_bias(rng, cout)), cin, lay[li], lay[lo], exact=False)
 
 
 @pytest.mark.parametrize("cin,cout", [(3, 3), (3, 32), (32, 3), (8, 16), (16, 8), (16, 32), (32, 16), (32, 32), (64, 64)])

@@ -12,7 +12,7 @@ import pytest
 
 import denox_amd as dx
 from denox_amd import networks
-from util import assert_bits_equal, assert_conv_close
+from util import assert_bits_equal, assert_conv_close, assert_reference_allclose
 
 pytestmark = pytest.mark.gpu
 
@@ -21,13 +21,19 @@ def oracle_net(oracle, model, x, H, W, mode="fp32"):
     return oracle.run_graph(model.to_ops({"H": H, "W": W}), {"input": x}, mode)[model.outputs[0].name]
 
 
+def check_net(oracle, model, x, got, H, W, what):
+    """The stated bar against the fp32 evaluation; where the outputs are too large for binary16 tensors to meet it (the U-Net on
+    colour values up to 64), a small multiple of the binary16-storage evaluation's own error (util.assert_conv_close)."""
+    assert_conv_close(got, oracle_net(oracle, model, x, H, W), what, floor=lambda: oracle_net(oracle, model, x, H, W, "f16"))
+
+
 @pytest.mark.parametrize("H,W", [(128, 128), (37, 61), (2, 2)])
 def test_tiny_unet(oracle, H, W):
     H2, W2 = H // 2 * 2, W // 2 * 2  # the un-wrapped tiny net needs even extents
     m, _ = networks.build("tiny_unet", seed=3)
     x = networks.synthetic_input("tiny_unet", H2, W2, seed=3)
     got = dx.Module.compile(m).instance(H=H2, W=W2).infer(x)[0]
-    assert_conv_close(got, oracle_net(oracle, m, x, H2, W2), f"tiny {H2}x{W2}")
+    check_net(oracle, m, x, got, H2, W2, f"tiny {H2}x{W2}")
 
 
 @pytest.mark.parametrize("H,W", [(64, 96), (75, 101), (16, 16), (1, 1), (33, 250)])
@@ -38,7 +44,7 @@ def test_oidn_unet_small_extents(oracle, H, W):
     inst = mod.instance(H=H, W=W)
     got = inst.infer(x)[0]
     assert got.shape == (H, W, 3)
-    assert_conv_close(got, oracle_net(oracle, m, x, H, W), f"oidn {H}x{W}")
+    check_net(oracle, m, x, got, H, W, f"oidn {H}x{W}")
     # a second frame through the same instance (graph replay) and determinism
     again = inst.infer(x)[0]
     assert_bits_equal(again, got, "replay")
@@ -51,7 +57,7 @@ def test_oidn_unet_one_model_many_extents(oracle):
     for H, W in [(48, 80), (50, 70), (80, 48)]:
         x = networks.synthetic_input("oidn_unet", H, W, seed=H)
         got = mod.instance(H=H, W=W).infer(x)[0]
-        assert_conv_close(got, oracle_net(oracle, m, x, H, W), f"oidn dyn {H}x{W}")
+        check_net(oracle, m, x, got, H, W, f"oidn dyn {H}x{W}")
     with pytest.raises(dx.DenoxHipError):
         mod.instance(H=48)  # W missing
 
@@ -66,7 +72,7 @@ def test_double_width_unet_chw_interface(oracle):
     assert inst.input_desc()["layout"] == dx.Layout.CHW and inst.output_desc()["layout"] == dx.Layout.CHW
     got = inst.infer(np.ascontiguousarray(x.transpose(2, 0, 1)))[0]
     assert got.shape == (3, H, W)
-    assert_conv_close(got.transpose(1, 2, 0), oracle_net(oracle, m, x, H, W), "2x width CHW")
+    check_net(oracle, m, x, got.transpose(1, 2, 0), H, W, "2x width CHW")
 
 
 def test_chwc8_interface_bit_exact(oracle):
@@ -277,22 +283,16 @@ def test_full_size_oidn_unet_centre_of_crop(oracle):
     x = networks.synthetic_input("oidn_unet", FULL_H, FULL_W, seed=0)
     got = dx.Module.compile(m, assume={"H": FULL_H, "W": FULL_W}).instance(H=FULL_H, W=FULL_W).infer(x)[0]
     assert got.shape == (FULL_H, FULL_W, 3) and np.isfinite(got).all()
-    S, Mg = 272, 96
-    for y0, x0 in [(0, 0), (400, 800), (FULL_H - S + 8, FULL_W - S)]:  # last crop reaches the replicate-padded bottom rows
-        y0 -= y0 % 16
-        x0 -= x0 % 16
-        h = min(S, FULL_H - y0)
-        crop = np.ascontiguousarray(x[y0:y0 + h, x0:x0 + S])
-        want = oracle_net(oracle, m, crop, h, S)
-        ys = slice(0 if y0 == 0 else Mg, h if y0 + h >= FULL_H else h - Mg)
-        xs = slice(0 if x0 == 0 else Mg, S if x0 + S >= FULL_W else S - Mg)
-        assert_conv_close(got[y0:y0 + h, x0:x0 + S][ys, xs], want[ys, xs], f"crop at {(y0, x0)}")
+    # the last crop reaches the replicate-padded bottom rows
+    check_crops(oracle, m, x, got, FULL_H, FULL_W, [(0, 0), (400, 800), (FULL_H - 272 + 8, FULL_W - 272)], "1080p")
 
 
-def check_crops(oracle, m, x_hwc, got_hwc, H, W, spots, what, S=272, Mg=96):
+def check_crops(oracle, m, x_hwc, got_hwc, H, W, spots, what, S=272, Mg=96, floor_relative=True, reference_bar=False):
     """`got_hwc` (the full frame) against the oracle on 16-aligned S x S crops of the input: the U-Net's receptive field is
     below Mg pixels, so a crop evaluation equals the full-frame result Mg pixels inside every cut edge (true image edges
-    keep their own padding and are compared up to the border)."""
+    keep their own padding and are compared up to the border).  `floor_relative`: the bar may rise to a small multiple of the
+    binary16-storage evaluation's error (see check_net); `reference_bar`: also the reference's own acceptance, allclose with
+    rtol 1e-3 / atol 1e-2 against the binary16-storage evaluation (test/__init__.py:45-49,97 of the reference)."""
     for y0, x0 in spots:
         y0 -= y0 % 16
         x0 -= x0 % 16
@@ -301,7 +301,31 @@ def check_crops(oracle, m, x_hwc, got_hwc, H, W, spots, what, S=272, Mg=96):
         want = oracle_net(oracle, m, crop, h, w)
         ys = slice(0 if y0 == 0 else Mg, h if y0 + h >= H else h - Mg)
         xs = slice(0 if x0 == 0 else Mg, w if x0 + w >= W else w - Mg)
-        assert_conv_close(got_hwc[y0:y0 + h, x0:x0 + w][ys, xs], want[ys, xs], f"{what}: crop at {(y0, x0)}")
+        g = got_hwc[y0:y0 + h, x0:x0 + w][ys, xs]
+        floor = (lambda: oracle_net(oracle, m, crop, h, w, "f16")[ys, xs]) if (reference_bar or floor_relative) else None
+        assert_conv_close(g, want[ys, xs], f"{what}: crop at {(y0, x0)}", floor=floor if floor_relative else None)
+        if reference_bar:
+            assert_reference_allclose(g, floor(), f"{what}: crop at {(y0, x0)}")
+
+
+@pytest.mark.parametrize("tuned", [False, True], ids=["default-schedule", "tuned-schedule"])
+def test_full_size_oidn_unet_reference_input_distribution(oracle, tmp_path, tuned):
+    """The reference's own acceptance at the benchmark extent.  Its system tests feed `torch.rand` images (uniform [0, 1),
+    test/system/test_unet.py) and accept allclose(rtol 1e-3, atol 1e-2) against a binary16 evaluation
+    (test/__init__.py:45-49,97).  On that input distribution the U-Net's outputs stay below 4, and the HIP path has to meet
+    both bars as stated, with nothing scaled: 2e-2 / 2e-3 against the fp32 evaluation and the reference's allclose against
+    the binary16-storage evaluation -- for the default schedule and for one selected from a timing table measured here."""
+    m, _ = networks.build("oidn_unet", seed=0)
+    x = np.random.default_rng(0).random((FULL_H, FULL_W, 9), dtype=np.float32).astype(np.float16)
+    db = None
+    if tuned:
+        db = dx.Db(str(tmp_path / "gpu.db"))
+        db.populate(m, assume={"H": FULL_H, "W": FULL_W})
+        db.bench(min_samples=5, max_relative_error=0.05, max_samples=20)
+    blob = dx.compile_model(m, assume={"H": FULL_H, "W": FULL_W}, db=db)
+    got = dx.Module.load(blob).instance(H=FULL_H, W=FULL_W).infer(x)[0]
+    check_crops(oracle, m, x, got, FULL_H, FULL_W, [(0, 0), (400, 800), (FULL_H - 272 + 8, FULL_W - 272), (600, 0)], "uniform input",
+                floor_relative=False, reference_bar=True)
 
 
 def test_full_size_4k_oidn_unet_centre_of_crop(oracle):

@@ -60,3 +60,32 @@ def test_static_scratch_entry_point_refuses_what_does_not_fit():
     with pytest.raises(dx.DenoxHipError) as e:
         inst.infer_device_static(None, None)
     assert "static scratch" in str(e.value)
+
+
+def test_static_scratch_is_not_shared_by_calls_that_overlap():
+    """Two contexts of one GPU launch on two streams and share the one array.  While calls made through the first are still
+    running, a call through the second is refused (INVALID_ARGUMENT) instead of overwriting their tensors; once the first
+    context has been synchronized the second runs and gives the bits of its graph path."""
+    torch = pytest.importorskip("torch")
+    m, _ = networks.build("oidn_unet", seed=21)
+    blob = dx.compile_model(m)
+    H, W = 256, 448  # about 30 MiB of intermediate tensors: a call lasts a few hundred microseconds
+    a = dx.Module.load(blob, dx.Context(0)).instance(H=H, W=W)
+    b = dx.Module.load(blob, dx.Context(0)).instance(H=H, W=W)
+    x = networks.synthetic_input("oidn_unet", H, W, seed=3)
+    want = b.infer(x)[0]
+    a.infer(x)
+    d_out = torch.full((H, W, 3), float("nan"), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    for _ in range(40):  # milliseconds of queued work on the first context's stream
+        a.infer_device_static(None, None)
+    with pytest.raises(dx.DenoxHipError) as e:
+        b.infer_device_static(None, [d_out.data_ptr()])
+    assert e.value.status == 1 and "another context" in str(e.value)
+    a.synchronize()
+    b.infer_device_static(None, [d_out.data_ptr()])
+    b.synchronize()
+    assert_bits_equal(d_out.cpu().numpy(), want, "second context after the first has finished")
+    # and back: the first context may take the array again once the second's call is done
+    a.infer_device_static(None, None)
+    a.synchronize()

@@ -1,9 +1,8 @@
 """Helpers shared by the GPU parity tests: seeded tensors and the parity bar."""
 import numpy as np
 
-# north-star tolerance for conv outputs, on the final fp16 output against an fp32 evaluation
-CONV_MAX_ABS = 2e-2
-CONV_MEAN_ABS = 2e-3
+# the bars live beside the checker, which bench.py's parity leg uses as well
+from oracle import CONV_MAX_ABS, CONV_MEAN_ABS, FLOOR_FACTOR_MAX, FLOOR_FACTOR_MEAN, conv_parity  # noqa: F401
 
 
 def he_weights(rng, K, C, R=3, S=3):
@@ -14,16 +13,21 @@ def small_bias(rng, K):
     return (rng.standard_normal(K) * 0.01).astype(np.float16)
 
 
-def assert_conv_close(got_f16, want_f32, what=""):
-    got = np.asarray(got_f16, np.float32)
-    want = np.asarray(want_f32, np.float32)
-    assert got.shape == want.shape, (got.shape, want.shape)
-    assert np.isfinite(got).all(), f"{what}: non-finite output"
-    err = np.abs(got - want)
-    # the bar is absolute on outputs of O(1) magnitude; scale it for layers whose outputs are larger
-    scale = max(1.0, float(np.abs(want).max()))
-    assert err.max() <= CONV_MAX_ABS * scale, f"{what}: max abs err {err.max():.4g} (scale {scale:.3g}) at {np.unravel_index(err.argmax(), err.shape)}"
-    assert err.mean() <= CONV_MEAN_ABS * scale, f"{what}: mean abs err {err.mean():.4g}"
+def assert_conv_close(got_f16, want_f32, what="", floor=None):
+    """max abs <= 2e-2 and mean abs <= 2e-3 against the fp32 evaluation; where that is out of reach of binary16 storage, at most
+    FLOOR_FACTOR_MAX / FLOOR_FACTOR_MEAN times the error of the oracle's binary16-storage evaluation (`floor`)."""
+    r = conv_parity(got_f16, want_f32, floor)
+    assert r["finite"], f"{what}: non-finite output"
+    note = "" if r["floor_max_abs"] is None else f" (binary16-storage floor {r['floor_max_abs']:.4g} / {r['floor_mean_abs']:.4g})"
+    if not r["literal_ok"] and floor is None:
+        note = " (no binary16-storage floor was given for this case: the absolute bar applies)"
+    assert r["max_abs"] <= r["bar_max_abs"], f"{what}: max abs err {r['max_abs']:.4g} > {r['bar_max_abs']:.4g}{note} at {r['argmax']}"
+    assert r["mean_abs"] <= r["bar_mean_abs"], f"{what}: mean abs err {r['mean_abs']:.4g} > {r['bar_mean_abs']:.4g}{note}"
+
+
+def f16_floor(oracle, ops, inputs, name):
+    """The binary16-storage evaluation of a graph, for `assert_conv_close(..., floor=...)`; evaluated only when needed."""
+    return lambda: oracle.run_graph(ops, inputs, "f16")[name]
 
 
 def assert_reference_allclose(got_f16, want_f16, what="", rtol=1e-3, atol=1e-2):
