@@ -629,10 +629,14 @@ private:
 // ck: input channels of the first convolution per LDS stage; pw: extra waves that only move halos (the others then only compute)
 // w1reg: the first convolution's weights in registers of the computing waves (needs pw)
 // c2stage: the second convolution, its epilogue and its stores on the staging waves (needs pw == waves)
-struct PairConfig { unsigned waves, rpw, ck; const char *name; unsigned pw = 0; bool w1reg = false; bool c2stage = false; };
+// dlds: halos loaded from memory straight into LDS by the staging waves (DLDS in conv_common.h; needs pw, channel counts that
+// are multiples of 8 and every LDS stage inside one source); nbuf: halo buffers (3: those loads are issued two stages ahead)
+struct PairConfig { unsigned waves, rpw, ck; const char *name; unsigned pw = 0; bool w1reg = false; bool c2stage = false; bool dlds = false; unsigned nbuf = 2; };
 const PairConfig kPairConfigs[] = {{8, 2, 16, "x8r2k16"}, {4, 2, 32, "x4r2k32"}, {4, 4, 16, "x4r4k16"}, {4, 2, 16, "x4r2k16"},
                                    {4, 2, 32, "y4r2k32", 4}, {4, 2, 64, "z4r2k64", 4, true},
-                                   {4, 2, 64, "v4r2k64", 4, true, true}, {4, 2, 16, "v4r2k16", 4, true, true}, {4, 2, 32, "u4r2k32", 4, false, true}};
+                                   {4, 2, 64, "v4r2k64", 4, true, true}, {4, 2, 16, "v4r2k16", 4, true, true}, {4, 2, 32, "u4r2k32", 4, false, true},
+                                   {4, 2, 64, "d4r2k64", 4, true, true, true},
+                                   {4, 2, 32, "t4r2k32", 4, false, true, true, 3}};
 constexpr unsigned kNumPairConfigs = sizeof(kPairConfigs) / sizeof(kPairConfigs[0]);
 
 bool isPairConfigName(const std::string &name) {
@@ -649,6 +653,7 @@ bool choosePair(const PairConfig &cfg, unsigned CA, unsigned CB, unsigned K1, un
   g.ck = std::min(cfg.ck, g.CPAD);
   const unsigned ih = cfg.waves * cfg.rpw, haloPix = (ih + 2) * 34, ckp = g.ck + 8, threads = (cfg.pw ? cfg.pw : cfg.waves) * 64; // threads that move halos
   if ((haloPix * (g.ck / 8) + threads - 1) / threads > 64) return false;
+  if (cfg.dlds && (!cfg.pw || CA % 8 || CB % 8 || (CB && CA % g.ck))) return false;
   const unsigned regBudget = std::min(256u, 512u / ((cfg.waves + cfg.pw + 3) / 4));
   // A second convolution with at most 5 output channels carries its three filter columns in the matrix rows (TAPM in
   // conv3x3_pair.hip): a third of the matrix instructions, weights of 3 instead of 9 taps in registers.
@@ -657,13 +662,15 @@ bool choosePair(const PairConfig &cfg, unsigned CA, unsigned CB, unsigned K1, un
   if ((g.tapm ? 24 : 72) + cfg.rpw * 16 + 96 > regBudget) return false;
   if (cfg.c2stage) {
     // a staging wave then holds, besides its two sets of halo registers, what the second convolution needs
-    const unsigned nv = (haloPix * (g.ck / 8) + threads - 1) / threads;
+    const unsigned nv = cfg.dlds ? 0 : (haloPix * (g.ck / 8) + threads - 1) / threads; // (straight into LDS: no halo registers)
     if (cfg.pw != cfg.waves || 2 * nv * 4 + (g.tapm ? 24 : 72) + cfg.rpw * 16 + 2 * (cfg.rpw + 2) * 4 + 48 > regBudget) return false;
   }
   const unsigned nchunk = (g.CPAD + g.ck - 1) / g.ck;
   const unsigned ringRows = nchunk == 1 ? 2 * ih + 2 : ih + 2; // see conv3x3_pair.hip
   if (cfg.w1reg && 9 * (g.CPAD / 16) * 4 > 144) return false; // the first convolution's weights must fit the register file next to everything else
-  g.ldsBytes = (cfg.w1reg ? 0 : static_cast<size_t>(9 * 32) * (g.CPAD + 8) * 2) + 2 * static_cast<size_t>(haloPix) * ckp * 2 + (static_cast<size_t>(ringRows) * 32 + 2) * 40 * 2 + 2 * 32 * 4;
+  // (straight into LDS: unpadded pixels, whole loads of all staging threads)
+  const size_t haloBytes = cfg.dlds ? static_cast<size_t>((haloPix * (g.ck / 8) + threads - 1) / threads) * threads * 16 : static_cast<size_t>(haloPix) * ckp * 2;
+  g.ldsBytes = (cfg.w1reg ? 0 : static_cast<size_t>(9 * 32) * (g.CPAD + 8) * 2) + cfg.nbuf * haloBytes + (static_cast<size_t>(ringRows) * 32 + 2) * 40 * 2 + 2 * 32 * 4;
   if (g.ldsBytes > dev.maxComputeSharedMemory) return false;
   g.slots = std::max(1u, dev.computeUnits / dev.xcdCount);
   return true;
@@ -822,6 +829,8 @@ public:
     if (cfg.pw) k.define("PW", cfg.pw);
     if (cfg.w1reg) k.define("W1REG", 1);
     if (cfg.c2stage) k.define("C2STAGE", 1);
+    if (cfg.dlds) k.define("DLDS", 1);
+    if (cfg.nbuf != 2) k.define("NBUF", cfg.nbuf);
     const bool blockedIn = !m.inputFormats.empty() && m.inputFormats[0] != 0, blockedOut = m.outputFormat != 0;
     if (blockedIn) k.define("LAYIN", 1);
     if (blockedOut) k.define("LAYOUT_OUT", 1);

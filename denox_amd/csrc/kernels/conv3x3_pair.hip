@@ -72,6 +72,10 @@
 #ifndef C2STAGE
 #define C2STAGE 0
 #endif
+#ifndef NBUF
+#define NBUF 2 // halo buffers.  3 (with DLDS): the loads of chunk c + 2 are issued while chunk c is multiplied, a whole chunk earlier
+#endif
+static_assert(NBUF == 2 || (NBUF == 3 && DLDS), "a third halo buffer serves loads that go straight into LDS");
 static_assert(!C2STAGE || PW == WAVES, "second convolution on the staging waves: one staging wave per computing wave");
 static_assert(!TAPM || (3 * KOUT <= 15 && !POOL), "filter columns in the matrix rows: at most 5 output channels, no pooling");
 
@@ -253,7 +257,12 @@ template <int L, int WPITCH>
 __device__ DNX_INLINE void mma_first(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, int wv, int lane) {
   const int l32 = lane & 31;
   const int kq = (lane >> 5) * 8;
+#if DLDS
+  PxBase pxb;
+  px_base_init(pxb, sIn, wv * RPW, lane);
+#else
   lds_half_t *pxb = lds_opaque(sIn + (wv * RPW * HALO_W + l32) * CKP + kq);
+#endif
   lds_half_t *wb = lds_opaque(sW + l32 * WPITCH + wofs + kq);
   constexpr int NG = 3 * (L / 16);
   half8 px[2][PXROWS], wf[2][3];
@@ -261,7 +270,11 @@ __device__ DNX_INLINE void mma_first(const _Float16 *sIn, const _Float16 *sW, in
     const int s = g / (L / 16), ks = g % (L / 16);
 #pragma unroll
     for (int hr = 0; hr < PXROWS; ++hr)
+#if DLDS
+      px[g & 1][hr] = PX_READ(pxb, hr, s, ks);
+#else
       px[g & 1][hr] = *reinterpret_cast<lds_half8_t *>(pxb + (hr * HALO_W + s) * CKP + ks * 16);
+#endif
 #pragma unroll
     for (int r = 0; r < 3; ++r)
       wf[g & 1][r] = *reinterpret_cast<lds_half8_t *>(wb + ((r * 3 + s) * 32) * WPITCH + ks * 16);
@@ -301,14 +314,23 @@ template <int L, int CHUNK>
 __device__ DNX_INLINE void mma_first_reg(const _Float16 *sIn, const FirstWeights &fw, Acc &acc, int wv, int lane) {
   const int l32 = lane & 31;
   const int kq = (lane >> 5) * 8;
+#if DLDS
+  PxBase pxb;
+  px_base_init(pxb, sIn, wv * RPW, lane);
+#else
   lds_half_t *pxb = lds_opaque(sIn + (wv * RPW * HALO_W + l32) * CKP + kq);
+#endif
   constexpr int NG = 3 * (L / 16);
   half8 px[2][PXROWS];
   auto load = [&](int g) {
     const int s = g / (L / 16), ks = g % (L / 16);
 #pragma unroll
     for (int hr = 0; hr < PXROWS; ++hr)
+#if DLDS
+      px[g & 1][hr] = PX_READ(pxb, hr, s, ks);
+#else
       px[g & 1][hr] = *reinterpret_cast<lds_half8_t *>(pxb + (hr * HALO_W + s) * CKP + ks * 16);
+#endif
   };
   load(0);
 #pragma unroll
@@ -385,7 +407,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
 #if !W1REG
   __shared__ __attribute__((aligned(16))) _Float16 sW1[NTAPS * 32 * CPADP];
 #endif
-  __shared__ __attribute__((aligned(16))) _Float16 sIn[2][HALO_PIX * CKP];
+  __shared__ __attribute__((aligned(16))) _Float16 sIn[NBUF][HALO_ELEMS];
   __shared__ __attribute__((aligned(16))) _Float16 sMid[(NS * IW + 2) * C2P];
   __shared__ __attribute__((aligned(16))) bias_t sBias1[32];
   __shared__ __attribute__((aligned(16))) bias_t sBias2[32];
@@ -450,12 +472,12 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   // ---- the fetch cursor walks the same sequence of (unit, step, channel chunk) as the compute cursor, two chunks ahead.
   // Every unit has one step more than it has rows for: the last one only drains the second convolution, its loads are
   // aimed past the end of the sources (they return zeros without touching memory) and its matrix work is skipped. ----
+  Geo fg = geometry(unit);
+  int funit = unit, fk = 0, fchunk = 0;
   typedef Halo<(PW > 0 ? PW : WAVES) * 64> H;
   H::Map map;
   H::Src fsrc;
   H::map_init(map, PW > 0 ? tid - WAVES * 64 : tid); // (computing waves of the specialised variant never use it)
-  Geo fg = geometry(unit);
-  int funit = unit, fk = 0, fchunk = 0;
 #if SRC_UNIFORM
   H::Cols fcols; // the column part of the offsets: one strip, one set of columns
   H::cols_init(fcols, PW > 0 ? tid - WAVES * 64 : tid, fg.xs - 1, pc);
@@ -488,6 +510,25 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
       }
     }
   };
+#if DLDS
+  // the halo of the fetch cursor's chunk straight into `dst`, and the cursor one chunk on (as issue() above)
+  auto dma = [&](_Float16 *dst) {
+    if (fchunk == 0)
+      aim();
+    H::dma_step(srcs, dst, map, fsrc, fchunk, wv - WAVES);
+    if (++fchunk == NCHUNK) {
+      fchunk = 0;
+      if (funit < units && ++fk > fg.steps) {
+        fk = 0;
+        funit += GRID;
+        if (funit < units) {
+          fg = geometry(funit);
+          H::cols_init(fcols, tid - WAVES * 64, fg.xs - 1, pc);
+        }
+      }
+    }
+  };
+#endif
 
   Geo g = geometry(unit);
   int k = 0, cchunk = 0, buf = 0;
@@ -495,21 +536,32 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   Acc acc;       // the first convolution's accumulators during a step's chunks, the second's in between
   // outputs of step k - 1, in the first chunk of step k: its `mid` rows and the two before them are in the ring.
   // rw: the wave whose rows these are
-  auto second = [&](int rw) {
-    if (cchunk == 0 && unit < units && k > 0) { // (unit >= units: a spare chunk behind the last step)
+  // (the store of a step's outputs can be put off: its arguments)
+  struct PairStore { Packed pk; int ob, xs, ylo, yhi, rw; bool valid; };
+  auto second_compute = [&](int rw, PairStore &ps) {
+    ps.valid = cchunk == 0 && unit < units && k > 0; // (unit >= units: a spare chunk behind the last step)
+    if (ps.valid) {
       init_acc(acc, sBias2, lane);
       int rslot = wslot - IH - 2;
       rslot = rslot < 0 ? rslot + NS : rslot;
       rslot = rslot < 0 ? rslot + NS : rslot;
       mma_mid(sMid, rslot, w2, acc, rw, lane);
-      Packed pk;
 #if TAPM
-      pack_tapm(acc, pk);
+      pack_tapm(acc, ps.pk);
 #else
-      pack_tile(acc, pk);
+      pack_tile(acc, ps.pk);
 #endif
-      store_pair(pk, out, g.ys + (k - 1) * IH - 2, g.xs, g.ys, g.ye, rw, lane, pc);
+      ps.ob = g.ys + (k - 1) * IH - 2; ps.xs = g.xs; ps.ylo = g.ys; ps.yhi = g.ye; ps.rw = rw;
     }
+  };
+  auto second_store = [&](const PairStore &ps) {
+    if (ps.valid)
+      store_pair(ps.pk, out, ps.ob, ps.xs, ps.ylo, ps.yhi, ps.rw, lane, pc);
+  };
+  auto second = [&](int rw) {
+    PairStore ps;
+    second_compute(rw, ps);
+    second_store(ps);
   };
   // what the computing side does in one chunk, after the barrier that published the chunk's halo
   auto compute = [&]() {
@@ -547,7 +599,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
         mma_first<TAIL, CPADP>(sIn[buf], sW1, cchunk * CK, acc, wv, lane);
 #endif
     }
-    buf ^= 1;
+    buf = buf == NBUF - 1 ? 0 : buf + 1;
     if (real && cchunk == NCHUNK - 1)
       store_mid(acc, sMid, wslot, g.ys - 1 + k * IH, g.xs - 1, Hc, Wc, wv, lane);
     advance();
@@ -578,6 +630,47 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   for (int u = unit; u < units; u += GRID)
     chunks += (geometry(u).steps + 1) * NCHUNK;
   if (wv >= WAVES) {
+#if DLDS
+    // ---- staging waves, halos straight into LDS: chunk c + 1's loads are issued right after the barrier that starts chunk c
+    // (all waves have left sIn[(c + 1) & 1] by then) and have to land before the barrier that starts chunk c + 1.  With
+    // C2STAGE the second convolution's outputs are stored one chunk late, in front of the next loads: the wait for those
+    // loads then never waits for stores that have only just been issued. ----
+    dma(sIn[0]); // chunk 0
+#if NBUF == 3
+    dma(sIn[1]); // chunk 1
+#endif
+    H::dma_wait();
+#if C2STAGE
+    PairStore pend;
+    pend.valid = false;
+#endif
+    int nb = NBUF - 1; // buffer of the chunk whose loads are issued next
+    for (int c = 0; c < chunks; ++c) {
+      DNX_SYNC(); // chunk c starts: its halo is complete, the buffer chunk c - 1 used is free
+#if C2STAGE
+      second_store(pend);
+#endif
+      // (past the last chunk the loads are issued all the same, aimed outside the image: the wait below counts them)
+      dma(sIn[nb]);
+      nb = nb == NBUF - 1 ? 0 : nb + 1;
+#if C2STAGE
+      __builtin_amdgcn_s_setprio(1);
+      second_compute(wv - WAVES, pend);
+      __builtin_amdgcn_s_setprio(0);
+      advance();
+#endif
+#if NBUF == 3
+      // The next chunk's halo was requested one chunk ago: everything but the loads just issued has to have landed.  Loads and
+      // stores complete in the order they were issued, and this interval's stores precede its loads.
+      H::dma_wait_all_but_last();
+#else
+      H::dma_wait();
+#endif
+    }
+#if C2STAGE
+    second_store(pend);
+#endif
+#else
     // ---- staging waves: chunk c's halo is written to sIn[c & 1] during chunk c - 1 ----
     H::Regs st0, st1;
     int commitChunk = 0; // channel chunk of the halo being written
@@ -619,6 +712,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
       }
       rest();
     }
+#endif
   } else {
     // ---- computing waves ----
     for (int c = 0; c < chunks; ++c) {

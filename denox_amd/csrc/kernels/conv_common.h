@@ -124,6 +124,25 @@ typedef unsigned short ushort_t;
 #endif
 #define NT ((WAVES + PW) * 64)
 #define KOUTP (((KOUT) + MF - 1) / MF * MF)
+// DLDS 1: halos go from memory straight into LDS (buffer_load_dwordx4 ... lds, new with gfx950) instead of through registers
+// of the staging waves.  The hardware writes the 64 lanes of such a load to 64 consecutive 16-byte slots, so the slot a
+// vector lands in is fixed by who loads it: staging thread t's it-th load fills slot t + it * (staging threads).  What each
+// lane is free to choose is WHICH vector it loads into its slot.  The staged halo stays pixel-major without padding (G = CK / 8
+// slots per pixel), and slot P * G + r of pixel P receives channel group (r - P / (8 / G)) mod G: a rotation that puts the same
+// channel group of 8 consecutive pixels into 8 different 16-byte bank groups, so the matrix loop's fragment reads stay free of
+// bank conflicts, while the G lanes of a pixel still read one contiguous piece of memory.  Needs staging waves, whole
+// 8-channel groups and every LDS step inside one source.
+#ifndef DLDS
+#define DLDS 0
+#endif
+#define DG (CK / 8)                                                        // 16-byte slots per staged pixel
+#define DD (8 / DG)                                                        // pixels that share a 128-byte row of LDS
+#if DLDS
+#define HALO_SLOTS (((HALO_PIX * DG + PW * 64 - 1) / (PW * 64)) * (PW * 64)) // whole loads of all staging threads
+#define HALO_ELEMS (HALO_SLOTS * 8)
+#else
+#define HALO_ELEMS (HALO_PIX * CKP)
+#endif
 
 struct PushConstants {
   unsigned int IN_W;
@@ -154,6 +173,7 @@ __device__ DNX_INLINE int clampi(int v, int lo, int hi) { return v < lo ? lo : (
 // field for: immediate offsets.
 typedef __attribute__((address_space(3))) const _Float16 lds_half_t;
 typedef __attribute__((address_space(3))) const half8 lds_half8_t;
+typedef __attribute__((address_space(3))) void lds_void_t;
 __device__ DNX_INLINE lds_half_t *lds_opaque(const _Float16 *p) {
   unsigned a = (unsigned)(size_t)(lds_half_t *)p;
   __asm__ volatile("" : "+v"(a));
@@ -346,7 +366,7 @@ struct Halo {
 #pragma unroll
     for (int it = 0; it < NV; ++it) {
       const int i = t + it * NTH;
-#if LAYIN
+#if LAYIN && !DLDS
       // block-major sources: consecutive lanes take consecutive pixels of one 8-channel plane (16 consecutive bytes each)
       const int v = i / HALO_PIX;
       const int pix = i - v * HALO_PIX;
@@ -356,8 +376,14 @@ struct Halo {
 #endif
       m.hy[it] = pix / HALO_W;
       m.hx[it] = pix - m.hy[it] * HALO_W;
+#if DLDS
+      // slot i = pix * DG + v is where the hardware puts this lane's load; the channel group that belongs there
+      m.v8[it] = ((v - pix / DD) & (DG - 1)) * 8;
+      m.lds[it] = i < HALO_PIX * VPPK ? i * 8 : -1;
+#else
       m.v8[it] = v * 8;
       m.lds[it] = i < HALO_PIX * VPPK ? pix * CKP + v * 8 : -1;
+#endif
     }
   }
 
@@ -426,7 +452,7 @@ struct Halo {
 #pragma unroll
     for (int it = 0; it < NV; ++it) {
       const int i = t + it * NTH;
-#if LAYIN
+#if LAYIN && !DLDS
       const int pix = i % HALO_PIX;
 #else
       const int pix = i / VPPK;
@@ -529,6 +555,46 @@ struct Halo {
 #endif
   }
 
+#if DLDS
+  // The same loads with LDS as their destination: thread t's it-th vector lands in slot t + it * NTH of `dst` (64 consecutive
+  // slots per wave and load), zeros where fetch() would have produced zeros.  No wave may read `dst` before these loads have
+  // been waited for (dma_wait) and a barrier has passed.
+  template <int L>
+  static __device__ DNX_INLINE void dma(const Sources &src, _Float16 *dst, const Map &m, const Src &s, int c0, int wave) {
+    const bool fromA = CB == 0 || c0 < CA; // the same for all lanes
+    const int cs = fromA ? CA : CB;
+    const int cbase = fromA ? 0 : CA;
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<_Float16 *>(fromA ? src.A : src.B), 0, (int)(fromA ? src.bytesA : src.bytesB), 0x00020000);
+#pragma unroll
+    for (int it = 0; it < NV; ++it) {
+      const int rel = c0 + m.v8[it] - cbase;
+      const unsigned pixoff = (unsigned)(fromA ? s.pa[it] : s.pb[it]);
+#if LAYIN
+      unsigned off = pixoff + (unsigned)(rel >> 3) * (fromA ? src.planeA : src.planeB);
+      off = pixoff == NO_LOAD ? NO_LOAD : off;
+#else
+      unsigned off = pixoff + 2u * (unsigned)rel;
+#endif
+      off = (m.lds[it] >= 0 && m.v8[it] < L && rel < cs) ? off : NO_LOAD;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_t *)(dst + (wave * 64 + it * NTH) * 8), 16, off, 0, 0, LOAD_AUX);
+    }
+  }
+  static __device__ DNX_INLINE void dma_step(const Sources &src, _Float16 *dst, const Map &m, const Src &s, int chunk, int wave) {
+    if (TAIL == CK || chunk < NCHUNK - 1)
+      dma<CK>(src, dst, m, s, chunk * CK, wave);
+    else
+      dma<TAIL>(src, dst, m, s, chunk * CK, wave);
+  }
+  // every load of this wave has arrived (in front of the barrier that publishes the halo)
+  static __device__ DNX_INLINE void dma_wait() { __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+  // ... every load and store older than the NV loads of the last dma() call has (memory instructions complete in issue order)
+  static __device__ DNX_INLINE void dma_wait_all_but_last() {
+    static_assert(NV <= 63, "the counter's field");
+    __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(NV) : "memory");
+  }
+#endif
+
   // ... and write them to the staged halo.
   template <int L>
   static __device__ DNX_INLINE void commit(const Regs &st, _Float16 *sIn, const Map &m, int c0) {
@@ -563,6 +629,31 @@ struct Halo {
       commit<TAIL>(st, sIn, m, chunk * CK);
   }
 };
+
+#if DLDS
+static_assert(SRC_UNIFORM && CA % 8 == 0 && CB % 8 == 0 && PW > 0 && MF == 32 && SX == 1 && SY == 1 && CK >= 16 && CK <= 64 && (DG & (DG - 1)) == 0,
+              "halos straight into LDS: see DLDS above");
+// Reading side of DLDS.  A pixel fragment of the matrix loop is channel group 2 ks + kh (kh: the lane's k half) of pixel
+// u + c, where u = (first halo row of the wave) * HALO_W + (lane & 31) belongs to the lane and c = hr * HALO_W + s is a
+// compile-time constant.  Its slot is (u + c) * DG + ((2 ks + kh + (u + c) / DD) mod DG); the rotation splits into a part of
+// the lane, which depends on c only through a = c % DD (a carry) and k = (2 ks + c / DD) mod DG, and the constant c * DG.
+// So a lane keeps DD * DG = 8 base addresses and every read is `base[a][k] + immediate`.
+struct PxBase {
+  lds_half_t *b[DD][DG];
+};
+__device__ DNX_INLINE void px_base_init(PxBase &pb, const _Float16 *sIn, int row0, int lane) {
+  const int u = row0 * HALO_W + (lane & 31), kh = lane >> 5;
+#pragma unroll
+  for (int a = 0; a < DD; ++a)
+#pragma unroll
+    for (int k = 0; k < DG; ++k) {
+      const int rot = (kh + u / DD + ((u % DD + a) >= DD ? 1 : 0) + k) & (DG - 1);
+      pb.b[a][k] = lds_opaque(sIn + (u * DG + rot) * 8);
+    }
+}
+#define PX_READ(pb, hr, s, ks) \
+  (*reinterpret_cast<lds_half8_t *>((pb).b[((hr) * HALO_W + (s)) % DD][(2 * (ks) + ((hr) * HALO_W + (s)) / DD) & (DG - 1)] + ((hr) * HALO_W + (s)) * DG * 8))
+#endif
 
 __device__ DNX_INLINE float apply_act(float v) {
 #if ACT == 1
@@ -786,7 +877,12 @@ __device__ DNX_INLINE void
 mma_chunk(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, int wv, int lane) {
   const int l32 = lane & 31;
   const int kq = (lane >> 5) * 8;
+#if DLDS
+  PxBase pxb;
+  px_base_init(pxb, sIn, wv * RPW, lane);
+#else
   lds_half_t *pxb = lds_opaque(sIn + (wv * RPW * SY * HALO_W + l32 * SX) * CKP + kq);
+#endif
   lds_half_t *wb = lds_opaque(sW + l32 * WPITCH + wofs + kq);
 #pragma unroll
   for (int s = 0; s < KS; ++s) {
@@ -796,7 +892,11 @@ mma_chunk(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, int wv, i
 #pragma unroll
       for (int hr = 0; hr < PXROWS; ++hr)
         if (SY == 1 || hr % SY < KR) // with a stride larger than the filter some halo rows are never read
+#if DLDS
+          px[hr] = PX_READ(pxb, hr, s, ks);
+#else
           px[hr] = *reinterpret_cast<lds_half8_t *>(pxb + (hr * HALO_W + s) * CKP + ks * 16);
+#endif
 #pragma unroll
       for (int r = 0; r < KR; ++r) {
         half8 wf[KB];

@@ -178,7 +178,7 @@ def test_full_size_oidn_unet_blocked(oracle):
     check_crops(oracle, m, x, got, H, W, [(0, 0), (400, 800), (H - 272 + 8, W - 272)], "blocked 1080p")
 
 
-@pytest.mark.parametrize("config", ["x8r2k16", "x4r2k32", "x4r4k16", "x4r2k16", "y4r2k32", "z4r2k64", "v4r2k64", "v4r2k16", "u4r2k32"])
+@pytest.mark.parametrize("config", ["x8r2k16", "x4r2k32", "x4r4k16", "x4r2k16", "y4r2k32", "z4r2k64", "v4r2k64", "v4r2k16", "u4r2k32", "d4r2k64", "t4r2k32"])
 @pytest.mark.parametrize("C,K1,K2,tail", [(64, 32, 32, "pool"), (40, 32, 16, "relu"), (48, 16, 24, "none")])
 def test_conv_pair_reads_and_writes_either_layout(oracle, config, C, K1, K2, tail):
     """conv -> conv in one dispatch between two block-major tensors."""

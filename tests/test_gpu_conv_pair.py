@@ -12,7 +12,7 @@ from util import assert_bits_equal, assert_conv_close, fill_lds_with_nans, he_we
 
 pytestmark = pytest.mark.gpu
 
-PAIR_CONFIGS = ["x8r2k16", "x4r4k16", "x4r2k16", "x4r2k32", "y4r2k32", "z4r2k64", "v4r2k64", "v4r2k16", "u4r2k32"]
+PAIR_CONFIGS = ["x8r2k16", "x4r4k16", "x4r2k16", "x4r2k32", "y4r2k32", "z4r2k64", "v4r2k64", "v4r2k16", "u4r2k32", "d4r2k64", "t4r2k32"]
 
 
 def build(rng, C, K1, K2, tail, pad=False, act1=True, bias=True):
@@ -104,7 +104,8 @@ def integer_pair(x, K1, K2):
     return np.repeat(out[:, :, None], K2, axis=2)
 
 
-@pytest.mark.parametrize("config,C,density", [("x8r2k16", 8, 0.15), ("y4r2k32", 32, 0.04), ("z4r2k64", 64, 0.02), ("v4r2k64", 64, 0.02), ("v4r2k16", 8, 0.15), ("u4r2k32", 32, 0.04)])
+@pytest.mark.parametrize("config,C,density", [("x8r2k16", 8, 0.15), ("y4r2k32", 32, 0.04), ("z4r2k64", 64, 0.02), ("v4r2k64", 64, 0.02), ("v4r2k16", 8, 0.15), ("u4r2k32", 32, 0.04),
+                                              ("d4r2k64", 64, 0.02), ("t4r2k32", 32, 0.04)])
 @pytest.mark.parametrize("H,W", [(33, 47), (288, 31), (1080, 1920), (24, 9000)])  # the last: more strips than workgroups
 def test_pair_exact_on_small_integers(H, W, config, C, density):
     """Inputs in {0, 1}, all weights one: every intermediate and final value is an integer below 2048, which binary16
