@@ -51,7 +51,9 @@ std::string fmtFloat(float v) {
 // ostage: the finished tile goes to memory through LDS, stored by the staging waves (OSTAGE in conv3x3_mfma_ws.hip).
 // ksplit: computing waves share a tile's rows AND its output channels (KSP in conv3x3_upfold_ws.hip): wave w takes block
 // w % ksplit of the 32-channel blocks and row group w / ksplit.
-struct ConvConfig { unsigned waves, rpw, ck; bool resident; unsigned pw; unsigned maxKT; unsigned mf, xb; const char *name; bool pp = false; bool fold = false; bool wideHalo = false; bool ntStore = false; bool ostage = false; unsigned ksplit = 1; };
+// hrot: the staged halo unpadded, its 16-byte slots rotated per pixel instead (HROT in conv_common.h: 32-channel steps fit where the
+// padded form allowed 16).  swp: the matrix loop reads the next group's fragments while it issues the current group's (SWP).
+struct ConvConfig { unsigned waves, rpw, ck; bool resident; unsigned pw; unsigned maxKT; unsigned mf, xb; const char *name; bool pp = false; bool fold = false; bool wideHalo = false; bool ntStore = false; bool ostage = false; unsigned ksplit = 1; bool hrot = false; bool swp = false; };
 const ConvConfig kConvConfigs[] = {
     // weights streamed per step
     {4, 2, 16, false, 0, 0, 32, 1, "w4r2k16"}, {4, 2, 32, false, 0, 0, 32, 1, "w4r2k32"}, {4, 4, 16, false, 0, 0, 32, 1, "w4r4k16"}, {4, 4, 32, false, 0, 0, 32, 1, "w4r4k32"},
@@ -74,6 +76,13 @@ const ConvConfig kConvConfigs[] = {
     {4, 2, 16, true, 4, 0, 32, 1, "r4r2k16", false, false, false, false, true}, {4, 2, 16, true, 4, 0, 32, 1, "r4r2k16n", false, false, false, true, true},
     {8, 1, 16, true, 4, 0, 32, 1, "r8r1k16n", false, false, false, true, true}, {4, 2, 32, true, 4, 0, 32, 1, "r4r2k32n", false, false, false, true, true},
     {4, 1, 16, true, 4, 0, 32, 1, "r4r1k16n", false, false, false, true, true},
+    // ... with the rotated halo layout and the pipelined matrix loop
+    {4, 2, 32, true, 4, 0, 32, 1, "c4r2k32n", false, false, false, true, true, 1, true, true}, {4, 2, 16, true, 4, 0, 32, 1, "c4r2k16n", false, false, false, true, true, 1, true, true},
+    {4, 2, 16, true, 4, 0, 32, 1, "c4r2k16m", false, false, false, true, true, 1, false, true},
+    // the pipelined matrix loop (and, with 32-channel steps, the rotated layout) in the other kernel families
+    {4, 2, 16, false, 0, 0, 32, 1, "w4r2k16s", false, false, false, false, false, 1, false, true}, {4, 2, 32, false, 0, 0, 32, 1, "w4r2k32s", false, false, false, false, false, 1, true, true},
+    {8, 2, 16, true, 4, 0, 32, 1, "s8r2k16s", false, false, false, false, false, 1, false, true}, {8, 2, 32, true, 4, 0, 32, 1, "s8r2k32s", false, false, false, false, false, 1, true, true},
+    {8, 2, 32, true, 0, 0, 32, 1, "p8r2k32s", false, false, false, false, false, 1, true, true},
     // 16x16x32 matrix shape: output channels in blocks of 16, tiles of 16 or 32 pixels width
     {4, 2, 32, false, 0, 0, 16, 2, "m4r2k32x2"}, {4, 2, 64, false, 0, 0, 16, 2, "m4r2k64x2"}, {4, 1, 32, false, 0, 0, 16, 2, "m4r1k32x2"}, {4, 2, 32, false, 0, 0, 16, 1, "m4r2k32x1"},
     {4, 4, 32, false, 0, 0, 16, 1, "m4r4k32x1"}, {8, 2, 32, false, 0, 0, 16, 2, "m8r2k32x2"}, {4, 2, 0, false, 0, 0, 16, 1, "m4r2kfx1"},  {4, 1, 0, false, 0, 0, 16, 2, "m4r1kfx2"},
@@ -104,7 +113,7 @@ constexpr unsigned kNumConvConfigs = sizeof(kConvConfigs) / sizeof(kConvConfigs[
 // Configurations that are also offered with channel-block-major (CHWC8) sources and / or result: one or two of each kernel
 // family and matrix shape, so that the layout alternative adds half as many candidates again instead of three times as many.
 bool offeredBlocked(const ConvConfig &cfg) {
-  for (const char *n : {"w4r2k16", "w8r2k32", "w4r1kfn", "p16r2k16", "s8r2k16", "t8r2k32", "t16r1k32", "m4r2k32x1", "m8r2k32x2", "m4r2kfx1", "q8r2k32x2", "s12r1k16", "r4r2k16n"})
+  for (const char *n : {"w4r2k16", "w8r2k32", "w4r1kfn", "p16r2k16", "s8r2k16", "t8r2k32", "t16r1k32", "m4r2k32x1", "m8r2k32x2", "m4r2kfx1", "q8r2k32x2", "s12r1k16", "r4r2k16n", "c4r2k32n", "s8r2k32s"})
     if (std::strcmp(n, cfg.name) == 0) return true;
   return false;
 }
@@ -147,7 +156,9 @@ bool chooseKT(const ConvConfig &cfgIn, unsigned CA, unsigned CB, unsigned K, con
   const unsigned th = cfg.waves * cfg.rpw;
   const unsigned tw = cfg.mf == 32 ? 32 : 16 * cfg.xb;
   const unsigned haloPix = ((th - 1) * g.SY + g.R) * ((tw - 1) * g.SX + g.S), taps = g.R * g.S;
-  const unsigned ckp = cfg.ck + 8;
+  const unsigned ckp = cfg.hrot ? cfg.ck : cfg.ck + 8; // halves per staged halo pixel
+  if (cfg.hrot && (cfg.mf != 32 || g.SY != 1 || g.SX != 1 || (cfg.ck != 16 && cfg.ck != 32 && cfg.ck != 64))) return false;
+  if (cfg.swp && (cfg.mf != 32 || g.SY != 1)) return false;
   const unsigned blocks = g.KOUTP / blk;
   // registers per lane: 512 shared by the waves of one SIMD; a workgroup of `waves` waves puts waves/4 on each
   const unsigned wavesPerSimd = (cfg.waves + cfg.pw + 3) / 4;
@@ -158,7 +169,7 @@ bool chooseKT(const ConvConfig &cfgIn, unsigned CA, unsigned CB, unsigned K, con
     const unsigned accRegs = cfg.mf == 32 ? kb * cfg.rpw * 16 : kb * cfg.rpw * cfg.xb * 4;
     if (accRegs + 64 + (cfg.mf == 16 ? kb * 4 : 0) > regBudget) continue;
     const size_t lds = (cfg.resident ? static_cast<size_t>(taps * kb * blk) * (g.CPAD + 8) * 2u + 2u * static_cast<size_t>(haloPix) * ckp * 2u
-                                     : (static_cast<size_t>(haloPix) + taps * kb * blk) * ckp * 2u) +
+                                     : (static_cast<size_t>(haloPix) * ckp + static_cast<size_t>(taps * kb * blk) * (cfg.ck + 8)) * 2u) +
                        static_cast<size_t>(kb * blk) * 4u + // + the staged bias (fp32)
                        (cfg.ostage ? static_cast<size_t>(th * tw) * (kb * blk / 8 + 1) * 16u : 0u); // + the finished tile (one spare 16-byte slot per pixel)
     if (lds > dev.maxComputeSharedMemory) continue;
@@ -455,7 +466,7 @@ public:
       }
       if (cfg.wideHalo && conv.strideX == 1 && conv.strideY == 1) continue;
       if (cfg.ostage) { // whole 16-byte slots of a pixel-major result, at least two steps per tile
-        if ((m.pattern & (PAT_POOL | PAT_CROP)) || m.outputFormat || conv.K % 8 || cpad / stepChannels(cfg, cpad) < 2) continue;
+        if ((m.pattern & (PAT_POOL | PAT_CROP)) || m.outputFormat || conv.K % 8 || (cpad + stepChannels(cfg, cpad) - 1) / stepChannels(cfg, cpad) < 2) continue; // (a shorter last step counts)
         if (m.outputVariant) {
           const ConcatView v = concatViewOf(model, m.output);
           if (!v.valid || v.pitch % 8 || v.channelOffset % 8) continue;
@@ -518,6 +529,8 @@ public:
     if (cfg.ksplit > 1) k.define("KSP", cfg.ksplit);
     if (cfg.ntStore) k.define("STORE_AUX", 2);
     if (cfg.ostage) k.define("OSTAGE", 1);
+    if (cfg.hrot) k.define("HROT", 1);
+    if (cfg.swp) k.define("SWP", 1);
     k.define("CA", CA); k.define("CB", CB); k.define("UPA", up ? 1 : 0);
     k.define("KOUT", conv.K); k.define("KT", g.KT);
     k.define("ACT", act);

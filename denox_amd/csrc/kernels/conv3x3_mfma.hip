@@ -59,7 +59,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     const _Float16 *__restrict__ BIAS,
 #endif
     PushConstants pc) {
-  __shared__ __attribute__((aligned(16))) _Float16 sIn[HALO_PIX * CKP];
+  __shared__ __attribute__((aligned(16))) _Float16 sIn[HALO_ELEMS];
   __shared__ __attribute__((aligned(16))) _Float16 sW[NTAPS * KT * CKP];
   __shared__ __attribute__((aligned(16))) bias_t sBias[KT];
 #if CB == 0

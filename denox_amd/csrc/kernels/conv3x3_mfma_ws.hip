@@ -55,7 +55,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
 #endif
     PushConstants pc) {
   __shared__ __attribute__((aligned(16))) _Float16 sW[NTAPS * KT * CPADP];
-  __shared__ __attribute__((aligned(16))) _Float16 sIn[2][HALO_PIX * CKP];
+  __shared__ __attribute__((aligned(16))) _Float16 sIn[2][HALO_ELEMS];
   __shared__ __attribute__((aligned(16))) bias_t sBias[KT];
 #if OSTAGE
   __shared__ uint4v sOut[TH * TW * OSLOTS];

@@ -76,6 +76,10 @@
 #define NBUF 2 // halo buffers.  3 (with DLDS): the loads of chunk c + 2 are issued while chunk c is multiplied, a whole chunk earlier
 #endif
 static_assert(NBUF == 2 || (NBUF == 3 && DLDS), "a third halo buffer serves loads that go straight into LDS");
+// Where the registers allow it, a convolution's accumulators start from its bias held in registers (see load_bias_regs);
+// where the first convolution's weights fill the register file they start from the bias staged in LDS.
+#define BIAS1REG (!W1REG)
+#define BIAS2REG (!(W1REG && (!C2STAGE || DLDS)))
 static_assert(!C2STAGE || PW == WAVES, "second convolution on the staging waves: one staging wave per computing wave");
 static_assert(!TAPM || (3 * KOUT <= 15 && !POOL), "filter columns in the matrix rows: at most 5 output channels, no pooling");
 
@@ -113,6 +117,7 @@ __device__ DNX_INLINE half8 finish8_first(const float *v) {
 #endif
 }
 
+// (W1REG: no registers left for the first convolution's bias; its accumulators start from the bias staged in LDS)
 __device__ DNX_INLINE void init_acc_first(Acc &acc, const bias_t *sBias1, int lane) {
   const int hsel = lane >> 5;
 #pragma unroll
@@ -124,6 +129,16 @@ __device__ DNX_INLINE void init_acc_first(Acc &acc, const bias_t *sBias1, int la
 #else
       acc.v[0][j][i] = 0.0f;
 #endif
+}
+
+// The bias of a convolution as an accumulator-shaped register set: lane's 16 output channels (lane >> 5) * 16 + i.  The first
+// matrix instruction into each accumulator of a step takes it as its addend, so no pass over the accumulators starts a step
+// (vector ALU instructions are not free beside matrix instructions here: what a wave issues between them delays them).
+__device__ DNX_INLINE float16v load_bias_regs(const _Float16 *__restrict__ bias, bool has, int lane) {
+  float16v b;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) b[i] = has ? (float)bias[(lane >> 5) * 16 + i] : 0.0f;
+  return b;
 }
 
 // The wave's RPW finished rows of `mid` -> ring.  acc.v[0][j] holds, for row j of the wave and pixel lane & 31, the 16
@@ -189,7 +204,8 @@ __device__ DNX_INLINE void load_second_weights(SecondWeights &sw, const _Float16
 
 // Second convolution: 9 taps x (C2PAD / 16) reduction steps from the ring.  rslot0: ring row that holds `mid` row
 // (first output row of the step) - 1.
-__device__ DNX_INLINE void mma_mid(const _Float16 *sMid, int rslot0, const SecondWeights &sw, Acc &acc, int wv, int lane) {
+// BIAS2REG: the accumulators start from `bias`; else they hold their start values already
+__device__ DNX_INLINE void mma_mid(const _Float16 *sMid, int rslot0, const SecondWeights &sw, Acc &acc, const float16v &bias, int wv, int lane) {
   const int l32 = lane & 31;
   const int kq = (lane >> 5) * 8;
   lds_half_t *pr[PXROWS];
@@ -222,7 +238,7 @@ __device__ DNX_INLINE void mma_mid(const _Float16 *sMid, int rslot0, const Secon
     for (int r = 0; r < 3; ++r)
 #pragma unroll
       for (int j = 0; j < RPW; ++j)
-        acc.v[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sw.w[TAPM ? r : r * 3 + s][ks], px[g & 1][j + r], acc.v[0][j], 0, 0, 0);
+        acc.v[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sw.w[TAPM ? r : r * 3 + s][ks], px[g & 1][j + r], (BIAS2REG && g == 0 && r == 0) ? bias : acc.v[0][j], 0, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
   }
 }
@@ -253,11 +269,12 @@ __device__ DNX_INLINE void pack_tapm(const Acc &acc, Packed &pk) {
 
 // First convolution, one chunk of L channels: as mma_chunk of conv_common.h (32 weight rows, pitch WPITCH; halo pitch CKP),
 // pipelined as described above.
-template <int L, int WPITCH>
-__device__ DNX_INLINE void mma_first(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, int wv, int lane) {
+// FIRST: the accumulators start from `bias` (their contents are not read).
+template <int L, int WPITCH, bool FIRST>
+__device__ DNX_INLINE void mma_first(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, const float16v &bias, int wv, int lane) {
   const int l32 = lane & 31;
   const int kq = (lane >> 5) * 8;
-#if DLDS
+#if HROTL
   PxBase pxb;
   px_base_init(pxb, sIn, wv * RPW, lane);
 #else
@@ -270,7 +287,7 @@ __device__ DNX_INLINE void mma_first(const _Float16 *sIn, const _Float16 *sW, in
     const int s = g / (L / 16), ks = g % (L / 16);
 #pragma unroll
     for (int hr = 0; hr < PXROWS; ++hr)
-#if DLDS
+#if HROTL
       px[g & 1][hr] = PX_READ(pxb, hr, s, ks);
 #else
       px[g & 1][hr] = *reinterpret_cast<lds_half8_t *>(pxb + (hr * HALO_W + s) * CKP + ks * 16);
@@ -289,7 +306,7 @@ __device__ DNX_INLINE void mma_first(const _Float16 *sIn, const _Float16 *sW, in
     for (int r = 0; r < 3; ++r)
 #pragma unroll
       for (int j = 0; j < RPW; ++j)
-        acc.v[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[g & 1][r], px[g & 1][j + r], acc.v[0][j], 0, 0, 0);
+        acc.v[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[g & 1][r], px[g & 1][j + r], (FIRST && g == 0 && r == 0) ? bias : acc.v[0][j], 0, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
   }
 }
@@ -314,7 +331,7 @@ template <int L, int CHUNK>
 __device__ DNX_INLINE void mma_first_reg(const _Float16 *sIn, const FirstWeights &fw, Acc &acc, int wv, int lane) {
   const int l32 = lane & 31;
   const int kq = (lane >> 5) * 8;
-#if DLDS
+#if HROTL
   PxBase pxb;
   px_base_init(pxb, sIn, wv * RPW, lane);
 #else
@@ -326,7 +343,7 @@ __device__ DNX_INLINE void mma_first_reg(const _Float16 *sIn, const FirstWeights
     const int s = g / (L / 16), ks = g % (L / 16);
 #pragma unroll
     for (int hr = 0; hr < PXROWS; ++hr)
-#if DLDS
+#if HROTL
       px[g & 1][hr] = PX_READ(pxb, hr, s, ks);
 #else
       px[g & 1][hr] = *reinterpret_cast<lds_half8_t *>(pxb + (hr * HALO_W + s) * CKP + ks * 16);
@@ -406,11 +423,14 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     PushConstants pc) {
 #if !W1REG
   __shared__ __attribute__((aligned(16))) _Float16 sW1[NTAPS * 32 * CPADP];
+#else
+  __shared__ __attribute__((aligned(16))) bias_t sBias1[32];
+#endif
+#if !BIAS2REG
+  __shared__ __attribute__((aligned(16))) bias_t sBias2[32];
 #endif
   __shared__ __attribute__((aligned(16))) _Float16 sIn[NBUF][HALO_ELEMS];
   __shared__ __attribute__((aligned(16))) _Float16 sMid[(NS * IW + 2) * C2P];
-  __shared__ __attribute__((aligned(16))) bias_t sBias1[32];
-  __shared__ __attribute__((aligned(16))) bias_t sBias2[32];
 #if CB == 0
   const _Float16 *B = nullptr;
 #endif
@@ -445,13 +465,13 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   };
 
   // ---- resident weights and biases ----
-#if HAS_BIAS1
-  for (int i = tid; i < 32; i += NT) sBias1[i] = (float)BIAS1[i];
-#endif
-#if HAS_BIAS
+#if !BIAS2REG && HAS_BIAS
   for (int i = tid; i < 32; i += NT) sBias2[i] = (float)BIAS2[i];
 #endif
 #if W1REG
+#if HAS_BIAS1
+  for (int i = tid; i < 32; i += NT) sBias1[i] = (float)BIAS1[i];
+#endif
   static_assert(PW > 0, "weights in registers: computing waves that hold nothing else");
   FirstWeights w1;
   if (wv < WAVES)
@@ -468,6 +488,18 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   SecondWeights w2;
   if (!C2STAGE || wv >= WAVES) // (with C2STAGE the computing waves never touch them: dead there, no registers)
     load_second_weights(w2, FILT2, lane);
+#if !W1REG
+#if HAS_BIAS1
+  const float16v bias1 = load_bias_regs(BIAS1, true, lane);
+#else
+  const float16v bias1 = load_bias_regs(nullptr, false, lane);
+#endif
+#endif
+#if BIAS2REG && HAS_BIAS
+  const float16v bias2 = load_bias_regs(BIAS2, true, lane);
+#else
+  const float16v bias2 = load_bias_regs(nullptr, false, lane); // (zeros, or unused)
+#endif
 
   // ---- the fetch cursor walks the same sequence of (unit, step, channel chunk) as the compute cursor, two chunks ahead.
   // Every unit has one step more than it has rows for: the last one only drains the second convolution, its loads are
@@ -541,11 +573,13 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   auto second_compute = [&](int rw, PairStore &ps) {
     ps.valid = cchunk == 0 && unit < units && k > 0; // (unit >= units: a spare chunk behind the last step)
     if (ps.valid) {
+#if !BIAS2REG
       init_acc(acc, sBias2, lane);
+#endif
       int rslot = wslot - IH - 2;
       rslot = rslot < 0 ? rslot + NS : rslot;
       rslot = rslot < 0 ? rslot + NS : rslot;
-      mma_mid(sMid, rslot, w2, acc, rw, lane);
+      mma_mid(sMid, rslot, w2, acc, bias2, rw, lane);
 #if TAPM
       pack_tapm(acc, ps.pk);
 #else
@@ -568,8 +602,10 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
 #if !C2STAGE
     second(wv);
 #endif
+#if W1REG
     if (cchunk == 0)
       init_acc_first(acc, sBias1, lane);
+#endif
   };
   // moves the cursor (unit, k, cchunk, wslot) one chunk on
   auto advance = [&]() {
@@ -593,10 +629,12 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
 #if W1REG
       mma_first_reg_chunk<0>(cchunk, sIn[buf], w1, acc, wv, lane);
 #else
-      if (TAIL == CK || cchunk < NCHUNK - 1)
-        mma_first<CK, CPADP>(sIn[buf], sW1, cchunk * CK, acc, wv, lane);
+      if (cchunk == 0)
+        mma_first<(NCHUNK > 1 ? CK : TAIL), CPADP, true>(sIn[buf], sW1, 0, acc, bias1, wv, lane);
+      else if (TAIL == CK || cchunk < NCHUNK - 1)
+        mma_first<CK, CPADP, false>(sIn[buf], sW1, cchunk * CK, acc, bias1, wv, lane);
       else
-        mma_first<TAIL, CPADP>(sIn[buf], sW1, cchunk * CK, acc, wv, lane);
+        mma_first<TAIL, CPADP, false>(sIn[buf], sW1, cchunk * CK, acc, bias1, wv, lane);
 #endif
     }
     buf = buf == NBUF - 1 ? 0 : buf + 1;

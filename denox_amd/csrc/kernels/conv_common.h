@@ -135,13 +135,27 @@ typedef unsigned short ushort_t;
 #ifndef DLDS
 #define DLDS 0
 #endif
+// HROT 1: the same rotated, unpadded halo layout with the halo still staged through registers (the staging threads write each
+// vector to its rotated slot themselves).  A pixel then takes CK / 8 slots instead of CK / 8 + 1: halos of 32 channels fit
+// where the padded form allowed 16, which halves the barriers per tile.
+#ifndef HROT
+#define HROT 0
+#endif
+#define HROTL (DLDS || HROT)                                               // the rotated layout is in use
 #define DG (CK / 8)                                                        // 16-byte slots per staged pixel
 #define DD (8 / DG)                                                        // pixels that share a 128-byte row of LDS
 #if DLDS
 #define HALO_SLOTS (((HALO_PIX * DG + PW * 64 - 1) / (PW * 64)) * (PW * 64)) // whole loads of all staging threads
 #define HALO_ELEMS (HALO_SLOTS * 8)
+#elif HROT
+#define HALO_ELEMS (HALO_PIX * DG * 8)
 #else
 #define HALO_ELEMS (HALO_PIX * CKP)
+#endif
+// SWP 1: the matrix loop reads the fragments of the next group of matrix instructions while it issues the current group's,
+// one LDS read behind each instruction, in an order that scheduling barriers pin (32 x 32 x 16 shape).
+#ifndef SWP
+#define SWP 0
 #endif
 
 struct PushConstants {
@@ -380,6 +394,9 @@ struct Halo {
       // slot i = pix * DG + v is where the hardware puts this lane's load; the channel group that belongs there
       m.v8[it] = ((v - pix / DD) & (DG - 1)) * 8;
       m.lds[it] = i < HALO_PIX * VPPK ? i * 8 : -1;
+#elif HROT
+      m.v8[it] = v * 8;
+      m.lds[it] = i < HALO_PIX * VPPK ? (pix * DG + ((v + pix / DD) & (DG - 1))) * 8 : -1;
 #else
       m.v8[it] = v * 8;
       m.lds[it] = i < HALO_PIX * VPPK ? pix * CKP + v * 8 : -1;
@@ -631,9 +648,11 @@ struct Halo {
 };
 
 #if DLDS
-static_assert(SRC_UNIFORM && CA % 8 == 0 && CB % 8 == 0 && PW > 0 && MF == 32 && SX == 1 && SY == 1 && CK >= 16 && CK <= 64 && (DG & (DG - 1)) == 0,
-              "halos straight into LDS: see DLDS above");
-// Reading side of DLDS.  A pixel fragment of the matrix loop is channel group 2 ks + kh (kh: the lane's k half) of pixel
+static_assert(SRC_UNIFORM && CA % 8 == 0 && CB % 8 == 0 && PW > 0, "halos straight into LDS: see DLDS above");
+#endif
+#if HROTL
+static_assert(MF == 32 && SX == 1 && SY == 1 && CK >= 16 && CK <= 64 && (DG & (DG - 1)) == 0, "rotated halo layout: 16, 32 or 64 channels per step, stride 1");
+// Reading side of the rotated layout.  A pixel fragment of the matrix loop is channel group 2 ks + kh (kh: the lane's k half) of pixel
 // u + c, where u = (first halo row of the wave) * HALO_W + (lane & 31) belongs to the lane and c = hr * HALO_W + s is a
 // compile-time constant.  Its slot is (u + c) * DG + ((2 ks + kh + (u + c) / DD) mod DG); the rotation splits into a part of
 // the lane, which depends on c only through a = c % DD (a carry) and k = (2 ks + c / DD) mod DG, and the constant c * DG.
@@ -869,7 +888,7 @@ store_packed(const Packed &pk, OutBuf out, int y0, int x0, int kt, int wv, int l
   }
 }
 
-// 9 taps x (L/16) reduction steps from one staged halo (row pitch CKP halves) and
+// 9 taps x (L/16) reduction steps from one staged halo (row pitch CKP halves, or the rotated layout) and
 // a weight slice whose rows are WPITCH halves apart; `wofs` selects the channel
 // offset of this chunk inside a weight row.
 template <int L, int WPITCH>
@@ -877,13 +896,47 @@ __device__ DNX_INLINE void
 mma_chunk(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, int wv, int lane) {
   const int l32 = lane & 31;
   const int kq = (lane >> 5) * 8;
-#if DLDS
+#if HROTL
   PxBase pxb;
   px_base_init(pxb, sIn, wv * RPW, lane);
+  auto px_read = [&](int hr, int s, int ks) { return PX_READ(pxb, hr, s, ks); };
 #else
   lds_half_t *pxb = lds_opaque(sIn + (wv * RPW * SY * HALO_W + l32 * SX) * CKP + kq);
+  auto px_read = [&](int hr, int s, int ks) { return *reinterpret_cast<lds_half8_t *>(pxb + (hr * HALO_W + s) * CKP + ks * 16); };
 #endif
   lds_half_t *wb = lds_opaque(sW + l32 * WPITCH + wofs + kq);
+  auto w_read = [&](int r, int kb, int s, int ks) { return *reinterpret_cast<lds_half8_t *>(wb + ((r * KS + s) * KT + kb * 32) * WPITCH + ks * 16); };
+#if SWP
+  // A group is one filter column s of one 16-channel slice: PXROWS pixel fragments and KR * KB weight fragments feed
+  // KR * KB * RPW matrix instructions.  Left to the compiler, each read was issued right in front of the instruction that
+  // needs it, and every few instructions waited out an LDS round trip.
+  static_assert(SY == 1, "the pipelined matrix loop reads every halo row");
+  constexpr int NG = KS * (L / 16), NREAD = PXROWS + KR * KB, NMMA = KR * KB * RPW;
+  half8 px[2][PXROWS], wf[2][KR][KB];
+  auto read_one = [&](int g, int i) { // read i of group g
+    const int s = g / (L / 16), ks = g % (L / 16);
+    if (i < PXROWS)
+      px[g & 1][i] = px_read(i, s, ks);
+    else
+      wf[g & 1][(i - PXROWS) / KB][(i - PXROWS) % KB] = w_read((i - PXROWS) / KB, (i - PXROWS) % KB, s, ks);
+  };
+#pragma unroll
+  for (int i = 0; i < NREAD; ++i) read_one(0, i);
+#pragma unroll
+  for (int g = 0; g < NG; ++g) {
+#pragma unroll
+    for (int i = 0; i < (NMMA > NREAD ? NMMA : NREAD); ++i) {
+      if (g + 1 < NG && i < NREAD)
+        read_one(g + 1, i);
+      __builtin_amdgcn_sched_barrier(0);
+      if (i < NMMA) {
+        const int r = i / (KB * RPW), kb = (i / RPW) % KB, j = i % RPW;
+        acc.v[kb][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[g & 1][r][kb], px[g & 1][j + r], acc.v[kb][j], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+#else
 #pragma unroll
   for (int s = 0; s < KS; ++s) {
 #pragma unroll
@@ -892,17 +945,13 @@ mma_chunk(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, int wv, i
 #pragma unroll
       for (int hr = 0; hr < PXROWS; ++hr)
         if (SY == 1 || hr % SY < KR) // with a stride larger than the filter some halo rows are never read
-#if DLDS
-          px[hr] = PX_READ(pxb, hr, s, ks);
-#else
-          px[hr] = *reinterpret_cast<lds_half8_t *>(pxb + (hr * HALO_W + s) * CKP + ks * 16);
-#endif
+          px[hr] = px_read(hr, s, ks);
 #pragma unroll
       for (int r = 0; r < KR; ++r) {
         half8 wf[KB];
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
-          wf[kb] = *reinterpret_cast<lds_half8_t *>(wb + ((r * KS + s) * KT + kb * 32) * WPITCH + ks * 16);
+          wf[kb] = w_read(r, kb, s, ks);
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -911,6 +960,7 @@ mma_chunk(const _Float16 *sIn, const _Float16 *sW, int wofs, Acc &acc, int wv, i
       }
     }
   }
+#endif
 }
 
 // Start of a tile: every accumulator holds the bias of its output channel (zero without one).  Reads the staged bias,

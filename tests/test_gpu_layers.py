@@ -58,7 +58,12 @@ ALL_CONFIGS += M16_CONFIGS
 ALL_CONFIGS += ["t16r1k16", "t16r1k32", "t16r2k16", "t8r2k16", "t8r2k32", "t8r4k16", "t8r1k16", "u8r2k32x2", "u16r1k32x2"]
 # staging waves that also store the result (through LDS, whole pixels per store instruction)
 OSTAGE_CONFIGS = ["r4r2k16", "r4r2k16n", "r8r1k16n", "r4r2k32n", "r4r1k16n"]
+# ... with the matrix loop's fragment reads pipelined (`m`), and the staged halo unpadded with rotated slots (`c`: 32-channel steps)
+OSTAGE_CONFIGS += ["c4r2k32n", "c4r2k16n", "c4r2k16m"]
 ALL_CONFIGS += OSTAGE_CONFIGS
+# the pipelined matrix loop / the rotated halo layout in the streaming, the staging-wave and the plain persistent kernel
+PIPELINED_CONFIGS = ["w4r2k16s", "w4r2k32s", "s8r2k16s", "s8r2k32s", "p8r2k32s"]
+ALL_CONFIGS += PIPELINED_CONFIGS
 
 
 # (tests/test_host.py checks on the CPU that every configuration of the library's table is in one of the lists of this file and
@@ -197,12 +202,12 @@ def test_full_size_fold_equals_the_unfolded_kernel_bit_for_bit():
     xa = rng.integers(0, 3, (H // 2, W // 2, CA)).astype(np.float16)
     xb = rng.integers(0, 3, (H - 8, W, CB)).astype(np.float16)
     outs = {}
-    for config in ("s8r2k16", "g4r1", "g4r1k32", "g4r1n", "h4r2n", "h4r2k32n", "f8r1", "r4r2k16n"):
+    for config in ("s8r2k16", "g4r1", "g4r1k32", "g4r1n", "h4r2n", "h4r2k32n", "f8r1", "r4r2k16n", "c4r2k32n", "w4r2k32s"):
         mod = dx.Module.compile(m, conv_config=config, assume={"H": H, "W": W})
         assert config in dx.last_compile_report() and mod.runtime_model.dispatch_count == 1
         outs[config] = mod.instance(H=H, W=W).infer(xa, xb)[0]
     assert outs["s8r2k16"].max() > 100 and np.array_equal(outs["s8r2k16"], np.round(outs["s8r2k16"]))
-    for config in ("g4r1", "g4r1k32", "g4r1n", "h4r2n", "h4r2k32n", "f8r1", "r4r2k16n"):
+    for config in ("g4r1", "g4r1k32", "g4r1n", "h4r2n", "h4r2k32n", "f8r1", "r4r2k16n", "c4r2k32n", "w4r2k32s"):
         assert_bits_equal(outs[config], outs["s8r2k16"], config)
     # and the unfolded kernel against the definition, on the four corners and a centre patch (float64 on the host)
     up = np.repeat(np.repeat(xa.astype(np.float64), 2, 0), 2, 1)
@@ -369,7 +374,7 @@ IN_PLACE_CASES = [  # (C, K0, K1, tail): channel range aligned / not aligned to 
     (8, 16, 16, "pool"), (12, 40, 24, "relu"), (32, 48, 80, "conv")]
 
 
-@pytest.mark.parametrize("config", [None, "s8r2k16", "m4r2k32x2", "t16r1k16", "q8r2k32x2", "r4r2k16n"])
+@pytest.mark.parametrize("config", [None, "s8r2k16", "m4r2k32x2", "t16r1k16", "q8r2k32x2", "r4r2k16n", "c4r2k32n"])
 @pytest.mark.parametrize("C,K0,K1,tail", IN_PLACE_CASES + [(48, 40, 24, "relu"), (64, 64, 32, "none")])
 def test_concat_sources_written_in_place(oracle, config, C, K0, K1, tail):
     """concat(conv(x), conv(x)): each conv stores into its channel range of the concat's tensor (pixel pitch K0 + K1),
