@@ -103,6 +103,9 @@ const ConvConfig kConvConfigs[] = {
     // ... and two rows of half the output channels per wave instead of one row of all of them (fewer LDS reads per matrix instruction)
     {4, 2, 0, true, 4, 0, 32, 1, "h4r2", false, true, false, false, false, 2}, {4, 2, 0, true, 4, 0, 32, 1, "h4r2n", false, true, false, true, false, 2},
     {4, 2, 32, true, 4, 0, 32, 1, "h4r2k32n", false, true, false, true, false, 2},
+    // ... and the fragment reads of the matrix loops issued three weight sets ahead (SWP in conv3x3_upfold_ws.hip)
+    {4, 2, 0, true, 4, 0, 32, 1, "h4r2p", false, true, false, true, false, 2, false, true}, {4, 1, 0, true, 4, 0, 32, 1, "g4r1p", false, true, false, true, false, 1, false, true},
+    {4, 2, 32, true, 4, 0, 32, 1, "h4r2k32p", false, true, false, true, false, 2, false, true},
     // the smallest tiles, offered to strided layers only: a stride multiplies the halo of a tile, and a 7 x 7 filter with
     // stride 4 fits the LDS next to its weights with nothing larger
     {2, 1, 16, false, 0, 32, 32, 1, "w2r1k16n", false, false, true}, {2, 1, 32, false, 0, 16, 16, 1, "m2r1k32x1n", false, false, true},

@@ -322,6 +322,46 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
                 for (int i = 0; i < 16; ++i)
                   acc[b].v[kb][j][i] = HAS_BIAS ? sBias[(kb0 + kb) * 32 + (lane >> 5) * 16 + i] : 0.0f;
         }
+#if SWP
+        {
+          // Software pipeline.  A unit is one weight fragment set: a 16-channel slice ks, a column cc = b + tx of the halo window,
+          // one of the (b, tx) pairs with that sum and a row tap ty -- KBW weight reads that feed KBW * RPW matrix
+          // instructions; the first unit of a column also reads the column's RPW + 1 pixel fragments.  The reads of unit
+          // u + SWPD are issued in front of unit u's matrix instructions, into rings of SWPD + 1 weight sets and three pixel
+          // columns (a column has at least two units, so the units u .. u + 3 touch at most three).  Left to the compiler,
+          // every weight read stood right in front of the instruction that needs it, which then waited out the LDS round
+          // trip: 2048 cycles of matrix work per tile took 3250.
+          constexpr int SWPD = 3, NU = (CKA / 16) * 8;
+          half8 px[3][RPW + 1], wf[SWPD + 1][KBW];
+          auto reads = [&](int u) {
+            const int ks = u >> 3, combo = (u >> 1) & 3, ty = u & 1, b = combo >> 1, tx = combo & 1, cc = b + tx;
+            const int kk = ks * 16 + kq;
+            if ((u & 7) == 0 || (u & 7) == 2 || (u & 7) == 6) {
+#pragma unroll
+              for (int t = 0; t < RPW + 1; ++t)
+                px[(ks * 3 + cc) % 3][t] = *reinterpret_cast<const half8 *>(sA[c] + ((rg * RPW + t) * AW + l32 + cc) * APITCH + kk);
+            }
+#pragma unroll
+            for (int kb = 0; kb < KBW; ++kb)
+              wf[u % (SWPD + 1)][kb] = *reinterpret_cast<const half8 *>(sWA[b] + ((ty * 2 + tx) * KT + (kb0 + kb) * 32 + l32) * WAP + c * CKA + kk);
+          };
+#pragma unroll
+          for (int u = 0; u < SWPD; ++u) reads(u);
+#pragma unroll
+          for (int u = 0; u < NU; ++u) {
+            if (u + SWPD < NU)
+              reads(u + SWPD);
+            __builtin_amdgcn_sched_barrier(0);
+            const int ks = u >> 3, combo = (u >> 1) & 3, ty = u & 1, b = combo >> 1, tx = combo & 1, cc = b + tx;
+#pragma unroll
+            for (int kb = 0; kb < KBW; ++kb)
+#pragma unroll
+              for (int j = 0; j < RPW; ++j)
+                acc[b].v[kb][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[u % (SWPD + 1)][kb], px[(ks * 3 + cc) % 3][j + ty], acc[b].v[kb][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+#else
 #pragma unroll
         for (int ks = 0; ks < CKA / 16; ++ks) {
           const int kk = ks * 16 + kq;
@@ -348,10 +388,45 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
                     acc[b].v[kb][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[kb], px[j + ty][b + tx], acc[b].v[kb][j], 0, 0, 0);
               }
         }
+#endif
       }
       // ---- the 9 taps over the full-resolution source: class (ca, b), tap (r, s) reads halo row 2 (y - yl0) + r,
       // halo column 2 (x - xl0) + b + s, which the de-interleaved halo holds at [parity (b + s) & 1][(x - xl0) + (b + s) / 2]
       DNX_SYNC();
+#if SWP
+      {
+        // a unit is one row tap r of one 16-channel slice: RPW x 4 pixel fragments (the weights are in registers) for 6 KBW RPW
+        // matrix instructions; the next unit's fragments are read in front of this unit's instructions
+        constexpr int NUB = (CBP / 16) * 3;
+        half8 px[2][RPW][4];
+        auto reads = [&](int u) {
+          const int ks = u / 3, r = u % 3, kk = ks * 16 + kq;
+#pragma unroll
+          for (int j = 0; j < RPW; ++j)
+#pragma unroll
+            for (int cc = 0; cc < 4; ++cc)
+              px[u & 1][j][cc] = *reinterpret_cast<const half8 *>(sB + ((2 * (rg * RPW + j) + r) * BW + (cc & 1) * 33 + l32 + (cc >> 1)) * BPITCH + kk);
+        };
+        reads(0);
+#pragma unroll
+        for (int u = 0; u < NUB; ++u) {
+          if (u + 1 < NUB)
+            reads(u + 1);
+          __builtin_amdgcn_sched_barrier(0);
+          const int ks = u / 3, r = u % 3;
+#pragma unroll
+          for (int s2 = 0; s2 < 3; ++s2)
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+              for (int kb = 0; kb < KBW; ++kb)
+#pragma unroll
+                for (int j = 0; j < RPW; ++j)
+                  acc[b].v[kb][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wB[r * 3 + s2][ks][kb], px[u & 1][j][b + s2], acc[b].v[kb][j], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+#else
 #pragma unroll
       for (int ks = 0; ks < CBP / 16; ++ks) {
         const int kk = ks * 16 + kq;
@@ -374,6 +449,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
                   acc[b].v[kb][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wB[r * 3 + s2][ks][kb], px[j][b + s2], acc[b].v[kb][j], 0, 0, 0);
         }
       }
+#endif
       // the tile as binary16 into LDS: this lane's 16 channels kb * 32 + (lane >> 5) * 16 .. of the pixels 2 l32 + b
 #pragma unroll
       for (int b = 0; b < 2; ++b)

@@ -27,7 +27,7 @@ LAST_PAIR = "conv3x3+relu+conv3x3+slice"                   # dec_conv1b -> dec_c
 FIRST_PAIR = "pad+conv3x3+relu+conv3x3+relu+maxpool"       # enc_conv0 -> enc_conv1 -> pool in one dispatch
 # Schedules to run: {operation: configuration} pairs that the selection is steered to.  The candidates of the three
 # longest dispatches that the timing table has been seen to select, in the layouts it combines them in.
-STEER = ([{DOMINANT_OPERATION: c} for c in ("h4r2n", "h4r2k32n", "h4r2", "g4r1n", "g4r1k32n", "g4r1", "g4r1k32", "s8r2k16", "s12r1k16", "t8r2k16", "p8r2k16", "f8r1")] +
+STEER = ([{DOMINANT_OPERATION: c} for c in ("h4r2n", "h4r2p", "g4r1p", "h4r2k32n", "h4r2", "g4r1n", "g4r1k32n", "g4r1", "g4r1k32", "s8r2k16", "s12r1k16", "t8r2k16", "p8r2k16", "f8r1")] +
          [{DOMINANT_OPERATION: "h4r2n", LAST_PAIR: c, FIRST_PAIR: f} for c, f in (("v4r2k64", "x8r2k16/hwc>chwc8"), ("d4r2k64", "x8r2k16/hwc>chwc8"), ("z4r2k64", "x8r2k16/hwc>chwc8"), ("y4r2k32", "v4r2k16"), ("u4r2k32", "x8r2k16"), ("x8r2k16", "x8r2k16"))] +
          [{DOMINANT_OPERATION: d + "/hwc>chwc8", LAST_PAIR: c + "/chwc8>hwc"} for d, c in (("s8r2k16", "v4r2k64"), ("s12r1k16", "z4r2k64"), ("s8r2k16", "y4r2k32"), ("s12r1k16", "x8r2k16"))] +
          # the same layers as four dispatches (conv -> conv fusion off, pixel-major), for comparison with the pairs

@@ -69,7 +69,7 @@ ALL_CONFIGS += PIPELINED_CONFIGS
 # (tests/test_host.py checks on the CPU that every configuration of the library's table is in one of the lists of this file and
 # compiles for at least one of the layer shapes it is tested on here: a configuration must not be covered by skips alone)
 EVERY_CONFIG_SHAPES = [(80, 64, 45, 70), (73, 96, 130, 300), (16, 32, 300, 530)]
-FOLD_CONFIGS = ["f8r1", "f4r2", "f4r1", "g4r1", "g4r1k32", "g4r1n", "g4r1k32n", "h4r2", "h4r2n", "h4r2k32n"]
+FOLD_CONFIGS = ["f8r1", "f4r2", "f4r1", "g4r1", "g4r1k32", "g4r1n", "g4r1k32n", "h4r2", "h4r2n", "h4r2k32n", "h4r2p", "g4r1p", "h4r2k32p"]
 FOLD_SHAPES = [(64, 9, 64, 36, 70, False), (16, 0, 32, 18, 34, False), (32, 24, 40, 62, 130, False), (8, 3, 3, 2, 2, False), (24, 9, 16, 40, 52, True),
                (96, 32, 64, 34, 66, False), (32, 16, 32, 50, 70, True), (48, 12, 96, 22, 134, False), (64, 8, 64, 2, 2, False), (16, 9, 32, 8, 64, False), (128, 9, 128, 20, 70, True)]
 STRIDED_ONLY_CONFIGS = ["m2r1k32x1n", "w2r2k16n", "w2r1k16n"]  # offered to strided layers only
@@ -202,12 +202,12 @@ def test_full_size_fold_equals_the_unfolded_kernel_bit_for_bit():
     xa = rng.integers(0, 3, (H // 2, W // 2, CA)).astype(np.float16)
     xb = rng.integers(0, 3, (H - 8, W, CB)).astype(np.float16)
     outs = {}
-    for config in ("s8r2k16", "g4r1", "g4r1k32", "g4r1n", "h4r2n", "h4r2k32n", "f8r1", "r4r2k16n", "c4r2k32n", "w4r2k32s"):
+    for config in ("s8r2k16", "g4r1", "g4r1k32", "g4r1n", "h4r2n", "h4r2k32n", "h4r2p", "g4r1p", "h4r2k32p", "f8r1", "r4r2k16n", "c4r2k32n", "w4r2k32s"):
         mod = dx.Module.compile(m, conv_config=config, assume={"H": H, "W": W})
         assert config in dx.last_compile_report() and mod.runtime_model.dispatch_count == 1
         outs[config] = mod.instance(H=H, W=W).infer(xa, xb)[0]
     assert outs["s8r2k16"].max() > 100 and np.array_equal(outs["s8r2k16"], np.round(outs["s8r2k16"]))
-    for config in ("g4r1", "g4r1k32", "g4r1n", "h4r2n", "h4r2k32n", "f8r1", "r4r2k16n", "c4r2k32n", "w4r2k32s"):
+    for config in ("g4r1", "g4r1k32", "g4r1n", "h4r2n", "h4r2k32n", "h4r2p", "g4r1p", "h4r2k32p", "f8r1", "r4r2k16n", "c4r2k32n", "w4r2k32s"):
         assert_bits_equal(outs[config], outs["s8r2k16"], config)
     # and the unfolded kernel against the definition, on the four corners and a centre patch (float64 on the host)
     up = np.repeat(np.repeat(xa.astype(np.float64), 2, 0), 2, 1)
