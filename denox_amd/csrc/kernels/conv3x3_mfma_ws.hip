@@ -44,6 +44,41 @@ static_assert(PW > 0 && MF == 32 && NCHUNK >= 2 && !POOL && !CROP && !LAYOUT_OUT
 #define NVO ((TH * TW * SPP + NSTAGE - 1) / NSTAGE) // slots per staging thread
 #endif
 
+// The resident weights ([tap][KT][CPAD] in memory, one chunk = the whole reduction, to LDS rows of CPADP) and the bias, by all
+// threads of the workgroup: every thread issues all of its loads before it waits for the first, in batches of at most WBATCH
+// vectors -- one memory round trip, where a loop of load / store pairs (which the compiler unrolls six times) took one per six
+// vectors, in front of a kernel whose whole run may be ten such round trips long.
+#define WBATCH 24
+__device__ DNX_INLINE void stage_weights_and_bias(_Float16 *sW, bias_t *sBias, const _Float16 *__restrict__ wsrc, const _Float16 *__restrict__ BIAS, int kt, int tid) {
+  constexpr int VPR = CPAD / 8, N = NTAPS * KT * VPR, PER = (N + NT - 1) / NT;
+#if HAS_BIAS
+  static_assert(KT <= NT, "one bias value per thread");
+  const _Float16 bias = BIAS[kt * KT + (tid < KT ? tid : 0)];
+#endif
+#pragma unroll
+  for (int r0 = 0; r0 < PER; r0 += WBATCH) {
+    uint4v w[WBATCH];
+#pragma unroll
+    for (int k = 0; k < WBATCH; ++k)
+      if (r0 + k < PER) {
+        const int i = tid + (r0 + k) * NT;
+        w[k] = ld16(wsrc + (size_t)(i < N ? i : N - 1) * 8); // threads past the end re-read the last vector
+      }
+#pragma unroll
+    for (int k = 0; k < WBATCH; ++k)
+      if (r0 + k < PER) {
+        const int i = tid + (r0 + k) * NT;
+        const int row = i / VPR, v = i - row * VPR;
+        if (i < N)
+          *reinterpret_cast<uint4v *>(sW + row * CPADP + v * 8) = w[k];
+      }
+  }
+#if HAS_BIAS
+  if (tid < KT)
+    sBias[tid] = (float)bias;
+#endif
+}
+
 extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     const _Float16 *__restrict__ A,
 #if CB > 0
@@ -92,18 +127,6 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   auto tileY = [&](int t) { return ((rev ? numTiles - 1 - t : t) / tilesX) * TH; };
   auto tileX = [&](int t) { return ((rev ? numTiles - 1 - t : t) % tilesX) * TW; };
 
-  stage_bias(sBias, BIAS, kt, tid);
-  // ---- resident weights: global [tap][KT][CPAD] (one chunk = whole reduction) -> LDS rows of CPADP ----
-  {
-    const _Float16 *wsrc = FILT + (size_t)kt * NTAPS * KT * CPAD;
-    constexpr int VPR = CPAD / 8;
-    for (int i = tid; i < NTAPS * KT * VPR; i += NT) {
-      const int row = i / VPR;
-      const int v = i - row * VPR;
-      *reinterpret_cast<uint4v *>(sW + row * CPADP + v * 8) = ld16(wsrc + (size_t)i * 8);
-    }
-  }
-
   // The fetch cursor walks the same sequence of steps as the compute cursor (tile by tile,
   // NCHUNK steps per tile), two steps ahead.
   typedef Halo<NSTAGE> H;
@@ -122,9 +145,20 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     }
   };
 
+  // The first two halos are on their way before the weights are asked for: everything a workgroup needs for its first step
+  // then arrives in one round trip.
+  H::Regs st0, st1;
+  if (PW == 0 || wv >= WAVES) {
+    H::map_init(map, PW > 0 ? tid - WAVES * 64 : tid);
+    H::src_init(fsrc, map, tileY(ftile), tileX(ftile), pc);
+    issue(st0); // step 0
+    __builtin_amdgcn_sched_barrier(0); // keep the two sets in issue order: the waits count loads in flight
+    issue(st1); // step 1
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  stage_weights_and_bias(sW, sBias, FILT + (size_t)kt * NTAPS * KT * CPAD, BIAS, kt, tid);
+
 #if PW == 0
-  H::map_init(map, tid);
-  H::src_init(fsrc, map, tileY(ftile), tileX(ftile), pc);
   Acc acc;
   // The finished tile, converted.  Its stores go out in NPARTS portions during the steps of the next tile: a
   // burst of all stores of all waves at once would hold the waves up at the store queue while nothing multiplies.
@@ -170,10 +204,6 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
       commitChunk = 0;
     issue(regs);
   };
-  H::Regs st0, st1;
-  issue(st0);
-  __builtin_amdgcn_sched_barrier(0); // keep the two sets in issue order: the waits count loads in flight
-  issue(st1);
   stage(st0, 0); // halo 0, by all waves
   DNX_SYNC();
   init_acc(acc, sBias, lane); // the staged bias is visible from here on
@@ -213,10 +243,6 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
       tile += SLOTS;
     }
   };
-  H::Regs st0, st1;
-  issue(st0);
-  __builtin_amdgcn_sched_barrier(0); // keep the two sets in issue order: the waits below count loads in flight
-  issue(st1);
   // The loop always runs both steps, so that it has one entry and one back edge with the same loads in flight on
   // both: the compiler then waits for exactly the register set a step needs.  When the last tile ends after the
   // first step, the second one is a spare: it stages and multiplies stale data and stores nothing.
@@ -235,9 +261,6 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   const int steps = myTiles * NCHUNK;
   if (wv >= WAVES) {
     // ---- staging waves: step g's halo is written to sIn[g & 1] during step g - 1 ----
-    H::map_init(map, tid - WAVES * 64);
-    H::src_init(fsrc, map, tileY(ftile), tileX(ftile), pc);
-    H::Regs st0, st1;
     int cchunk = 0; // chunk index of the step being committed
     auto commit = [&](H::Regs &regs, int g) {
       H::commit_step(regs, sIn[g & 1], map, cchunk);
@@ -262,8 +285,6 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
       }
     };
 #endif
-    issue(st0);         // step 0
-    issue(st1);         // step 1
     commit(st0, 0);
     issue(st0);         // step 2
     for (int g = 0; g < steps; g += 2) {
