@@ -217,6 +217,30 @@ def test_threads_with_their_own_handles_run_at_once():
             assert_bits_equal(o, alone[i], f"thread {i}")
 
 
+def test_two_frames_in_flight_on_two_streams():
+    """Two instances of one compiled model, each in a context (a stream) of its own, launched alternately from device memory
+    without waiting in between: their dispatches overlap on the GPU, and each writes what a single instance writes."""
+    torch = pytest.importorskip("torch")
+    H, W = 270, 478
+    m, _ = networks.build("oidn_unet", seed=4)
+    blob = dx.compile_model(m)
+    frames = [networks.synthetic_input("oidn_unet", H, W, seed=s) for s in (1, 2)]
+    want = [dx.Module.load(blob).instance(H=H, W=W).infer(x)[0] for x in frames]
+    ctxs = [dx.Context(), dx.Context()]
+    mods = [dx.Module.load(blob, c) for c in ctxs]
+    insts = [mod.instance(H=H, W=W) for mod in mods]
+    d_in = [torch.from_numpy(x).cuda() for x in frames]
+    d_out = [torch.full((H, W, 3), float("nan"), dtype=torch.float16, device="cuda") for _ in frames]
+    torch.cuda.synchronize()
+    for _ in range(40):
+        for i, inst in enumerate(insts):
+            inst.infer_device([d_in[i].data_ptr()], [d_out[i].data_ptr()])
+    for inst in insts:
+        inst.synchronize()
+    for i in range(2):
+        assert_bits_equal(d_out[i].cpu().numpy(), want[i], f"stream {i}")
+
+
 # ----------------------------------------------------------------------------- full size
 FULL_H, FULL_W = 1080, 1920
 
