@@ -80,7 +80,6 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   const int kt = DNX_BID_Z; // output-channel tile
 
   Acc acc;
-  stage_bias(sBias, BIAS, kt, tid);
 
   // packed filter: [kt][chunk][tap][KT][len(chunk)]
   const _Float16 *wbase = FILT + (size_t)kt * NTAPS * KT * CPAD;
@@ -96,6 +95,15 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     weights_fetch<CK>(wbase, stW, tid);
   else
     weights_fetch<TAIL>(wbase, stW, tid);
+  // The bias travels with the first step's loads and goes to LDS behind that step's halo and weights (loaded and staged in front
+  // of them, it cost the kernel a memory round trip of its own).
+#if HAS_BIAS
+  constexpr int NBV = (KT + NT - 1) / NT;
+  _Float16 biasv[NBV];
+#pragma unroll
+  for (int k = 0; k < NBV; ++k)
+    biasv[k] = BIAS[kt * KT + (tid + k * NT < KT ? tid + k * NT : 0)];
+#endif
   for (int chunk = 0; chunk < NCHUNK; ++chunk) {
     const bool fullNow = (TAIL == CK) || (chunk < NCHUNK - 1);
     H::commit_step(stIn, sIn, map, chunk);
@@ -103,6 +111,14 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
       weights_commit<CK>(stW, sW, tid);
     else
       weights_commit<TAIL>(stW, sW, tid);
+#if HAS_BIAS
+    if (chunk == 0) {
+#pragma unroll
+      for (int k = 0; k < NBV; ++k)
+        if (tid + k * NT < KT)
+          sBias[tid + k * NT] = (float)biasv[k];
+    }
+#endif
     DNX_SYNC();
     if (chunk == 0)
       init_acc(acc, sBias, lane); // the staged bias is visible from here on

@@ -464,27 +464,47 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     return g;
   };
 
-  // ---- resident weights and biases ----
+  // ---- resident weights and biases.  What goes to LDS is loaded here and written there by publish_resident(), which every role
+  // calls once it has asked for its first halos (and before its first barrier): written at once, each of these small pieces cost
+  // the kernel a memory round trip of its own in front of everything else. ----
 #if !BIAS2REG && HAS_BIAS
-  for (int i = tid; i < 32; i += NT) sBias2[i] = (float)BIAS2[i];
+  const _Float16 stagedBias2 = BIAS2[tid & 31];
 #endif
 #if W1REG
 #if HAS_BIAS1
-  for (int i = tid; i < 32; i += NT) sBias1[i] = (float)BIAS1[i];
+  const _Float16 stagedBias1 = BIAS1[tid & 31];
 #endif
   static_assert(PW > 0, "weights in registers: computing waves that hold nothing else");
   FirstWeights w1;
   if (wv < WAVES)
     load_first_weights(w1, FILT1, lane);
 #else
-  {
-    constexpr int VPR = CPAD / 8; // global [tap][32 rows][CPAD] -> LDS rows of CPADP
-    for (int i = tid; i < NTAPS * 32 * VPR; i += NT) {
-      const int row = i / VPR, v = i - row * VPR;
-      *reinterpret_cast<uint4v *>(sW1 + row * CPADP + v * 8) = ld16(FILT1 + (size_t)i * 8);
-    }
+  constexpr int VPR1 = CPAD / 8, NW1 = NTAPS * 32 * VPR1, PER1 = (NW1 + NT - 1) / NT; // global [tap][32 rows][CPAD] -> LDS rows of CPADP
+  uint4v stagedW1[PER1];
+#pragma unroll
+  for (int k = 0; k < PER1; ++k) {
+    const int i = tid + k * NT;
+    stagedW1[k] = ld16(FILT1 + (size_t)(i < NW1 ? i : NW1 - 1) * 8);
   }
 #endif
+  auto publish_resident = [&]() {
+#if !BIAS2REG && HAS_BIAS
+    if (tid < 32) sBias2[tid] = (float)stagedBias2;
+#endif
+#if W1REG
+#if HAS_BIAS1
+    if (tid < 32) sBias1[tid] = (float)stagedBias1;
+#endif
+#else
+#pragma unroll
+    for (int k = 0; k < PER1; ++k) {
+      const int i = tid + k * NT;
+      const int row = i / VPR1, v = i - row * VPR1;
+      if (i < NW1)
+        *reinterpret_cast<uint4v *>(sW1 + row * CPADP + v * 8) = stagedW1[k];
+    }
+#endif
+  };
   SecondWeights w2;
   if (!C2STAGE || wv >= WAVES) // (with C2STAGE the computing waves never touch them: dead there, no registers)
     load_second_weights(w2, FILT2, lane);
@@ -656,6 +676,8 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   issue(st0);
   __builtin_amdgcn_sched_barrier(0); // keep the two sets in issue order: the waits count loads in flight
   issue(st1);
+  __builtin_amdgcn_sched_barrier(0);
+  publish_resident();
   // The loop always runs two chunks, so that it has one entry and one back edge with the same loads in flight on both.
   // When the last step ends after the first of them, the second is a spare: it multiplies nothing and stores nothing.
   do {
@@ -677,6 +699,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
 #if NBUF == 3
     dma(sIn[1]); // chunk 1
 #endif
+    publish_resident();
     H::dma_wait();
 #if C2STAGE
     PairStore pend;
@@ -720,6 +743,8 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     issue(st0);   // chunk 0
     __builtin_amdgcn_sched_barrier(0);
     issue(st1);   // chunk 1
+    __builtin_amdgcn_sched_barrier(0);
+    publish_resident();
     commit(st0, 0);
     issue(st0);   // chunk 2
     // with C2STAGE: the second convolution of the step the cursor (unit, k, ...) has just left, for the rows of
@@ -753,6 +778,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
 #endif
   } else {
     // ---- computing waves ----
+    publish_resident();
     for (int c = 0; c < chunks; ++c) {
       DNX_SYNC();
       compute();

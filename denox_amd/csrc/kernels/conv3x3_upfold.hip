@@ -97,7 +97,6 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   auto tileY = [&](int t) { return ((rev ? numTiles - 1 - t : t) / tilesX) * TLH; }; // low-resolution coordinates
   auto tileX = [&](int t) { return ((rev ? numTiles - 1 - t : t) % tilesX) * 32; };
 
-  stage_bias(sBias, BIAS, kt, tid);
   { // resident weights of this (class, kt)
     const _Float16 *w = FILT + (size_t)(cls * NKT + kt) * KT * (4 * CAP + 9 * CBP);
     for (int i = tid; i < 4 * KT * VA; i += NT) {
@@ -210,6 +209,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   __builtin_amdgcn_sched_barrier(0);
   issueB(tile);
 #endif
+  stage_bias(sBias, BIAS, kt, tid); // (behind the first halos' loads, so that it does not cost a memory round trip of its own)
   for (; tile < last; tile += SLOTS) {
     // ---- step A: the folded 2x2 taps over the low-resolution source
     commitA();

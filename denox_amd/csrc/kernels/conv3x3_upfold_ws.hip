@@ -114,18 +114,40 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
   auto tileY = [&](int t) { return ((rev ? numTiles - 1 - t : t) / tilesX) * TLH; }; // low-resolution coordinates
   auto tileX = [&](int t) { return ((rev ? numTiles - 1 - t : t) % tilesX) * 32; };
 
-  stage_bias(sBias, BIAS, kt, tid);
-  { // resident weights of the classes (ca, 0) and (ca, 1) of this kt, by all waves
-    constexpr int VWA = CAP / 8;
+  // Resident weights of the classes (ca, 0) and (ca, 1) of this kt and the bias, by all waves: every load of a thread is in flight before
+  // the first is waited for, and the staging waves have asked for the first tile's halos before that (see their branch) -- one memory
+  // round trip in front of the first step instead of one per portion the compiler happened to unroll.
+  auto stage_weights_and_bias = [&]() {
+    constexpr int VWA = CAP / 8, NW = 4 * KT * VWA, PER = (NW + NT - 1) / NT;
+    static_assert(2 * PER <= 32, "weight vectors per thread");
+    uint4v wreg[2][PER];
+#if HAS_BIAS
+    static_assert(KT <= NT, "one bias value per thread");
+    const _Float16 bias = BIAS[kt * KT + (tid < KT ? tid : 0)];
+#endif
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
       const _Float16 *w = FILT + (size_t)((ca * 2 + b) * NKT + kt) * KT * (4 * CAP + 9 * CBP);
-      for (int i = tid; i < 4 * KT * VWA; i += NT) {
-        const int row = i / VWA, v = i - row * VWA;
-        *reinterpret_cast<uint4v *>(sWA[b] + row * WAP + v * 8) = ld16(w + (size_t)i * 8);
+#pragma unroll
+      for (int k = 0; k < PER; ++k) {
+        const int i = tid + k * NT;
+        wreg[b][k] = ld16(w + (size_t)(i < NW ? i : NW - 1) * 8);
       }
     }
-  }
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int k = 0; k < PER; ++k) {
+        const int i = tid + k * NT;
+        const int row = i / VWA, v = i - row * VWA;
+        if (i < NW)
+          *reinterpret_cast<uint4v *>(sWA[b] + row * WAP + v * 8) = wreg[b][k];
+      }
+#if HAS_BIAS
+    if (tid < KT)
+      sBias[tid] = (float)bias;
+#endif
+  };
 
   if (wv >= WAVES) {
     // ---- staging waves ---------------------------------------------------------------------------------------
@@ -263,6 +285,8 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
       issue(k, 0);
       __builtin_amdgcn_sched_barrier(0); // keep the register sets in issue order: the waits count loads in flight
     }
+    stage_weights_and_bias();
+    __builtin_amdgcn_sched_barrier(0);
     commit(0);
     issue(0, 1);
     for (int n = 0; n < myTiles; ++n) {
@@ -288,6 +312,7 @@ extern "C" __global__ DNX_LAUNCH_BOUNDS(NT) void KERNEL_NAME(
     store_part(myTiles - 1, 0, NVO);
   } else {
     // ---- computing waves -------------------------------------------------------------------------------------
+    stage_weights_and_bias();
     const int l32 = lane & 31;
     const int kq = (lane >> 5) * 8;
     const int rg = wv / KSP;           // row group: low-resolution rows rg * RPW .. of the tile
