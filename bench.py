@@ -281,7 +281,7 @@ def measure(args, workload: str, steps: int, warmup: int, brief: bool):
     # other.  A throughput figure for a stream of frames; a frame then takes about twice as long to come back, so it is
     # reported beside `value`, which stays one frame at a time.
     two_ms = None
-    if not brief:
+    if not brief and not args.no_two_frames:
         ctx2 = dx.Context(0)
         mod2 = dx.Module.load(blob, ctx2)
         inst2 = mod2.instance(H=H, W=W)
@@ -413,7 +413,8 @@ def measure(args, workload: str, steps: int, warmup: int, brief: bool):
         "config": {"workload": f"{description}; {mod.runtime_model.dispatch_count} dispatches in one hipGraph", "device_bytes": inst.device_bytes,
                    "schedule": "min-cost over measured dispatch latencies" if db is not None else "min-cost over roofline estimates",
                    "tuning_seconds": round(tune_s, 2), "host_pointer_path_ms_per_frame": round(host_ms, 3), "host_pointer_pipelined_ms_per_frame": round(pipelined_ms, 3),
-                   "two_frames_in_flight_ms_per_frame": round(two_ms, 4), "two_frames_in_flight_Mpix_s": round(H * W / (two_ms * 1e-3) * 1e-6, 1),
+                   "two_frames_in_flight_ms_per_frame": round(two_ms, 4) if two_ms else None,
+                   "two_frames_in_flight_Mpix_s": round(H * W / (two_ms * 1e-3) * 1e-6, 1) if two_ms else None,
                    "single_replay_ms_median": round(singles[len(singles) // 2], 4), "single_replay_ms_p95": round(singles[int(len(singles) * 0.95)], 4),
                    "settle_seconds": args.settle_seconds,
                    "layout_preference": args.layout_preference, "internal_tensors_in_chwc8": chwc8, "schedule_configs": chosen,
@@ -454,6 +455,8 @@ def main() -> int:
     ap.add_argument("--no-blocked-layout", action="store_true", help="internal tensors pixel-major (HWC) only: no CHWC8 candidates")
     ap.add_argument("--no-unfused-pass", action="store_true", help="skip the second, unfused schedule that times the stand-alone bandwidth kernels")
     ap.add_argument("--settle-seconds", type=float, default=0.3, help="untimed back-to-back frames before --warmup, until clocks have settled")
+    ap.add_argument("--no-two-frames", action="store_true",
+                    help="skip the two-frames-in-flight figure (under a profiler its overlapping kernels would blur the per-kernel durations)")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="only the selected workload; by default the headline run appends short runs of the other benchmark configurations")
     args = ap.parse_args()
